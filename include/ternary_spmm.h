@@ -1,0 +1,220 @@
+/*
+ * ternary_spmm.h -- C ABI of libternary_spmm.so: ternary (-1/0/+1) sparse GEMM for
+ * AMD MI355X (gfx950).
+ *
+ * The library replaces the four callables of the reference's pybind11 module
+ * `ter_spmm` (ternaryLLM_GPU/csrc/ter_spmm_wrapper.cu:350-355) and the two device
+ * kernels behind them (ternaryLLM_GPU/csrc/ter_spmm_kernel.cuh:24-78, :106-308).
+ *
+ * Conventions
+ *   - plain pointers and sizes only; no torch / ATen / pybind types.
+ *   - every function returns an int status: TL_OK (0) or a negative TL_ERR_* code;
+ *     tl_last_error() returns a thread-local message for the last failure.
+ *   - the library never allocates or frees device memory.  Device buffers
+ *     (inputs, outputs, workspace) are the caller's; sizes come from the *_size /
+ *     *_workspace calls.
+ *   - host packers write into caller-provided arrays after a sizing call.
+ *   - compute entry points enqueue on the hipStream_t passed as `void* stream`
+ *     (NULL = the default stream) and return without synchronising.
+ *   - all functions are re-entrant; there is no mutable global state besides the
+ *     thread-local error text.
+ */
+#ifndef TERNARY_SPMM_H
+#define TERNARY_SPMM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- status codes ------------------------------------------------------ */
+#define TL_OK 0
+#define TL_ERR_ARG (-1)         /* null pointer, negative size, bad flag          */
+#define TL_ERR_SHAPE (-2)       /* sizes inconsistent with each other             */
+#define TL_ERR_DTYPE (-3)       /* unknown dtype code                             */
+#define TL_ERR_ALIGN (-4)       /* pointer or leading dimension not aligned       */
+#define TL_ERR_UNSUPPORTED (-5) /* valid request this build cannot serve          */
+#define TL_ERR_LAUNCH (-6)      /* HIP reported an error at launch                */
+#define TL_ERR_VALUE (-7)       /* data error: non-ternary weight, count mismatch */
+#define TL_ERR_SIZE (-8)        /* caller buffer too small                        */
+#define TL_ERR_FORMAT (-9)      /* packed blob failed validation                  */
+
+/* ---- dtype / layout / flag codes --------------------------------------- */
+#define TL_F32 0
+#define TL_F16 1
+
+#define TL_X_ROW_MAJOR 0 /* X is [M][ldx], K contiguous (what the nn.Module callers pass)      */
+#define TL_X_K_MAJOR 1   /* X is [K][ldx], M contiguous (what the reference kernel itself reads, */
+                         /* ter_spmm_kernel.cuh:173)                                            */
+
+#define TL_ACT_NONE 0
+#define TL_ACT_SILU_GATE 1 /* out = silu(gate) * up, for tl_mlp_gate_up */
+
+const char* tl_last_error(void);
+int tl_version(void);
+
+/* ======================================================================== */
+/* Host packers: bit-exact replacements of the reference's converters.      */
+/* `w` is a host, row-major int32 [inners][columns] matrix with values in   */
+/* {-1, 0, +1}; argument order follows the reference (columns BEFORE        */
+/* inners, cnt_pos BEFORE cnt_neg, outputs negative stream first).          */
+/* ======================================================================== */
+
+/* Counts the +1 and -1 entries (the reference caller does this in Python,
+ * TernaryLinear.py:104-105).  Fails with TL_ERR_VALUE on any other value. */
+int tl_count_nnz(const int32_t* w, int columns, int inners, int64_t* cnt_pos, int64_t* cnt_neg);
+
+/* Replaces convert_to_ter_csc (ter_spmm_wrapper.cu:39-78).
+ * neg_row[cnt_neg], neg_off[columns+1], pos_row[cnt_pos], pos_off[columns+1]. */
+int tl_convert_to_ter_csc(const int32_t* w, int columns, int inners, int cnt_pos, int cnt_neg,
+                          int32_t* neg_row, int32_t* neg_off, int32_t* pos_row, int32_t* pos_off);
+
+/* Replaces convert_to_ter_tiled_csc (ter_spmm_wrapper.cu:92-152).
+ * Offsets hold columns * ceil(inners / tile_k) * 2 entries:
+ * off[(y*T + t)*2 + {0,1}] = [start, end) of tile t of column y; row indices are
+ * tile-local.  Rows past `inners` in a ragged last tile count as zero (the
+ * reference reads out of bounds there). */
+int tl_convert_to_ter_tiled_csc(const int32_t* w, int columns, int inners, int cnt_pos, int cnt_neg,
+                                int tile_k, int32_t* neg_row, int32_t* neg_off_tiled,
+                                int32_t* pos_row, int32_t* pos_off_tiled);
+
+/* Sizing call for tl_convert_to_ter_tiled_mcsc: number of entries of the merged
+ * index array (cnt_pos + cnt_neg, or the padded total, ter_spmm_wrapper.cu:198-230). */
+int tl_tiled_mcsc_size(const int32_t* w, int columns, int inners, int cnt_pos, int cnt_neg,
+                       int tile_k, int padding, int padding_size, int64_t* n_index);
+
+/* Replaces convert_to_ter_tiled_mcsc + inter_tile_swizzle
+ * (ter_spmm_wrapper.cu:156-315, :9-27), including the truncation of the pair and
+ * remainder counts to multiples of 4 (:277-291) and the overwrite order.
+ * merged_row[n_index], merged_off[columns*T*4], col_tile_idx[columns*T]. */
+int tl_convert_to_ter_tiled_mcsc(const int32_t* w, int columns, int inners, int cnt_pos, int cnt_neg,
+                                 int tile_k, int padding, int padding_size,
+                                 int32_t* merged_row, int64_t n_index,
+                                 int32_t* merged_off, int32_t* col_tile_idx);
+
+/* Decodes merged arrays back to the ternary matrix they encode, i.e. the matrix
+ * the reference kernels' loops (ter_spmm_kernel.cuh:197-300) would multiply by.
+ * index_width is 2 (int16, what TernaryLinear stores, TernaryLinear.py:110) or 4.
+ * w_out is int32 [inners][columns].  TL_ERR_VALUE when an entry of the decoded
+ * matrix falls outside {-1, 0, +1} (possible only with padded arrays). */
+int tl_tiled_mcsc_to_dense(const void* merged_row, int index_width, int64_t n_index,
+                           const int32_t* merged_off, int columns, int inners, int tile_k,
+                           int32_t* w_out);
+
+/* ======================================================================== */
+/* Device format ("wave-tiled CSC"): one relocatable blob, built on the     */
+/* host from tiled CSC, copied to the GPU by the caller.                    */
+/*   - K is cut into tiles of `tile_rows` <= 255 rows; indices are 8-bit    */
+/*     tile-local, value 255 is a padding sentinel that addresses a zero.   */
+/*   - +1 and -1 rows of one (column, tile) are two separate runs, each     */
+/*     padded to a multiple of 4 bytes (the -1 run follows the +1 run).     */
+/*   - the index stream is tile-major: all runs of tile 0 in column order,  */
+/*     then tile 1, ...; columns are grouped in blocks of 64 and            */
+/*     blockstart[tile][block] gives the dword where a block's runs begin.  */
+/*   - per (tile, column) one 32-bit descriptor: +1 count (bits 0-7), -1    */
+/*     count (bits 8-15), dword offset of the run inside its block (16-31). */
+/*     The descriptor table is padded to whole blocks with empty columns.   */
+/* The blob starts with a tl_layout_header (256 bytes).                     */
+/* ======================================================================== */
+
+#define TL_LAYOUT_MAGIC 0x32474C54u /* "TLG2" */
+#define TL_BLOCK_COLUMNS 64
+
+typedef struct tl_layout_header {
+    uint32_t magic;
+    uint32_t version;
+    uint32_t inners;      /* K */
+    uint32_t columns;     /* N */
+    uint32_t tile_rows;   /* rows per device tile, <= 255 */
+    uint32_t n_tiles;     /* T = ceil(K / tile_rows) */
+    uint32_t n_blocks;    /* NB = ceil(N / 64) */
+    uint32_t reserved0;
+    uint64_t nnz_pos;
+    uint64_t nnz_neg;
+    uint64_t off_blockstart; /* byte offset of uint32 blockstart[T*NB + 1] (dword units into idx) */
+    uint64_t off_desc;       /* byte offset of uint32 desc[T][NB*64]                               */
+    uint64_t off_idx;        /* byte offset of the index bytes                                     */
+    uint64_t idx_bytes;      /* padded index bytes (multiple of 4)                                 */
+    uint64_t total_bytes;    /* bytes of the blob that are in use, multiple of 256                 */
+    uint32_t max_run_dwords; /* largest (+1 run dwords + -1 run dwords) of any (column, tile)      */
+    uint32_t mean_run_dwords_x16; /* mean of the same, times 16, rounded up                        */
+    uint32_t reserved[40];
+} tl_layout_header;
+
+/* Bytes of the blob that tl_layout_build will write for these tiled-CSC arrays
+ * (as produced by tl_convert_to_ter_tiled_csc with tile height tile_k).
+ * tile_rows = 0 picks the default (the largest balanced height <= 255). */
+int tl_layout_size(const int32_t* neg_off_tiled, const int32_t* pos_off_tiled,
+                   int columns, int inners, int tile_k, int tile_rows, int64_t* blob_bytes);
+
+/* Builds the blob into host memory `blob` (blob_bytes as returned above). */
+int tl_layout_build(const int32_t* neg_row, const int32_t* neg_off_tiled,
+                    const int32_t* pos_row, const int32_t* pos_off_tiled,
+                    int columns, int inners, int tile_k, int tile_rows,
+                    void* blob, int64_t blob_bytes);
+
+/* Convenience: dense int32 [inners][columns] -> blob (runs the tiled-CSC packer
+ * internally).  Call with blob == NULL to get blob_bytes only. */
+int tl_layout_from_dense(const int32_t* w, int columns, int inners, int tile_rows,
+                         void* blob, int64_t* blob_bytes);
+
+/* Validates a host copy of a blob (header, bounds, monotone offsets, sentinel use). */
+int tl_layout_validate(const void* blob, int64_t blob_bytes);
+
+/* Decodes a host blob back to dense int32 [inners][columns] (round-trip check). */
+int tl_layout_to_dense(const void* blob, int64_t blob_bytes, int32_t* w_out);
+
+/* ======================================================================== */
+/* Compute.                                                                 */
+/* ======================================================================== */
+
+/* Workspace bytes tl_spmm needs for M rows of x_dtype in x_layout (0 when none).
+ * `header` is a host copy of the blob's first 256 bytes. */
+int tl_spmm_workspace(const tl_layout_header* header, int64_t M, int x_dtype, int x_layout,
+                      int64_t* workspace_bytes);
+
+/* Y[M][N] = (X[M][K] * W) * scale  -- replaces ter_spmm (ter_spmm_wrapper.cu:318-348)
+ * and both kernels behind it (ter_spmm_kernel.cuh:24-78 for M = 1, :106-308 for M > 1).
+ *   header      host copy of the blob header
+ *   blob_dev    device pointer to the whole blob (256-byte aligned)
+ *   X           device, x_dtype, layout x_layout, leading dimension ldx (elements)
+ *   Y           device, y_dtype, row-major [M][ldy]
+ *   scale       device per-output-column factor of scale_dtype, or NULL (the
+ *               reference has none; its result equals scale == NULL)
+ *   workspace   device scratch of at least tl_spmm_workspace() bytes (may be NULL when 0)
+ * Accumulation is always fp32. */
+int tl_spmm(const tl_layout_header* header, const void* blob_dev,
+            const void* X, int x_dtype, int x_layout, int64_t ldx, int64_t M,
+            void* Y, int y_dtype, int64_t ldy,
+            const void* scale, int scale_dtype,
+            void* workspace, int64_t workspace_bytes, void* stream);
+
+/* H[M][N] = act(X*Wg * sg, X*Wu * su): the gate and up projections of the
+ * reference's LlamaTernaryMLP (TernaryLLM/TernaryMLP.py:33-35) in one pass over X
+ * with the SiLU-gate product fused into the epilogue (the reference runs two
+ * ter_spmm calls and two elementwise kernels).  Both blobs must share K, N and
+ * tile_rows.  Arguments as for tl_spmm. */
+int tl_mlp_gate_up(const tl_layout_header* gate_header, const void* gate_blob_dev,
+                   const tl_layout_header* up_header, const void* up_blob_dev,
+                   const void* X, int x_dtype, int x_layout, int64_t ldx, int64_t M,
+                   void* H, int h_dtype, int64_t ldh,
+                   const void* gate_scale, const void* up_scale, int scale_dtype,
+                   int activation,
+                   void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Times `iters` back-to-back tl_spmm launches on `stream` with HIP events recorded
+ * on that same stream and returns the mean milliseconds per launch.  Used by the
+ * benchmark so that the figure covers exactly the kernels tl_spmm enqueues. */
+int tl_spmm_time(const tl_layout_header* header, const void* blob_dev,
+                 const void* X, int x_dtype, int x_layout, int64_t ldx, int64_t M,
+                 void* Y, int y_dtype, int64_t ldy,
+                 const void* scale, int scale_dtype,
+                 void* workspace, int64_t workspace_bytes, void* stream,
+                 int iters, float* mean_ms);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TERNARY_SPMM_H */

@@ -1,0 +1,668 @@
+// gfx950 kernels and launchers of libternary_spmm: Y = (X * W) * scale for a ternary W
+// held in the wave-tiled CSC blob (see tl_layout.cpp for the format).
+//
+// Two kernels replace the reference's pair
+// (ternaryLLM_GPU/csrc/ter_spmm_kernel.cuh:24-78 SpMV, :106-308 SpMM):
+//
+//   tl_spmm_small  M <= 48 (decode and small batches).  A group of LPC lanes owns
+//                  one output column and splits each (column, tile) run between its
+//                  lanes, one dword = four 8-bit row indices per lane; the
+//                  activation tiles sit in LDS as fp32 [slot][row]; every index is
+//                  one LDS gather and one fp32 add per activation row; the LPC
+//                  partial sums are folded with cross-lane shuffles.
+//   tl_spmm_rows   larger M (prefill).  Lanes own activation rows, a wave owns C
+//                  output columns, so an index is wave-uniform: it is read through
+//                  the scalar path once and serves 64*R rows; the activation tile
+//                  is staged in LDS as [slot][row] so the gather of a wave is one
+//                  contiguous, conflict-free LDS read.
+//
+// Only additions and subtractions touch the data; fp32 accumulation throughout.
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+
+#include <cstdlib>
+#include <cstring>
+
+#include "tl_common.h"
+
+using namespace tl;
+
+namespace {
+
+// Loads through this pointer type may use the scalar (constant) path when the address is wave-uniform.
+typedef const __attribute__((address_space(4))) uint32_t* const_u32_ptr;
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));  // one 16-byte chunk in registers
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Wold-style-cast"
+__device__ __forceinline__ const_u32_ptr as_const(const uint32_t* p) { return (const_u32_ptr)p; }
+#pragma clang diagnostic pop
+
+struct WeightPtrs {
+    const uint32_t* blockstart;  // [T * NB + 1]
+    const uint32_t* desc;        // [T][NB * 64]
+    const uint32_t* idx;         // dwords of four 8-bit rows
+    const void* scale;           // per-column factor or null
+};
+
+struct KernelArgs {
+    WeightPtrs w0;
+    WeightPtrs w1;  // second weight set of the fused gate/up kernel
+    const void* X;
+    void* Y;
+    long long ldx, ldy;
+    int M, N, K, T, tile_rows, NB;
+    int x_f16, x_kmajor, y_f16, scale_f16;
+    int tiles_per_stage;
+    float one;  // 1.0f, passed in so that the fp16 -> fp32 accumulate stays a single mixed-precision fma
+};
+
+__device__ __forceinline__ float load_scale(const void* scale, int is_f16, int n)
+{
+    if (!scale) return 1.0f;
+    return is_f16 ? __half2float(static_cast<const __half*>(scale)[n]) : static_cast<const float*>(scale)[n];
+}
+
+__device__ __forceinline__ void store_out(void* Y, int is_f16, long long off, float v)
+{
+    if (is_f16) static_cast<__half*>(Y)[off] = __float2half(v);
+    else static_cast<float*>(Y)[off] = v;
+}
+
+__device__ __forceinline__ float silu(float g) { return g / (1.0f + __expf(-g)); }
+
+__device__ __forceinline__ int run_pos_dwords(uint32_t d) { return (int)(((d & 0xffu) + 3u) >> 2); }
+__device__ __forceinline__ int run_neg_dwords(uint32_t d) { return (int)((((d >> 8) & 0xffu) + 3u) >> 2); }
+
+// ---------------------------------------------------------------------------
+// Small-M kernel.
+// ---------------------------------------------------------------------------
+template <int MT>
+__device__ __forceinline__ void gather_add(float (&acc)[MT], const float* __restrict__ xt, uint32_t word, float sign)
+{
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+        const uint32_t r = (word >> (8 * b)) & 0xffu;
+        const float* row = xt + r * MT;
+        if constexpr (MT % 4 == 0) {
+#pragma unroll
+            for (int m = 0; m < MT; m += 4) {
+                const float4 v = *reinterpret_cast<const float4*>(row + m);
+                acc[m + 0] = fmaf(v.x, sign, acc[m + 0]);
+                acc[m + 1] = fmaf(v.y, sign, acc[m + 1]);
+                acc[m + 2] = fmaf(v.z, sign, acc[m + 2]);
+                acc[m + 3] = fmaf(v.w, sign, acc[m + 3]);
+            }
+        } else if constexpr (MT == 2) {
+            const float2 v = *reinterpret_cast<const float2*>(row);
+            acc[0] = fmaf(v.x, sign, acc[0]);
+            acc[1] = fmaf(v.y, sign, acc[1]);
+        } else {
+            acc[0] = fmaf(row[0], sign, acc[0]);
+        }
+    }
+}
+
+template <int MT, int LPC>
+__global__ __launch_bounds__(256) void tl_spmm_small(KernelArgs a)
+{
+    // LDS: activation tiles as fp32 [tiles_per_stage * 256 slots][MT], then the
+    // descriptors of this workgroup's columns for every tile, then the block starts.
+    extern __shared__ __align__(16) float xs[];
+    constexpr int CPB = 256 / LPC;  // columns per workgroup; divides 64, so they share one column block
+    constexpr int TB = 16;          // tiles whose index loads are in flight together
+    uint32_t* dsc = reinterpret_cast<uint32_t*>(xs + (size_t)a.tiles_per_stage * kTileSlots * MT);
+    uint32_t* bst = dsc + (size_t)a.T * CPB;
+
+    const int tid = threadIdx.x;
+    const int lig = tid % LPC, col = tid / LPC;
+    const int n_first = blockIdx.x * CPB;
+    const int n = n_first + col;
+    const int m0 = blockIdx.y * MT;
+    const int NP = a.NB * TL_BLOCK_COLUMNS;
+    const uint32_t* __restrict__ idx = a.w0.idx;
+
+    for (int e = tid; e < a.T * CPB; e += 256) dsc[e] = a.w0.desc[(size_t)(e / CPB) * NP + n_first + e % CPB];
+    for (int e = tid; e < a.T; e += 256) bst[e] = a.w0.blockstart[(size_t)e * a.NB + n_first / TL_BLOCK_COLUMNS];
+    __syncthreads();
+
+    float acc[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) acc[m] = 0.f;
+
+    // One dword (four rows) per lane and tile; lanes past the run's end take an
+    // all-sentinel word, i.e. four gathers of the zero slot, so nothing branches.
+    auto fetch = [&](int tb, uint32_t(&w)[TB]) {
+#pragma unroll
+        for (int u = 0; u < TB; ++u) {
+            const int t = tb + u;
+            uint32_t word = 0xffffffffu;
+            if (t < a.T) {
+                const uint32_t d = dsc[t * CPB + col];
+                if (lig < run_pos_dwords(d) + run_neg_dwords(d)) word = idx[bst[t] + (d >> 16) + lig];
+            }
+            w[u] = word;
+        }
+    };
+
+    uint32_t wn[TB];
+    fetch(0, wn);
+    for (int tb = 0; tb < a.T; tb += TB) {
+        uint32_t wc[TB];
+#pragma unroll
+        for (int u = 0; u < TB; ++u) wc[u] = wn[u];
+        if (tb + TB < a.T) fetch(tb + TB, wn);
+#pragma unroll
+        for (int u = 0; u < TB; ++u) {
+            const int t = tb + u;
+            if (t >= a.T) break;
+            if (t % a.tiles_per_stage == 0) {  // uniform: stage the next group of activation tiles
+                const int slots = min(a.tiles_per_stage, a.T - t) * kTileSlots;
+                __syncthreads();
+                for (int e = tid; e < slots * MT; e += 256) {
+                    const int slot = e % slots, m = e / slots;
+                    const int r = slot & (kTileSlots - 1);
+                    const long long k = (long long)(t + (slot >> 8)) * a.tile_rows + r;
+                    float v = 0.f;
+                    if (r < a.tile_rows && k < a.K && m0 + m < a.M) {
+                        const long long off = a.x_kmajor ? k * a.ldx + (m0 + m) : (long long)(m0 + m) * a.ldx + k;
+                        v = a.x_f16 ? __half2float(static_cast<const __half*>(a.X)[off]) : static_cast<const float*>(a.X)[off];
+                    }
+                    xs[slot * MT + m] = v;
+                }
+                __syncthreads();
+            }
+            const uint32_t d = dsc[t * CPB + col];
+            const int pd = run_pos_dwords(d), tot = pd + run_neg_dwords(d);
+            const float* xt = xs + (size_t)(t % a.tiles_per_stage) * kTileSlots * MT;
+            gather_add<MT>(acc, xt, wc[u], lig < pd ? 1.0f : -1.0f);
+            for (int i = lig + LPC; i < tot; i += LPC)  // runs longer than the lane group: rare
+                gather_add<MT>(acc, xt, idx[bst[t] + (d >> 16) + i], i < pd ? 1.0f : -1.0f);
+        }
+    }
+
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+#pragma unroll
+        for (int off = LPC / 2; off > 0; off >>= 1) acc[m] += __shfl_xor(acc[m], off, 64);
+    }
+    if (n < a.N && lig == 0) {
+        const float s = load_scale(a.w0.scale, a.scale_f16, n);
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+            if (m0 + m < a.M) store_out(a.Y, a.y_f16, (long long)(m0 + m) * a.ldy + n, acc[m] * s);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Activation re-layout for the row-parallel kernel: XT[k][m] (m contiguous, padded
+// with zeros to ldm columns) from row-major X[m][k] or K-major X[k][m].
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void tl_relayout_x(const T* __restrict__ X, long long ldx, int kmajor, T* __restrict__ XT,
+                                                     long long ldm, int M, int K)
+{
+    __shared__ T tile[64][65];
+    const int k0 = blockIdx.x * 64, m0 = blockIdx.y * 64;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;  // 64 x 4
+    if (kmajor) {
+        for (int j = ty; j < 64; j += 4) {
+            const int k = k0 + j, m = m0 + tx;
+            if (k < K) XT[(long long)k * ldm + m] = (m < M) ? X[(long long)k * ldx + m] : T(0.0f);
+        }
+        return;
+    }
+    for (int j = ty; j < 64; j += 4) {
+        const int m = m0 + j, k = k0 + tx;
+        tile[j][tx] = (m < M && k < K) ? X[(long long)m * ldx + k] : T(0.0f);
+    }
+    __syncthreads();
+    for (int j = ty; j < 64; j += 4) {
+        const int k = k0 + j, m = m0 + tx;
+        if (k < K) XT[(long long)k * ldm + m] = tile[tx][j];
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Row-parallel kernel.
+// ---------------------------------------------------------------------------
+template <typename XT, int R>
+struct RowVec;
+template <>
+struct RowVec<__half, 4> {
+    using type = uint2;
+    static __device__ __forceinline__ void add(float (&acc)[4], uint2 v, float sgn_one)
+    {
+        const __half2 lo = *reinterpret_cast<const __half2*>(&v.x), hi = *reinterpret_cast<const __half2*>(&v.y);
+        acc[0] = fmaf(__low2float(lo), sgn_one, acc[0]);
+        acc[1] = fmaf(__high2float(lo), sgn_one, acc[1]);
+        acc[2] = fmaf(__low2float(hi), sgn_one, acc[2]);
+        acc[3] = fmaf(__high2float(hi), sgn_one, acc[3]);
+    }
+};
+template <>
+struct RowVec<float, 2> {
+    using type = float2;
+    static __device__ __forceinline__ void add(float (&acc)[2], float2 v, float sgn_one)
+    {
+        acc[0] = fmaf(v.x, sgn_one, acc[0]);
+        acc[1] = fmaf(v.y, sgn_one, acc[1]);
+    }
+};
+
+// The runs of one wave (C neighbouring columns) for one tile: descriptors, the
+// dword where the wave's piece of the stream starts, and its first NPRE * 64 dwords
+// (one per lane and chunk), fetched one tile ahead of their use.
+constexpr int NPRE = 3;
+template <int C>
+struct WaveRuns {
+    uint32_t d[C];
+    uint32_t base;
+    uint32_t pre[NPRE];
+};
+
+template <int C>
+__device__ __forceinline__ void fetch_runs(WaveRuns<C>& r, const WeightPtrs& w, int t, int NP, int NB, int n0, int lane)
+{
+    const_u32_ptr dp = as_const(w.desc) + (size_t)t * NP + n0;
+#pragma unroll
+    for (int c = 0; c < C; ++c) r.d[c] = dp[c];
+    r.base = as_const(w.blockstart)[(size_t)t * NB + n0 / TL_BLOCK_COLUMNS] + (r.d[0] >> 16);
+    // Reads past the wave's piece stay inside the blob (it ends with spare bytes) and are never used.
+#pragma unroll
+    for (int ch = 0; ch < NPRE; ++ch) r.pre[ch] = w.idx[r.base + ch * 64 + lane];
+}
+
+template <typename XT, int R>
+__device__ __forceinline__ void rows_add4(float (&acc)[R], const XT* __restrict__ tile_lane, uint32_t word, float sgn_one)
+{
+    using V = typename RowVec<XT, R>::type;
+    constexpr int MTILE = 64 * R;
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+        const uint32_t r = (word >> (8 * b)) & 0xffu;
+        RowVec<XT, R>::add(acc, *reinterpret_cast<const V*>(tile_lane + r * MTILE), sgn_one);
+    }
+}
+
+// One 64-dword chunk of the wave's piece: dword i of the piece sits in lane i - cb of `v`
+// and is broadcast from there, so its four row indices are wave-uniform.
+template <typename XT, int R, int C>
+__device__ __forceinline__ void rows_chunk(float (&acc)[C][R], const int (&pb)[C], const int (&pe)[C], const int (&ne)[C],
+                                           uint32_t v, int cb, const XT* __restrict__ tile_lane, float one)
+{
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+        for (int i = max(pb[c], cb); i < min(pe[c], cb + 64); ++i)
+            rows_add4<XT, R>(acc[c], tile_lane, (uint32_t)__builtin_amdgcn_readlane((int)v, i - cb), one);
+        for (int i = max(pe[c], cb); i < min(ne[c], cb + 64); ++i)
+            rows_add4<XT, R>(acc[c], tile_lane, (uint32_t)__builtin_amdgcn_readlane((int)v, i - cb), -one);
+    }
+}
+
+template <typename XT, int R, int C>
+__device__ __forceinline__ void rows_consume(float (&acc)[C][R], const WaveRuns<C>& r, const uint32_t* __restrict__ idx,
+                                             const XT* __restrict__ tile_lane, int lane, float one)
+{
+    int pb[C], pe[C], ne[C];
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+        pb[c] = (int)((r.d[c] >> 16) - (r.d[0] >> 16));
+        pe[c] = pb[c] + run_pos_dwords(r.d[c]);
+        ne[c] = pe[c] + run_neg_dwords(r.d[c]);
+    }
+    const int total = ne[C - 1];
+#pragma unroll
+    for (int ch = 0; ch < NPRE; ++ch)
+        if (ch * 64 < total) rows_chunk<XT, R, C>(acc, pb, pe, ne, r.pre[ch], ch * 64, tile_lane, one);
+    for (int cb = NPRE * 64; cb < total; cb += 64)  // pieces longer than the prefetch window: fetched on demand
+        rows_chunk<XT, R, C>(acc, pb, pe, ne, idx[r.base + cb + lane], cb, tile_lane, one);
+}
+
+// Staging of one activation tile in two halves: global -> registers (issued a tile
+// ahead), registers -> LDS.  A thread owns the same 16-byte chunks in both halves.
+template <typename XT, int CHUNKS, int NT, int PER>
+__device__ __forceinline__ void tile_to_regs(u32x4 (&pf)[PER], const unsigned char* __restrict__ XTr, const KernelArgs& a, int t, int m0)
+{
+    const int n_chunks = min(a.tile_rows, a.K - t * a.tile_rows) * CHUNKS;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        // Chunks past the tile's end re-read its last chunk (never stored): the load stays unconditional.
+        const int e = min((int)threadIdx.x + i * NT, n_chunks - 1);
+        const int r = e / CHUNKS, ch = e % CHUNKS;
+        pf[i] = *reinterpret_cast<const u32x4*>(XTr + ((size_t)(t * a.tile_rows + r) * a.ldx + m0) * sizeof(XT) + ch * 16);
+    }
+}
+
+template <int CHUNKS, int NT, int PER>
+__device__ __forceinline__ void regs_to_lds(const u32x4 (&pf)[PER], unsigned char* smem, const KernelArgs& a, int t)
+{
+    const int n_chunks = min(a.tile_rows, a.K - t * a.tile_rows) * CHUNKS;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const int e = (int)threadIdx.x + i * NT;
+        if (e < n_chunks) *reinterpret_cast<u32x4*>(smem + (size_t)e * 16) = pf[i];
+    }
+}
+
+template <typename XT, int R, int C, int WAVES, bool GATED>
+__global__ __launch_bounds__(WAVES * 64) void tl_spmm_rows(KernelArgs a)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    constexpr int MTILE = 64 * R;
+    constexpr int NT = WAVES * 64;
+    constexpr int CHUNKS = MTILE * (int)sizeof(XT) / 16;                 // 16-byte chunks per staged row
+    constexpr int PER = (kMaxTileRows * CHUNKS + NT - 1) / NT;           // chunks one thread stages per tile
+    static_assert(TL_BLOCK_COLUMNS % C == 0, "a wave's columns must not straddle column blocks");
+    XT* tile = reinterpret_cast<XT*>(smem);                              // [256 slots][MTILE]
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int m0 = blockIdx.y * MTILE;
+    const int n0 = blockIdx.x * (WAVES * C) + wave * C;
+    const int NP = a.NB * TL_BLOCK_COLUMNS;
+    const bool wave_live = n0 < a.N;                                       // uniform; n0 < NP whenever true
+    const unsigned char* __restrict__ XTr = static_cast<const unsigned char*>(a.X);  // [K][ldx] of XT, m contiguous
+
+    float acc[C][R];
+    float acc2[GATED ? C : 1][R];
+#pragma unroll
+    for (int c = 0; c < C; ++c)
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+            acc[c][j] = 0.f;
+            if (GATED) acc2[GATED ? c : 0][j] = 0.f;
+        }
+
+    // Slot 255 is what padding bytes address: zero it once, staging never writes it.
+    for (int e = threadIdx.x; e < MTILE; e += NT) tile[kSentinel * MTILE + e] = XT(0.0f);
+
+    // The next activation tile travels global -> registers while the current one is consumed.
+    u32x4 pf[PER];
+    WaveRuns<C> cur, nxt, cur2, nxt2;
+    if (wave_live) {
+        fetch_runs<C>(nxt, a.w0, 0, NP, a.NB, n0, lane);
+        if constexpr (GATED) fetch_runs<C>(nxt2, a.w1, 0, NP, a.NB, n0, lane);
+    }
+    tile_to_regs<XT, CHUNKS, NT, PER>(pf, XTr, a, 0, m0);
+    const XT* tile_lane = tile + lane * R;
+    for (int t = 0; t < a.T; ++t) {
+        __syncthreads();  // every wave is done with the previous tile
+        regs_to_lds<CHUNKS, NT, PER>(pf, smem, a, t);
+        __syncthreads();
+        if (t + 1 < a.T) tile_to_regs<XT, CHUNKS, NT, PER>(pf, XTr, a, t + 1, m0);
+        if (wave_live) {
+            cur = nxt;
+            if constexpr (GATED) cur2 = nxt2;
+            if (t + 1 < a.T) {
+                fetch_runs<C>(nxt, a.w0, t + 1, NP, a.NB, n0, lane);
+                if constexpr (GATED) fetch_runs<C>(nxt2, a.w1, t + 1, NP, a.NB, n0, lane);
+            }
+            rows_consume<XT, R, C>(acc, cur, a.w0.idx, tile_lane, lane, a.one);
+            if constexpr (GATED) rows_consume<XT, R, C>(acc2, cur2, a.w1.idx, tile_lane, lane, a.one);
+        }
+    }
+
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+        const int n = n0 + c;
+        if (n >= a.N) continue;
+        const float s = load_scale(a.w0.scale, a.scale_f16, n);
+        const float s2 = GATED ? load_scale(a.w1.scale, a.scale_f16, n) : 1.0f;
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+            const int m = m0 + lane * R + j;
+            if (m >= a.M) continue;
+            float v = acc[c][j] * s;
+            if constexpr (GATED) v = silu(v) * (acc2[GATED ? c : 0][j] * s2);
+            store_out(a.Y, a.y_f16, (long long)m * a.ldy + n, v);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Host side.
+// ---------------------------------------------------------------------------
+int check_header(const tl_layout_header* h)
+{
+    if (!h) return fail(TL_ERR_ARG, "layout header is null");
+    if (h->magic != TL_LAYOUT_MAGIC || h->version != 2) return fail(TL_ERR_FORMAT, "bad layout magic/version");
+    if (h->tile_rows == 0 || h->tile_rows > (uint32_t)kMaxTileRows || h->n_tiles != (uint32_t)ceil_div(h->inners, h->tile_rows) ||
+        h->n_blocks != (uint32_t)ceil_div(h->columns, TL_BLOCK_COLUMNS))
+        return fail(TL_ERR_FORMAT, "layout header geometry is inconsistent");
+    return TL_OK;
+}
+
+int check_dtype(int d, const char* what)
+{
+    if (d != TL_F32 && d != TL_F16) return fail(TL_ERR_DTYPE, "%s dtype code %d unknown", what, d);
+    return TL_OK;
+}
+
+constexpr int kSmallMaxM = 48;       // above this the row-parallel kernel takes over
+constexpr int kRowsWaves = 8;
+constexpr int kRowsCols = 8;
+
+inline int rows_mtile(int x_dtype) { return x_dtype == TL_F16 ? 256 : 128; }
+
+int env_int(const char* name, int fallback)
+{
+    const char* v = std::getenv(name);
+    return v && *v ? std::atoi(v) : fallback;
+}
+
+WeightPtrs weight_ptrs(const tl_layout_header* h, const void* blob_dev, const void* scale)
+{
+    const unsigned char* b = static_cast<const unsigned char*>(blob_dev);
+    WeightPtrs w;
+    w.blockstart = reinterpret_cast<const uint32_t*>(b + h->off_blockstart);
+    w.desc = reinterpret_cast<const uint32_t*>(b + h->off_desc);
+    w.idx = reinterpret_cast<const uint32_t*>(b + h->off_idx);
+    w.scale = scale;
+    return w;
+}
+
+template <int MT>
+int launch_small_lpc(const KernelArgs& a, int lpc, hipStream_t st)
+{
+    const size_t lds = (size_t)a.tiles_per_stage * kTileSlots * MT * sizeof(float) + ((size_t)a.T * (256 / lpc) + a.T) * sizeof(uint32_t);
+    dim3 grid((unsigned)ceil_div(a.N, 256 / lpc), (unsigned)ceil_div(a.M, MT));
+    switch (lpc) {
+        case 8: hipLaunchKernelGGL((tl_spmm_small<MT, 8>), grid, dim3(256), lds, st, a); break;
+        case 16: hipLaunchKernelGGL((tl_spmm_small<MT, 16>), grid, dim3(256), lds, st, a); break;
+        case 32: hipLaunchKernelGGL((tl_spmm_small<MT, 32>), grid, dim3(256), lds, st, a); break;
+        default: hipLaunchKernelGGL((tl_spmm_small<MT, 64>), grid, dim3(256), lds, st, a); break;
+    }
+    return TL_OK;
+}
+
+int launch_small(KernelArgs a, const tl_layout_header* h, hipStream_t st)
+{
+    int mt = 1;
+    while (mt < a.M && mt < 32) mt *= 2;
+    const double mean_run = h->mean_run_dwords_x16 / 16.0;
+    int lpc = 8;
+    while (lpc < 64 && lpc < mean_run * 1.1) lpc *= 2;
+    lpc = env_int("TL_LPC", lpc);
+    if (lpc != 8 && lpc != 16 && lpc != 32 && lpc != 64) return fail(TL_ERR_ARG, "TL_LPC=%d (8, 16, 32 or 64 expected)", lpc);
+    const int budget_slots = (48 * 1024) / (int)(mt * sizeof(float));
+    a.tiles_per_stage = (int)std::min<int64_t>(a.T, std::max(1, budget_slots / kTileSlots));
+    switch (mt) {
+        case 1: return launch_small_lpc<1>(a, lpc, st);
+        case 2: return launch_small_lpc<2>(a, lpc, st);
+        case 4: return launch_small_lpc<4>(a, lpc, st);
+        case 8: return launch_small_lpc<8>(a, lpc, st);
+        case 16: return launch_small_lpc<16>(a, lpc, st);
+        default: return launch_small_lpc<32>(a, lpc, st);
+    }
+}
+
+template <typename KernelT>
+int raise_lds_limit(KernelT kernel, size_t bytes)
+{
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) return fail(TL_ERR_LAUNCH, "hipFuncSetAttribute(%zu bytes of LDS): %s", bytes, hipGetErrorString(e));
+    return TL_OK;
+}
+
+template <typename XT, int R, bool GATED>
+int launch_rows_t(const KernelArgs& a, hipStream_t st)
+{
+    constexpr int MTILE = 64 * R;
+    const size_t lds = (size_t)kTileSlots * MTILE * sizeof(XT);
+    auto kernel = tl_spmm_rows<XT, R, kRowsCols, kRowsWaves, GATED>;
+    static bool raised = false;  // per instantiation; a repeated call is harmless
+    if (!raised) {
+        if (int rc = raise_lds_limit(kernel, lds)) return rc;
+        raised = true;
+    }
+    dim3 grid((unsigned)ceil_div(a.N, kRowsWaves * kRowsCols), (unsigned)ceil_div(a.M, MTILE));
+    hipLaunchKernelGGL(kernel, grid, dim3(kRowsWaves * 64), lds, st, a);
+    return TL_OK;
+}
+
+// Runs the re-layout pre-pass into `workspace`, then the row-parallel kernel.
+int launch_rows(KernelArgs a, int x_dtype, void* workspace, int64_t workspace_bytes, bool gated, hipStream_t st)
+{
+    const int mtile = rows_mtile(x_dtype);
+    const int64_t ldm = round_up(a.M, mtile);
+    const int64_t need = (int64_t)a.K * ldm * (x_dtype == TL_F16 ? 2 : 4);
+    if (!workspace || workspace_bytes < need)
+        return fail(TL_ERR_SIZE, "workspace has %lld bytes, %lld needed", (long long)workspace_bytes, (long long)need);
+    if (reinterpret_cast<uintptr_t>(workspace) % 16) return fail(TL_ERR_ALIGN, "workspace must be 16-byte aligned");
+    dim3 tgrid((unsigned)ceil_div(a.K, 64), (unsigned)(ldm / 64));
+    if (x_dtype == TL_F16)
+        hipLaunchKernelGGL(tl_relayout_x<__half>, tgrid, dim3(256), 0, st, static_cast<const __half*>(a.X), a.ldx, a.x_kmajor,
+                           static_cast<__half*>(workspace), ldm, a.M, a.K);
+    else
+        hipLaunchKernelGGL(tl_relayout_x<float>, tgrid, dim3(256), 0, st, static_cast<const float*>(a.X), a.ldx, a.x_kmajor,
+                           static_cast<float*>(workspace), ldm, a.M, a.K);
+    a.X = workspace;
+    a.ldx = ldm;
+    a.x_kmajor = 1;
+    if (x_dtype == TL_F16) return gated ? launch_rows_t<__half, 4, true>(a, st) : launch_rows_t<__half, 4, false>(a, st);
+    return gated ? launch_rows_t<float, 2, true>(a, st) : launch_rows_t<float, 2, false>(a, st);
+}
+
+int finish_launch()
+{
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(TL_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString(e));
+    return TL_OK;
+}
+
+int check_io(const void* blob_dev, const void* X, void* Y, int x_dtype, int x_layout, int64_t ldx, int64_t M, int y_dtype,
+             int64_t ldy, const void* scale, int scale_dtype, const tl_layout_header* h)
+{
+    if (!blob_dev || !X || !Y) return fail(TL_ERR_ARG, "device pointer is null");
+    if (reinterpret_cast<uintptr_t>(blob_dev) % 256) return fail(TL_ERR_ALIGN, "weight blob must be 256-byte aligned");
+    if (int rc = check_dtype(x_dtype, "x")) return rc;
+    if (int rc = check_dtype(y_dtype, "y")) return rc;
+    if (scale)
+        if (int rc = check_dtype(scale_dtype, "scale")) return rc;
+    if (x_layout != TL_X_ROW_MAJOR && x_layout != TL_X_K_MAJOR) return fail(TL_ERR_ARG, "x_layout=%d unknown", x_layout);
+    if (M <= 0 || M > (1 << 30)) return fail(TL_ERR_SHAPE, "M=%lld out of range", (long long)M);
+    const int64_t min_ldx = x_layout == TL_X_ROW_MAJOR ? h->inners : M;
+    if (ldx < min_ldx) return fail(TL_ERR_SHAPE, "ldx=%lld smaller than the %lld elements of a row", (long long)ldx, (long long)min_ldx);
+    if (ldy < (int64_t)h->columns) return fail(TL_ERR_SHAPE, "ldy=%lld smaller than N=%u", (long long)ldy, h->columns);
+    return TL_OK;
+}
+
+}  // namespace
+
+extern "C" int tl_spmm_workspace(const tl_layout_header* header, int64_t M, int x_dtype, int x_layout, int64_t* workspace_bytes)
+{
+    (void)x_layout;
+    if (int rc = check_header(header)) return rc;
+    if (int rc = check_dtype(x_dtype, "x")) return rc;
+    if (!workspace_bytes) return fail(TL_ERR_ARG, "workspace_bytes is null");
+    if (M <= 0) return fail(TL_ERR_SHAPE, "M=%lld must be positive", (long long)M);
+    if (M <= kSmallMaxM) {
+        *workspace_bytes = 0;
+        return TL_OK;
+    }
+    *workspace_bytes = (int64_t)header->inners * round_up(M, rows_mtile(x_dtype)) * (x_dtype == TL_F16 ? 2 : 4);
+    return TL_OK;
+}
+
+extern "C" int tl_spmm(const tl_layout_header* header, const void* blob_dev,
+                       const void* X, int x_dtype, int x_layout, int64_t ldx, int64_t M,
+                       void* Y, int y_dtype, int64_t ldy,
+                       const void* scale, int scale_dtype,
+                       void* workspace, int64_t workspace_bytes, void* stream)
+{
+    if (int rc = check_header(header)) return rc;
+    if (int rc = check_io(blob_dev, X, Y, x_dtype, x_layout, ldx, M, y_dtype, ldy, scale, scale_dtype, header)) return rc;
+    KernelArgs a;
+    std::memset(&a, 0, sizeof(a));
+    a.w0 = weight_ptrs(header, blob_dev, scale);
+    a.X = X; a.Y = Y;
+    a.ldx = ldx; a.ldy = ldy;
+    a.M = (int)M; a.N = (int)header->columns; a.K = (int)header->inners; a.T = (int)header->n_tiles; a.tile_rows = (int)header->tile_rows;
+    a.NB = (int)header->n_blocks;
+    a.x_f16 = x_dtype == TL_F16; a.x_kmajor = x_layout == TL_X_K_MAJOR; a.y_f16 = y_dtype == TL_F16; a.scale_f16 = scale_dtype == TL_F16;
+    a.one = 1.0f;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    int rc = (M <= kSmallMaxM) ? launch_small(a, header, st) : launch_rows(a, x_dtype, workspace, workspace_bytes, false, st);
+    if (rc) return rc;
+    return finish_launch();
+}
+
+extern "C" int tl_mlp_gate_up(const tl_layout_header* gate_header, const void* gate_blob_dev,
+                              const tl_layout_header* up_header, const void* up_blob_dev,
+                              const void* X, int x_dtype, int x_layout, int64_t ldx, int64_t M,
+                              void* H, int h_dtype, int64_t ldh,
+                              const void* gate_scale, const void* up_scale, int scale_dtype,
+                              int activation,
+                              void* workspace, int64_t workspace_bytes, void* stream)
+{
+    if (int rc = check_header(gate_header)) return rc;
+    if (int rc = check_header(up_header)) return rc;
+    if (gate_header->inners != up_header->inners || gate_header->columns != up_header->columns ||
+        gate_header->tile_rows != up_header->tile_rows)
+        return fail(TL_ERR_SHAPE, "gate and up weights must share K, N and tile height");
+    if (activation != TL_ACT_SILU_GATE) return fail(TL_ERR_UNSUPPORTED, "activation code %d (only TL_ACT_SILU_GATE)", activation);
+    if (!up_blob_dev || reinterpret_cast<uintptr_t>(up_blob_dev) % 256) return fail(TL_ERR_ALIGN, "up blob null or not 256-byte aligned");
+    if (int rc = check_io(gate_blob_dev, X, H, x_dtype, x_layout, ldx, M, h_dtype, ldh, gate_scale, scale_dtype, gate_header)) return rc;
+    if ((gate_scale == nullptr) != (up_scale == nullptr)) return fail(TL_ERR_ARG, "pass both scales or neither");
+    if (M <= kSmallMaxM) return fail(TL_ERR_UNSUPPORTED, "fused gate/up needs M > %d; use two tl_spmm calls below that", kSmallMaxM);
+    KernelArgs a;
+    std::memset(&a, 0, sizeof(a));
+    a.w0 = weight_ptrs(gate_header, gate_blob_dev, gate_scale);
+    a.w1 = weight_ptrs(up_header, up_blob_dev, up_scale);
+    a.X = X; a.Y = H;
+    a.ldx = ldx; a.ldy = ldh;
+    a.NB = (int)gate_header->n_blocks;
+    a.M = (int)M; a.N = (int)gate_header->columns; a.K = (int)gate_header->inners; a.T = (int)gate_header->n_tiles;
+    a.tile_rows = (int)gate_header->tile_rows;
+    a.x_f16 = x_dtype == TL_F16; a.x_kmajor = x_layout == TL_X_K_MAJOR; a.y_f16 = h_dtype == TL_F16; a.scale_f16 = scale_dtype == TL_F16;
+    a.one = 1.0f;
+    if (int rc = launch_rows(a, x_dtype, workspace, workspace_bytes, true, static_cast<hipStream_t>(stream))) return rc;
+    return finish_launch();
+}
+
+extern "C" int tl_spmm_time(const tl_layout_header* header, const void* blob_dev,
+                            const void* X, int x_dtype, int x_layout, int64_t ldx, int64_t M,
+                            void* Y, int y_dtype, int64_t ldy,
+                            const void* scale, int scale_dtype,
+                            void* workspace, int64_t workspace_bytes, void* stream,
+                            int iters, float* mean_ms)
+{
+    if (iters <= 0 || !mean_ms) return fail(TL_ERR_ARG, "iters must be positive and mean_ms non-null");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipEvent_t e0, e1;
+    if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) return fail(TL_ERR_LAUNCH, "hipEventCreate failed");
+    int rc = TL_OK;
+    (void)hipEventRecord(e0, st);
+    for (int i = 0; i < iters && rc == TL_OK; ++i)
+        rc = tl_spmm(header, blob_dev, X, x_dtype, x_layout, ldx, M, Y, y_dtype, ldy, scale, scale_dtype, workspace, workspace_bytes, stream);
+    (void)hipEventRecord(e1, st);
+    if (rc == TL_OK) {
+        hipError_t e = hipEventSynchronize(e1);
+        float ms = 0.f;
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+        if (e != hipSuccess) rc = fail(TL_ERR_LAUNCH, "event timing failed: %s", hipGetErrorString(e));
+        *mean_ms = ms / iters;
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    return rc;
+}

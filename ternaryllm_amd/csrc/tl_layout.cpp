@@ -1,0 +1,323 @@
+// Builder / validator / decoder of the device weight format ("wave-tiled CSC").
+//
+// Input is the lossless tiled CSC of the reference API
+// (ternaryLLM_GPU/csrc/ter_spmm_wrapper.cu:92-152: separate +1 / -1 row lists with
+// tile-local indices and [start, end) offsets per (column, tile)).  The device
+// format keeps the two separate streams but
+//   - re-tiles K into tiles of at most 255 rows so that an index is one byte and
+//     byte value 255 can act as a padding sentinel;
+//   - pads every run to whole dwords so that a lane (or a broadcast word) always
+//     carries four indices;
+//   - orders the stream tile-major, so that the runs a wave needs for one tile --
+//     those of a few neighbouring columns -- are one contiguous piece of memory.
+#include <cstring>
+#include <vector>
+
+#include "tl_common.h"
+
+using namespace tl;
+
+namespace {
+
+constexpr int kBlock = TL_BLOCK_COLUMNS;
+
+struct Geometry {
+    int tile_rows, n_tiles, n_blocks;
+};
+
+int pick_geometry(int columns, int inners, int tile_rows, Geometry* g)
+{
+    if (tile_rows < 0 || tile_rows > kMaxTileRows)
+        return fail(TL_ERR_ARG, "tile_rows=%d must be in [1, %d] (0 = default)", tile_rows, kMaxTileRows);
+    if (tile_rows == 0) {
+        const int t = (int)ceil_div(inners, kMaxTileRows);
+        tile_rows = (int)ceil_div(inners, t);
+    }
+    g->tile_rows = tile_rows;
+    g->n_tiles = (int)ceil_div(inners, tile_rows);
+    g->n_blocks = (int)ceil_div(columns, kBlock);
+    return TL_OK;
+}
+
+struct Sections {
+    int64_t off_blockstart, off_desc, off_idx, total;
+};
+
+Sections place_sections(const Geometry& g, int64_t idx_bytes)
+{
+    Sections s;
+    s.off_blockstart = 256;
+    s.off_desc = s.off_blockstart + round_up(((int64_t)g.n_tiles * g.n_blocks + 1) * 4, 256);
+    s.off_idx = s.off_desc + round_up((int64_t)g.n_tiles * g.n_blocks * kBlock * 4, 256);
+    // 512 spare bytes behind the indices: kernels fetch whole 64-dword vectors past a run's end.
+    s.total = s.off_idx + round_up(idx_bytes, 256) + 512;
+    return s;
+}
+
+int64_t idx_upper_bound(int64_t nnz, int columns, const Geometry& g)
+{
+    // every run rounds up by at most 3 bytes; two runs per (column, tile)
+    return round_up(nnz + (int64_t)6 * columns * g.n_tiles, 4);
+}
+
+// Per (device tile, column) counts from the tiled-CSC offsets and local rows.
+int count_device_tiles(const int32_t* row, const int32_t* off_tiled, int columns, int inners, int tile_k,
+                       const Geometry& g, std::vector<uint16_t>* counts)
+{
+    const int Ta = (int)ceil_div(inners, tile_k);
+    counts->assign((size_t)columns * g.n_tiles, 0);
+    for (int y = 0; y < columns; ++y)
+        for (int t = 0; t < Ta; ++t) {
+            const int32_t b = off_tiled[((size_t)y * Ta + t) * 2], e = off_tiled[((size_t)y * Ta + t) * 2 + 1];
+            if (b < 0 || e < b) return fail(TL_ERR_FORMAT, "column %d tile %d: offsets [%d, %d) are not ordered", y, t, b, e);
+            for (int32_t i = b; i < e; ++i) {
+                const int64_t k = (int64_t)t * tile_k + row[i];
+                if (row[i] < 0 || row[i] >= tile_k || k >= inners)
+                    return fail(TL_ERR_FORMAT, "column %d tile %d: local row %d out of range", y, t, row[i]);
+                (*counts)[(size_t)(k / g.tile_rows) * columns + y]++;
+            }
+        }
+    return TL_OK;
+}
+
+// Last "end" entry of a tiled-CSC offset array = number of stored rows of that sign.
+int64_t stream_length(const int32_t* off_tiled, int columns, int inners, int tile_k)
+{
+    const int Ta = (int)ceil_div(inners, tile_k);
+    return off_tiled[((size_t)columns * Ta - 1) * 2 + 1];
+}
+
+}  // namespace
+
+extern "C" int tl_layout_size(const int32_t* neg_off_tiled, const int32_t* pos_off_tiled,
+                              int columns, int inners, int tile_k, int tile_rows, int64_t* blob_bytes)
+{
+    if (!neg_off_tiled || !pos_off_tiled || !blob_bytes) return fail(TL_ERR_ARG, "null pointer");
+    if (columns <= 0 || inners <= 0 || tile_k <= 0) return fail(TL_ERR_SHAPE, "bad dimensions");
+    Geometry g;
+    if (int rc = pick_geometry(columns, inners, tile_rows, &g)) return rc;
+    const int64_t nnz = stream_length(neg_off_tiled, columns, inners, tile_k) + stream_length(pos_off_tiled, columns, inners, tile_k);
+    *blob_bytes = place_sections(g, idx_upper_bound(nnz, columns, g)).total;
+    return TL_OK;
+}
+
+extern "C" int tl_layout_build(const int32_t* neg_row, const int32_t* neg_off_tiled,
+                               const int32_t* pos_row, const int32_t* pos_off_tiled,
+                               int columns, int inners, int tile_k, int tile_rows,
+                               void* blob, int64_t blob_bytes)
+{
+    if (!neg_off_tiled || !pos_off_tiled || !blob) return fail(TL_ERR_ARG, "null pointer");
+    if (columns <= 0 || inners <= 0 || tile_k <= 0) return fail(TL_ERR_SHAPE, "bad dimensions");
+    Geometry g;
+    if (int rc = pick_geometry(columns, inners, tile_rows, &g)) return rc;
+    int64_t budget = 0;
+    if (int rc = tl_layout_size(neg_off_tiled, pos_off_tiled, columns, inners, tile_k, tile_rows, &budget)) return rc;
+    if (blob_bytes < budget) return fail(TL_ERR_SIZE, "blob has %lld bytes, %lld needed", (long long)blob_bytes, (long long)budget);
+    const int64_t n_pos = stream_length(pos_off_tiled, columns, inners, tile_k);
+    const int64_t n_neg = stream_length(neg_off_tiled, columns, inners, tile_k);
+    if ((n_pos > 0 && !pos_row) || (n_neg > 0 && !neg_row)) return fail(TL_ERR_ARG, "row array is null");
+
+    std::vector<uint16_t> cp, cn;  // [tile][column]
+    if (int rc = count_device_tiles(pos_row, pos_off_tiled, columns, inners, tile_k, g, &cp)) return rc;
+    if (int rc = count_device_tiles(neg_row, neg_off_tiled, columns, inners, tile_k, g, &cn)) return rc;
+
+    const int T = g.n_tiles, NB = g.n_blocks, NP = NB * kBlock;
+    const int Ta = (int)ceil_div(inners, tile_k);
+    const int64_t reserve = idx_upper_bound(n_pos + n_neg, columns, g);
+    const Sections s = place_sections(g, reserve);
+    std::memset(blob, 0, (size_t)blob_bytes);
+    uint8_t* base = static_cast<uint8_t*>(blob);
+    uint32_t* blockstart = reinterpret_cast<uint32_t*>(base + s.off_blockstart);
+    uint32_t* desc = reinterpret_cast<uint32_t*>(base + s.off_desc);
+    uint8_t* idx = base + s.off_idx;
+
+    // Pass 1: descriptors and block starts, tile-major.
+    uint64_t dwords = 0, run_sum = 0;
+    uint32_t run_max = 0;
+    for (int t = 0; t < T; ++t)
+        for (int nb = 0; nb < NB; ++nb) {
+            blockstart[(size_t)t * NB + nb] = (uint32_t)dwords;
+            uint32_t in_block = 0;
+            for (int j = 0; j < kBlock; ++j) {
+                const int y = nb * kBlock + j;
+                uint32_t p = 0, n = 0;
+                if (y < columns) {
+                    p = cp[(size_t)t * columns + y];
+                    n = cn[(size_t)t * columns + y];
+                }
+                if (p > 255 || n > 255) return fail(TL_ERR_FORMAT, "column %d tile %d holds %u/%u rows of one sign", y, t, p, n);
+                desc[(size_t)t * NP + y] = make_desc(p, n, in_block);
+                const uint32_t run = (p + 3) / 4 + (n + 3) / 4;
+                in_block += run;  // at most 64 * 128 dwords: always fits 16 bits
+                if (y < columns) {
+                    run_sum += run;
+                    if (run > run_max) run_max = run;
+                }
+            }
+            dwords += in_block;
+        }
+    blockstart[(size_t)T * NB] = (uint32_t)dwords;
+    if (dwords * 4 > (uint64_t)reserve || dwords > 0xffffffffull)
+        return fail(TL_ERR_UNSUPPORTED, "index stream of %llu dwords does not fit", (unsigned long long)dwords);
+    std::memset(idx, kSentinel, (size_t)dwords * 4);
+
+    // Pass 2: scatter the rows.  Rows arrive ascending per column, so one cursor per
+    // (device tile, sign) of the current column fills every run in ascending order.
+    std::vector<uint64_t> cursor((size_t)T * 2);
+    for (int y = 0; y < columns; ++y) {
+        for (int t = 0; t < T; ++t) {
+            const uint32_t d = desc[(size_t)t * NP + y];
+            const uint64_t start = ((uint64_t)blockstart[(size_t)t * NB + y / kBlock] + (d >> 16)) * 4;
+            cursor[2 * t] = start;
+            cursor[2 * t + 1] = start + (((d & 0xff) + 3) / 4) * 4;
+        }
+        for (int sign = 0; sign < 2; ++sign) {
+            const int32_t* row = sign == 0 ? pos_row : neg_row;
+            const int32_t* off = sign == 0 ? pos_off_tiled : neg_off_tiled;
+            for (int t = 0; t < Ta; ++t)
+                for (int32_t i = off[((size_t)y * Ta + t) * 2]; i < off[((size_t)y * Ta + t) * 2 + 1]; ++i) {
+                    const int k = t * tile_k + row[i];
+                    idx[cursor[2 * (k / g.tile_rows) + sign]++] = (uint8_t)(k % g.tile_rows);
+                }
+        }
+    }
+
+    tl_layout_header h;
+    std::memset(&h, 0, sizeof(h));
+    static_assert(sizeof(tl_layout_header) == 256, "header must stay 256 bytes");
+    h.magic = TL_LAYOUT_MAGIC;
+    h.version = 2;
+    h.inners = (uint32_t)inners;
+    h.columns = (uint32_t)columns;
+    h.tile_rows = (uint32_t)g.tile_rows;
+    h.n_tiles = (uint32_t)T;
+    h.n_blocks = (uint32_t)NB;
+    h.nnz_pos = (uint64_t)n_pos;
+    h.nnz_neg = (uint64_t)n_neg;
+    h.off_blockstart = (uint64_t)s.off_blockstart;
+    h.off_desc = (uint64_t)s.off_desc;
+    h.off_idx = (uint64_t)s.off_idx;
+    h.idx_bytes = dwords * 4;
+    // The blob handed in is sized by an upper bound; what the format occupies is smaller.
+    h.total_bytes = (uint64_t)place_sections(g, (int64_t)dwords * 4).total;
+    h.max_run_dwords = run_max;
+    h.mean_run_dwords_x16 = (uint32_t)ceil_div((int64_t)run_sum * 16, (int64_t)columns * T);
+    std::memcpy(blob, &h, sizeof(h));
+    return TL_OK;
+}
+
+extern "C" int tl_layout_from_dense(const int32_t* w, int columns, int inners, int tile_rows,
+                                    void* blob, int64_t* blob_bytes)
+{
+    if (!w || !blob_bytes) return fail(TL_ERR_ARG, "null pointer");
+    if (columns <= 0 || inners <= 0) return fail(TL_ERR_SHAPE, "bad dimensions");
+    int64_t p = 0, n = 0;
+    if (int rc = tl_count_nnz(w, columns, inners, &p, &n)) return rc;
+    if (p > INT32_MAX || n > INT32_MAX) return fail(TL_ERR_UNSUPPORTED, "more than 2^31 non-zeros of one sign");
+    Geometry g;
+    if (int rc = pick_geometry(columns, inners, tile_rows, &g)) return rc;
+    // Pack with the device tile height directly: the API-level tiles then coincide with device tiles.
+    const int T = g.n_tiles;
+    std::vector<int32_t> neg_row((size_t)n + 1), pos_row((size_t)p + 1), neg_off((size_t)columns * T * 2),
+        pos_off((size_t)columns * T * 2);
+    if (int rc = tl_convert_to_ter_tiled_csc(w, columns, inners, (int)p, (int)n, g.tile_rows, neg_row.data(),
+                                             neg_off.data(), pos_row.data(), pos_off.data()))
+        return rc;
+    int64_t need = 0;
+    if (int rc = tl_layout_size(neg_off.data(), pos_off.data(), columns, inners, g.tile_rows, g.tile_rows, &need)) return rc;
+    if (!blob) {
+        *blob_bytes = need;
+        return TL_OK;
+    }
+    if (*blob_bytes < need) return fail(TL_ERR_SIZE, "blob has %lld bytes, %lld needed", (long long)*blob_bytes, (long long)need);
+    return tl_layout_build(neg_row.data(), neg_off.data(), pos_row.data(), pos_off.data(), columns, inners, g.tile_rows,
+                           g.tile_rows, blob, *blob_bytes);
+}
+
+extern "C" int tl_layout_validate(const void* blob, int64_t blob_bytes)
+{
+    if (!blob) return fail(TL_ERR_ARG, "null blob");
+    if (blob_bytes < (int64_t)sizeof(tl_layout_header)) return fail(TL_ERR_FORMAT, "blob shorter than its header");
+    tl_layout_header h;
+    std::memcpy(&h, blob, sizeof(h));
+    if (h.magic != TL_LAYOUT_MAGIC || h.version != 2) return fail(TL_ERR_FORMAT, "bad magic/version %08x/%u", h.magic, h.version);
+    if (h.tile_rows == 0 || h.tile_rows > (uint32_t)kMaxTileRows || h.columns == 0 || h.inners == 0 ||
+        h.n_tiles != (uint32_t)ceil_div(h.inners, h.tile_rows) || h.n_blocks != (uint32_t)ceil_div(h.columns, kBlock))
+        return fail(TL_ERR_FORMAT, "inconsistent geometry K=%u N=%u rows=%u tiles=%u blocks=%u", h.inners, h.columns,
+                    h.tile_rows, h.n_tiles, h.n_blocks);
+    Geometry g{(int)h.tile_rows, (int)h.n_tiles, (int)h.n_blocks};
+    const Sections s = place_sections(g, (int64_t)h.idx_bytes);
+    if (h.off_blockstart != (uint64_t)s.off_blockstart || h.off_desc != (uint64_t)s.off_desc || h.off_idx != (uint64_t)s.off_idx ||
+        h.total_bytes != (uint64_t)s.total || h.total_bytes > (uint64_t)blob_bytes || (h.idx_bytes & 3))
+        return fail(TL_ERR_FORMAT, "section table does not match the geometry");
+    const uint8_t* base = static_cast<const uint8_t*>(blob);
+    const uint32_t* blockstart = reinterpret_cast<const uint32_t*>(base + h.off_blockstart);
+    const uint32_t* desc = reinterpret_cast<const uint32_t*>(base + h.off_desc);
+    const uint8_t* idx = base + h.off_idx;
+    const uint32_t T = h.n_tiles, NB = h.n_blocks, NP = NB * kBlock;
+    uint64_t np = 0, nn = 0, expect_start = 0;
+    uint32_t run_max = 0;
+    for (uint32_t t = 0; t < T; ++t) {
+        const uint32_t rows_here = (t + 1 == T) ? h.inners - t * h.tile_rows : h.tile_rows;
+        for (uint32_t nb = 0; nb < NB; ++nb) {
+            if (blockstart[(size_t)t * NB + nb] != expect_start)
+                return fail(TL_ERR_FORMAT, "tile %u block %u: start %u, expected %llu", t, nb, blockstart[(size_t)t * NB + nb],
+                            (unsigned long long)expect_start);
+            uint32_t expect = 0;
+            for (uint32_t j = 0; j < (uint32_t)kBlock; ++j) {
+                const uint32_t y = nb * kBlock + j;
+                const uint32_t d = desc[(size_t)t * NP + y], p = d & 0xff, n = (d >> 8) & 0xff, off = d >> 16;
+                if (off != expect) return fail(TL_ERR_FORMAT, "tile %u column %u: run offset %u, expected %u", t, y, off, expect);
+                if (y >= h.columns && (p || n)) return fail(TL_ERR_FORMAT, "tile %u: padding column %u is not empty", t, y);
+                const uint32_t pd = (p + 3) / 4, nd = (n + 3) / 4;
+                if ((expect_start + off + pd + nd) * 4 > h.idx_bytes) return fail(TL_ERR_FORMAT, "tile %u column %u: run leaves the stream", t, y);
+                const uint8_t* run = idx + (expect_start + off) * 4;
+                for (int sign = 0; sign < 2; ++sign) {
+                    const uint8_t* r = sign ? run + 4 * pd : run;
+                    const uint32_t cnt = sign ? n : p, padded = sign ? 4 * nd : 4 * pd;
+                    for (uint32_t i = 0; i < padded; ++i) {
+                        if (i < cnt) {
+                            if (r[i] >= rows_here || (i > 0 && r[i] <= r[i - 1]))
+                                return fail(TL_ERR_FORMAT, "tile %u column %u: rows not ascending / out of range", t, y);
+                        } else if (r[i] != kSentinel) {
+                            return fail(TL_ERR_FORMAT, "tile %u column %u: padding byte is not the sentinel", t, y);
+                        }
+                    }
+                }
+                np += p;
+                nn += n;
+                expect += pd + nd;
+                if (pd + nd > run_max) run_max = pd + nd;
+            }
+            expect_start += expect;
+        }
+    }
+    if (blockstart[(size_t)T * NB] != expect_start || expect_start * 4 != h.idx_bytes)
+        return fail(TL_ERR_FORMAT, "stream length does not match the block table");
+    if (np != h.nnz_pos || nn != h.nnz_neg || run_max != h.max_run_dwords)
+        return fail(TL_ERR_FORMAT, "header totals do not match the streams");
+    return TL_OK;
+}
+
+extern "C" int tl_layout_to_dense(const void* blob, int64_t blob_bytes, int32_t* w_out)
+{
+    if (!w_out) return fail(TL_ERR_ARG, "null output");
+    if (int rc = tl_layout_validate(blob, blob_bytes)) return rc;
+    tl_layout_header h;
+    std::memcpy(&h, blob, sizeof(h));
+    const uint8_t* base = static_cast<const uint8_t*>(blob);
+    const uint32_t* blockstart = reinterpret_cast<const uint32_t*>(base + h.off_blockstart);
+    const uint32_t* desc = reinterpret_cast<const uint32_t*>(base + h.off_desc);
+    const uint8_t* idx = base + h.off_idx;
+    const uint32_t NB = h.n_blocks, NP = NB * kBlock;
+    std::memset(w_out, 0, sizeof(int32_t) * (size_t)h.inners * h.columns);
+    for (uint32_t t = 0; t < h.n_tiles; ++t)
+        for (uint32_t y = 0; y < h.columns; ++y) {
+            const uint32_t d = desc[(size_t)t * NP + y], p = d & 0xff, n = (d >> 8) & 0xff;
+            const uint8_t* run = idx + ((size_t)blockstart[(size_t)t * NB + y / kBlock] + (d >> 16)) * 4;
+            for (uint32_t i = 0; i < p; ++i) w_out[((size_t)t * h.tile_rows + run[i]) * h.columns + y] = 1;
+            run += ((p + 3) / 4) * 4;
+            for (uint32_t i = 0; i < n; ++i) w_out[((size_t)t * h.tile_rows + run[i]) * h.columns + y] = -1;
+        }
+    return TL_OK;
+}

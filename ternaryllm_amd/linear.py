@@ -1,0 +1,169 @@
+"""TernaryLinear: the reference's module (ternaryLLM_GPU/TernaryLLM/TernaryLinear.py:115-182) on
+top of the gfx950 library.  Constructor arguments, buffer names and the forward contract are
+the reference's; additions are keyword-only."""
+import numpy as np
+import torch
+from torch import nn
+
+from . import ops, packing
+
+# K -> tile height of the merged format, TernaryLinear.py:9-16.  The reference raises KeyError for
+# any other K (e.g. 11008); here other sizes take the largest listed height that divides K, else 256.
+MapKSizeToTileSize = {8192: 512, 4096: 512, 3072: 512, 2048: 256, 1024: 256, 512: 64}
+
+
+def merged_tile_size(k):
+    if k in MapKSizeToTileSize:
+        return MapKSizeToTileSize[k]
+    for t in (512, 256, 64):
+        if k % t == 0:
+            return t
+    return 256
+
+
+def ternarize_weights(w):
+    raise NotImplementedError("ternarize_weights not implement")  # as in the reference, TernaryLinear.py:19-20
+
+
+def random_ternary_weights(size, sparsity=0.8, uniform=False, block_size=512, generator=None):
+    """Random ternary [K, N] int32 matrix, distributed as the reference's generator
+    (TernaryLinear.py:23-85).  i.i.d. mode: r ~ U[0,1); r < s -> 0, s <= r < (s+1)/2 -> -1, else +1.
+    uniform mode: the flattened [N, K] matrix is cut into blocks of `block_size`; every block gets the
+    same even number of non-zeros (plus 2 for the first few to reach the total), half +1 half -1, at
+    random positions.  `generator` (a CPU torch.Generator) makes the draw reproducible."""
+    K, N = int(size[0]), int(size[1])
+    if not uniform:
+        r = torch.rand((K, N), generator=generator)
+        w = torch.zeros((K, N), dtype=torch.int32)
+        w[(r >= sparsity) & (r < (sparsity + 1) / 2)] = -1
+        w[r >= (sparsity + 1) / 2] = 1
+        return w
+    total = K * N
+    n_blocks = total // block_size
+    if n_blocks == 0:
+        raise ValueError("block_size exceeds the matrix")
+    nnz = int(total * (1 - sparsity))
+    nnz -= nnz % 2
+    per_block = (nnz // n_blocks) // 2 * 2
+    counts = torch.full((n_blocks,), per_block, dtype=torch.int64)
+    extra = (nnz - per_block * n_blocks) // 2
+    if extra > 0:
+        reps = torch.arange(extra) % n_blocks
+        counts += 2 * torch.bincount(reps, minlength=n_blocks)
+    if int(counts.max()) > block_size:
+        raise ValueError("sparsity too low for this block size")
+    # rank of a random key inside each block = a random permutation of its positions
+    keys = torch.rand((n_blocks, block_size), generator=generator)
+    rank = keys.argsort(dim=1).argsort(dim=1)
+    half = (counts // 2).unsqueeze(1)
+    blocks = torch.zeros((n_blocks, block_size), dtype=torch.int32)
+    blocks[rank < half] = 1
+    blocks[(rank >= half) & (rank < 2 * half)] = -1
+    flat = torch.zeros(total, dtype=torch.int32)
+    flat[: n_blocks * block_size] = blocks.reshape(-1)
+    return flat.view(N, K).T.contiguous()
+
+
+def convert_ternary_weights(w, padding=False, padding_size=4, dtype=torch.int32, device="cpu"):
+    """Merged tiled-CSC arrays of a ternary weight: (row_indices, col_offsets, col_tile_indices),
+    as the reference's helper of the same name (TernaryLinear.py:87-113)."""
+    w_ = w.detach().to("cpu", torch.int32).contiguous()
+    cnt_pos, cnt_neg = packing.count_nnz(w_)
+    k, n = w_.shape
+    merged = packing.convert_to_ter_tiled_mcsc(w_, n, k, cnt_pos, cnt_neg, merged_tile_size(k), padding, padding_size)
+    row_indices = torch.from_numpy(merged[0]).to(device).contiguous().to(dtype)
+    col_offsets = torch.from_numpy(merged[1]).to(device).contiguous()
+    col_tile_indices = torch.from_numpy(merged[2]).to(device).contiguous().to(dtype)
+    return row_indices, col_offsets, col_tile_indices
+
+
+class TernaryLinear(nn.Module):
+    """y = x @ W (* scale) for a ternary W, W generated at random as in the reference.
+
+    Reference arguments: in_features (K), out_features (N), sparsity, uniform, uniform_blk_size,
+    padding, padding_size, bias, device, dtype.  As in the reference the bias is allocated but never
+    added (TernaryLinear.py:137-140, :152-182).
+    Keyword-only additions: `weight` (use this int32 [K, N] ternary matrix instead of a random one),
+    `scale` (per-output-channel factor, [N]), `generator` (seed for the random weight),
+    `reference_buffers` (also build the reference's merged arrays; they are not used by forward).
+    """
+    __constants__ = ["in_features", "out_features"]
+
+    def __init__(self, in_features, out_features, sparsity=0.8, uniform=False, uniform_blk_size=512, padding=False,
+                 padding_size=4, bias=True, device=None, dtype=torch.int32, *, weight=None, scale=None, generator=None,
+                 reference_buffers=True):
+        super().__init__()
+        if bias:
+            self.bias = nn.Parameter(torch.zeros(out_features, device=device), requires_grad=False)
+        else:
+            self.register_parameter("bias", None)
+        if weight is None:
+            weight = random_ternary_weights((in_features, out_features), sparsity, uniform, uniform_blk_size, generator)
+        else:
+            weight = torch.as_tensor(weight).to("cpu", torch.int32).contiguous()
+            if tuple(weight.shape) != (in_features, out_features):
+                raise ValueError(f"weight must be [{in_features}, {out_features}]")
+        self.ternary_weight = weight  # kept on the CPU as a plain attribute, as in the reference
+        if reference_buffers:
+            rows, offs, tiles = convert_ternary_weights(weight, padding=padding, padding_size=padding_size, device=device,
+                                                        dtype=torch.int16)
+        else:
+            rows, offs, tiles = (torch.zeros(0, dtype=torch.int16, device=device), torch.zeros(0, dtype=torch.int32, device=device),
+                                 torch.zeros(0, dtype=torch.int16, device=device))
+        self.register_buffer("w_row_indices", rows, False)
+        self.register_buffer("w_col_offsets", offs, False)
+        self.register_buffer("w_col_tile_indices", tiles, False)
+        packed = packing.PackedWeight.from_dense(weight)
+        self._header = packed.header
+        self._packed_nnz = packed.nnz
+        self.register_buffer("w_packed", torch.from_numpy(packed.blob.copy()).to(device), True)
+        if scale is not None:
+            scale = torch.as_tensor(scale).reshape(-1)
+            if scale.numel() != out_features:
+                raise ValueError("scale must have out_features elements")
+            self.register_buffer("w_scale", scale.to(device).contiguous(), True)
+        else:
+            self.w_scale = None
+        self.in_features = in_features
+        self.out_features = out_features
+        self.uniform = uniform
+        self.padding = padding
+        self._handle = None
+
+    def device_weight(self):
+        """The DeviceWeight view of `w_packed` on its current device."""
+        h = self._handle
+        if h is None or h.blob.data_ptr() != self.w_packed.data_ptr():
+            h = ops.DeviceWeight.__new__(ops.DeviceWeight)
+            h.header = self._header
+            h.blob = self.w_packed
+            if h.blob.device.type != "cuda":
+                raise RuntimeError("TernaryLinear runs on a GPU only: call .to('cuda') first")
+            self._handle = h
+        return h
+
+    def forward(self, input):
+        """input: (batch, rows, K), (rows, K) or (K,) -- also (batch, K, rows) as the reference kernel
+        reads it; returns (batch, rows, N) / (rows, N) / (N,) in the input dtype."""
+        if input.dim() > 3:
+            raise AssertionError("Input has dim larger than 3")  # the reference asserts (TernaryLinear.py:161)
+        w = self.device_weight()
+        K, N = self.in_features, self.out_features
+        if input.shape[-1] == K:
+            lead = input.shape[:-1]
+            y = ops.spmm(w, input.reshape(-1, K), self.w_scale)
+            return y.reshape(*lead, N)
+        if input.dim() >= 2 and input.shape[-2] == K:  # K-major activations
+            if input.dim() == 2:
+                return ops.spmm(w, input, self.w_scale, x_layout=1)
+            out = torch.empty((input.shape[0], input.shape[2], N), dtype=input.dtype, device=input.device)
+            for b in range(input.shape[0]):
+                ops.spmm(w, input[b], self.w_scale, x_layout=1, out=out[b])
+            return out
+        raise ValueError(f"input of shape {tuple(input.shape)} does not match in_features={K}")
+
+    def extra_repr(self):
+        return f"in_features={self.in_features}, out_features={self.out_features}, nnz={self._packed_nnz}"
+
+
+__all__ = ["TernaryLinear", "random_ternary_weights", "convert_ternary_weights", "MapKSizeToTileSize"]

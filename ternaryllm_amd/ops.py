@@ -1,0 +1,176 @@
+"""Tensor-level entry points over the C ABI: device weights and the ternary product.
+
+torch is used for device memory and streams only; every product runs in libternary_spmm.so.
+"""
+import ctypes
+
+import numpy as np
+import torch
+
+from . import _lib
+from .packing import PackedWeight
+
+_DTYPE_CODE = {torch.float32: _lib.TL_F32, torch.float16: _lib.TL_F16}
+
+
+def _code(dtype, what):
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise ValueError(f"{what} must be float32 or float16, got {dtype}") from None
+
+
+def _stream_ptr(device):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+class DeviceWeight:
+    """A packed ternary weight resident on one GPU: the blob as a uint8 tensor plus the host header."""
+
+    def __init__(self, packed, device):
+        if not isinstance(packed, PackedWeight):
+            raise TypeError("packed must be a PackedWeight")
+        self.header = packed.header
+        self.blob = torch.from_numpy(packed.blob).to(device)
+        if self.blob.device.type != "cuda":
+            raise RuntimeError("the ternary product runs on a GPU only: move the weight to a cuda device")
+        if self.blob.data_ptr() % 256:
+            raise RuntimeError("device allocator returned a blob that is not 256-byte aligned")
+        self.algorithmic_bytes = packed.algorithmic_bytes
+
+    @classmethod
+    def from_blob_tensor(cls, blob_tensor):
+        """Rebuilds the handle from a uint8 tensor that already holds a blob (e.g. a module buffer)."""
+        self = cls.__new__(cls)
+        head = blob_tensor[:256].cpu().numpy().tobytes()
+        self.header = _lib.LayoutHeader.from_buffer_copy(head)
+        if self.header.magic != _lib.TL_LAYOUT_MAGIC:
+            raise ValueError("tensor does not hold a packed ternary weight")
+        self.blob = blob_tensor
+        return self
+
+    @property
+    def inners(self):
+        return self.header.inners
+
+    @property
+    def columns(self):
+        return self.header.columns
+
+    @property
+    def device(self):
+        return self.blob.device
+
+
+def _x_geometry(x, K, x_layout):
+    if x.dim() != 2:
+        raise ValueError("x must be 2-D here; fold batch dimensions first")
+    if x_layout == _lib.TL_X_ROW_MAJOR:
+        if x.shape[1] != K:
+            raise ValueError(f"x has {x.shape[1]} columns, the weight has K={K}")
+        M = x.shape[0]
+    else:
+        if x.shape[0] != K:
+            raise ValueError(f"x has {x.shape[0]} rows, the weight has K={K}")
+        M = x.shape[1]
+    if x.stride(1) != 1:
+        x = x.contiguous()
+    return x, M, x.stride(0) if x.shape[0] > 1 else max(x.shape[1], 1)
+
+
+def _workspace(header, M, x_code, x_layout, device):
+    need = ctypes.c_int64(0)
+    _lib.check(_lib.lib().tl_spmm_workspace(ctypes.byref(header), M, x_code, x_layout, ctypes.byref(need)))
+    if need.value == 0:
+        return None, 0
+    ws = torch.empty(need.value, dtype=torch.uint8, device=device)
+    return ws, need.value
+
+
+def _scale_args(scale, N, device):
+    if scale is None:
+        return None, _lib.TL_F32
+    if scale.device != device or scale.numel() != N or not scale.is_contiguous():
+        raise ValueError("scale must be a contiguous tensor of N elements on the weight's device")
+    return scale, _code(scale.dtype, "scale")
+
+
+def spmm(weight, x, scale=None, out_dtype=None, x_layout=_lib.TL_X_ROW_MAJOR, out=None):
+    """y[M, N] = (x @ W) * scale with fp32 accumulation.
+
+    weight: DeviceWeight; x: cuda tensor [M, K] (row-major layout) or [K, M] (K-major layout),
+    float32 or float16; scale: optional [N] tensor; returns a new [M, N] tensor of out_dtype
+    (default: x.dtype)."""
+    if x.device != weight.device:
+        raise RuntimeError(f"x is on {x.device}, the weight on {weight.device}")
+    x_code = _code(x.dtype, "x")
+    x, M, ldx = _x_geometry(x, weight.inners, x_layout)
+    N = weight.columns
+    out_dtype = out_dtype or x.dtype
+    y_code = _code(out_dtype, "out_dtype")
+    if M == 0:
+        return torch.empty((0, N), dtype=out_dtype, device=x.device)
+    y = out if out is not None else torch.empty((M, N), dtype=out_dtype, device=x.device)
+    if y.shape != (M, N) or y.dtype != out_dtype or y.stride(1) != 1:
+        raise ValueError("out must be an [M, N] tensor of out_dtype with unit column stride")
+    scale, s_code = _scale_args(scale, N, x.device)
+    ws, ws_bytes = _workspace(weight.header, M, x_code, x_layout, x.device)
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().tl_spmm(ctypes.byref(weight.header), weight.blob.data_ptr(), x.data_ptr(), x_code, x_layout, ldx, M,
+                                y.data_ptr(), y_code, y.stride(0), scale.data_ptr() if scale is not None else None, s_code,
+                                ws.data_ptr() if ws is not None else None, ws_bytes, _stream_ptr(x.device))
+    _lib.check(rc)
+    if ws is not None:
+        ws.record_stream(torch.cuda.current_stream(x.device))
+    return y
+
+
+def mlp_gate_up(gate, up, x, gate_scale=None, up_scale=None, out_dtype=None):
+    """h[M, N] = silu((x @ Wg) * sg) * ((x @ Wu) * su) in one pass over x (M > 48), else two products."""
+    if gate.columns != up.columns or gate.inners != up.inners:
+        raise ValueError("gate and up weights must have the same shape")
+    x_code = _code(x.dtype, "x")
+    x, M, ldx = _x_geometry(x, gate.inners, _lib.TL_X_ROW_MAJOR)
+    N = gate.columns
+    out_dtype = out_dtype or x.dtype
+    if M <= 48 or gate.header.tile_rows != up.header.tile_rows:
+        g = spmm(gate, x, gate_scale, torch.float32)
+        u = spmm(up, x, up_scale, torch.float32)
+        return (torch.nn.functional.silu(g) * u).to(out_dtype)
+    h = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    gs, s_code = _scale_args(gate_scale, N, x.device)
+    us, s_code2 = _scale_args(up_scale, N, x.device)
+    if (gs is None) != (us is None) or (gs is not None and s_code != s_code2):
+        raise ValueError("pass both scales, of one dtype, or neither")
+    ws, ws_bytes = _workspace(gate.header, M, x_code, _lib.TL_X_ROW_MAJOR, x.device)
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().tl_mlp_gate_up(ctypes.byref(gate.header), gate.blob.data_ptr(), ctypes.byref(up.header),
+                                       up.blob.data_ptr(), x.data_ptr(), x_code, _lib.TL_X_ROW_MAJOR, ldx, M, h.data_ptr(),
+                                       _code(out_dtype, "out_dtype"), h.stride(0), gs.data_ptr() if gs is not None else None,
+                                       us.data_ptr() if us is not None else None, s_code, _lib.TL_ACT_SILU_GATE,
+                                       ws.data_ptr() if ws is not None else None, ws_bytes, _stream_ptr(x.device))
+    _lib.check(rc)
+    if ws is not None:
+        ws.record_stream(torch.cuda.current_stream(x.device))
+    return h
+
+
+def spmm_time(weight, x, iters, scale=None, out_dtype=None):
+    """Mean milliseconds per tl_spmm call over `iters` back-to-back calls, timed with HIP events
+    recorded on the stream the kernels run on."""
+    x_code = _code(x.dtype, "x")
+    x, M, ldx = _x_geometry(x, weight.inners, _lib.TL_X_ROW_MAJOR)
+    N = weight.columns
+    out_dtype = out_dtype or x.dtype
+    y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    scale, s_code = _scale_args(scale, N, x.device)
+    ws, ws_bytes = _workspace(weight.header, M, x_code, _lib.TL_X_ROW_MAJOR, x.device)
+    ms = ctypes.c_float(0)
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().tl_spmm_time(ctypes.byref(weight.header), weight.blob.data_ptr(), x.data_ptr(), x_code,
+                                     _lib.TL_X_ROW_MAJOR, ldx, M, y.data_ptr(), _code(out_dtype, "out_dtype"), y.stride(0),
+                                     scale.data_ptr() if scale is not None else None, s_code,
+                                     ws.data_ptr() if ws is not None else None, ws_bytes, _stream_ptr(x.device), iters,
+                                     ctypes.byref(ms))
+    _lib.check(rc)
+    return ms.value, y

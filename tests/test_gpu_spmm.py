@@ -1,0 +1,117 @@
+"""GPU parity of the ternary product against the CPU oracle, through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+from tests.util import FP16_TOL, FP32_TOL, activations, max_rel_err, ternary_weight
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(cuda, oracle, M, K, N, s, dtype, seed, integer=False, scale=False, out_dtype=None, tile_rows=0):
+    from ternaryllm_amd import ops
+    from ternaryllm_amd.packing import PackedWeight
+    w = ternary_weight(K, N, s, seed)
+    x = activations(M, K, seed + 1, dtype, integer)
+    pw = PackedWeight.from_dense(w, tile_rows)
+    dw = ops.DeviceWeight(pw, cuda)
+    sc = None
+    ref = oracle.fast_product(x.double().numpy(), w)
+    if scale:
+        g = torch.Generator().manual_seed(seed + 2)
+        sc = (0.5 + torch.rand(N, generator=g)).to(dtype)
+        ref = ref * sc.double().numpy()[None, :]
+    print(f"case M={M} K={K} N={N} s={s} dtype={dtype} int={integer} scale={scale}", flush=True)
+    y = ops.spmm(dw, x.to(cuda), sc.to(cuda) if sc is not None else None, out_dtype)
+    torch.cuda.synchronize()
+    return y.float().cpu().numpy(), ref, x.float().numpy(), w
+
+
+SHAPES = [
+    (1, 512, 256, 0.66), (1, 4096, 4096, 0.66), (2, 1000, 130, 0.5), (3, 777, 65, 0.8), (5, 4096, 1024, 0.9),
+    (8, 2048, 512, 0.8), (16, 4096, 4096, 0.5), (17, 1024, 320, 0.66), (33, 600, 200, 0.8), (48, 512, 512, 0.9),
+    (49, 512, 192, 0.8), (64, 1024, 256, 0.66), (100, 777, 130, 0.5), (256, 2048, 512, 0.8), (300, 4096, 1000, 0.9),
+    (1024, 4096, 1024, 0.8),
+]
+
+
+@pytest.mark.parametrize("M,K,N,s", SHAPES)
+def test_fp32_exact_on_integer_activations(cuda, oracle, M, K, N, s):
+    y, ref, x, w = _run(cuda, oracle, M, K, N, s, torch.float32, 11, integer=True)
+    assert np.array_equal(y.astype(np.float64), ref)
+
+
+@pytest.mark.parametrize("M,K,N,s", SHAPES)
+def test_fp16_exact_on_integer_activations(cuda, oracle, M, K, N, s):
+    y, ref, x, w = _run(cuda, oracle, M, K, N, s, torch.float16, 12, integer=True, out_dtype=torch.float32)
+    assert np.array_equal(y.astype(np.float64), ref)
+
+
+@pytest.mark.parametrize("M,K,N,s", SHAPES)
+def test_fp32_within_tolerance(cuda, oracle, M, K, N, s):
+    y, ref, x, w = _run(cuda, oracle, M, K, N, s, torch.float32, 21)
+    assert max_rel_err(y, ref, x, w) <= FP32_TOL
+
+
+@pytest.mark.parametrize("M,K,N,s", SHAPES)
+def test_fp16_within_tolerance(cuda, oracle, M, K, N, s):
+    y, ref, x, w = _run(cuda, oracle, M, K, N, s, torch.float16, 22, scale=True)
+    assert max_rel_err(y, ref, x, w) <= FP16_TOL
+
+
+@pytest.mark.parametrize("M", [1, 16, 128])
+def test_small_oracle_triple_loop(cuda, oracle, M):
+    """Same check against the oracle's own scalar triple loop (not BLAS) on a small case."""
+    K, N = 300, 70
+    w = ternary_weight(K, N, 0.6, 5)
+    x = activations(M, K, 6, torch.float32)
+    y, ref_fast, _, _ = _run(cuda, oracle, M, K, N, 0.6, torch.float32, 5)
+    ref = oracle.dense_product(x.numpy(), w)
+    assert np.allclose(ref, ref_fast, rtol=0, atol=1e-9)
+    assert max_rel_err(y, ref, x.numpy(), w) <= FP32_TOL
+
+
+@pytest.mark.parametrize("M", [1, 7, 200])
+@pytest.mark.parametrize("kind", ["zero", "one_per_column", "all_plus", "dense_pm"])
+def test_special_weights(cuda, oracle, M, kind):
+    from ternaryllm_amd import ops
+    from ternaryllm_amd.packing import PackedWeight
+    K, N = 520, 96
+    rng = np.random.default_rng(3)
+    w = np.zeros((K, N), np.int32)
+    if kind == "one_per_column":
+        rows = rng.integers(0, K, N)
+        signs = rng.choice([-1, 1], N)
+        w[rows, np.arange(N)] = signs
+    elif kind == "all_plus":
+        w[:, :] = 1
+    elif kind == "dense_pm":
+        w[:, :] = rng.choice([-1, 1], (K, N))
+    x = activations(M, K, 9, torch.float32, integer=True)
+    dw = ops.DeviceWeight(PackedWeight.from_dense(w), cuda)
+    y = ops.spmm(dw, x.to(cuda)).cpu().numpy()
+    xn = x.numpy().astype(np.float64)
+    if kind == "zero":
+        assert not y.any()
+    elif kind == "one_per_column":
+        assert np.array_equal(y, (xn[:, rows] * signs[None, :]).astype(np.float32))
+    elif kind == "all_plus":
+        assert np.array_equal(y, np.repeat(xn.sum(1, keepdims=True), N, 1).astype(np.float32))
+    else:
+        assert np.array_equal(y.astype(np.float64), xn @ w)
+
+
+def test_k_major_input_and_tile_heights(cuda, oracle):
+    from ternaryllm_amd import ops
+    from ternaryllm_amd.packing import PackedWeight
+    K, N = 1024, 256
+    w = ternary_weight(K, N, 0.7, 31)
+    for M in (4, 160):
+        x = activations(M, K, 32, torch.float32, integer=True)
+        ref = oracle.fast_product(x.numpy(), w)
+        for tile_rows in (0, 255, 128, 64, 100):
+            dw = ops.DeviceWeight(PackedWeight.from_dense(w, tile_rows), cuda)
+            y = ops.spmm(dw, x.to(cuda)).cpu().numpy()
+            assert np.array_equal(y.astype(np.float64), ref), (M, tile_rows)
+            yk = ops.spmm(dw, x.t().contiguous().to(cuda), x_layout=1).cpu().numpy()
+            assert np.array_equal(yk.astype(np.float64), ref), (M, tile_rows, "k-major")
