@@ -108,19 +108,23 @@ int tl_tiled_mcsc_to_dense(const void* merged_row, int index_width, int64_t n_in
 /* host from tiled CSC, copied to the GPU by the caller.                    */
 /*   - K is cut into tiles of `tile_rows` <= 255 rows; indices are 8-bit    */
 /*     tile-local, value 255 is a padding sentinel that addresses a zero.   */
-/*   - +1 and -1 rows of one (column, tile) are two separate runs, each     */
-/*     padded to a multiple of 4 bytes (the -1 run follows the +1 run).     */
-/*   - the index stream is tile-major: all runs of tile 0 in column order,  */
-/*     then tile 1, ...; columns are grouped in blocks of 64 and            */
-/*     blockstart[tile][block] gives the dword where a block's runs begin.  */
-/*   - per (tile, column) one 32-bit descriptor: +1 count (bits 0-7), -1    */
-/*     count (bits 8-15), dword offset of the run inside its block (16-31). */
-/*     The descriptor table is padded to whole blocks with empty columns.   */
+/*   - columns are grouped in blocks of 16.  The unit of the stream is the  */
+/*     chunk of one (block, tile): 16 descriptor dwords, then the runs of   */
+/*     the block's 16 columns for that tile.  Per column the +1 rows and    */
+/*     the -1 rows are two separate runs, each padded to a multiple of 4    */
+/*     bytes (the -1 run follows the +1 run).  A chunk is padded to a       */
+/*     multiple of 16 bytes.                                                */
+/*   - descriptor: +1 count (bits 0-7), -1 count (bits 8-15), dword offset  */
+/*     of the column's runs from the start of the chunk (bits 16-31).       */
+/*   - the stream is block-major: all tiles of block 0, then block 1, ...;  */
+/*     chunkstart[block * T + tile] is the dword where a chunk begins       */
+/*     (one extra entry marks the end).                                     */
 /* The blob starts with a tl_layout_header (256 bytes).                     */
 /* ======================================================================== */
 
-#define TL_LAYOUT_MAGIC 0x32474C54u /* "TLG2" */
-#define TL_BLOCK_COLUMNS 64
+#define TL_LAYOUT_MAGIC 0x34474C54u /* "TLG4" */
+#define TL_LAYOUT_VERSION 4
+#define TL_BLOCK_COLUMNS 16
 
 typedef struct tl_layout_header {
     uint32_t magic;
@@ -129,18 +133,17 @@ typedef struct tl_layout_header {
     uint32_t columns;     /* N */
     uint32_t tile_rows;   /* rows per device tile, <= 255 */
     uint32_t n_tiles;     /* T = ceil(K / tile_rows) */
-    uint32_t n_blocks;    /* NB = ceil(N / 64) */
-    uint32_t reserved0;
+    uint32_t n_blocks;    /* NB = ceil(N / 16) */
+    uint32_t max_chunk_dwords; /* largest chunk, descriptors included */
     uint64_t nnz_pos;
     uint64_t nnz_neg;
-    uint64_t off_blockstart; /* byte offset of uint32 blockstart[T*NB + 1] (dword units into idx) */
-    uint64_t off_desc;       /* byte offset of uint32 desc[T][NB*64]                               */
-    uint64_t off_idx;        /* byte offset of the index bytes                                     */
-    uint64_t idx_bytes;      /* padded index bytes (multiple of 4)                                 */
-    uint64_t total_bytes;    /* bytes of the blob that are in use, multiple of 256                 */
-    uint32_t max_run_dwords; /* largest (+1 run dwords + -1 run dwords) of any (column, tile)      */
-    uint32_t mean_run_dwords_x16; /* mean of the same, times 16, rounded up                        */
-    uint32_t reserved[40];
+    uint64_t off_chunkstart; /* byte offset of uint32 chunkstart[NB*T + 1] (dword units into the stream) */
+    uint64_t off_stream;     /* byte offset of the stream (descriptors + index bytes)                     */
+    uint64_t stream_bytes;   /* bytes of the stream (multiple of 16)                                      */
+    uint64_t total_bytes;    /* bytes of the blob that are in use, multiple of 256                        */
+    uint32_t max_run_dwords; /* largest (+1 run dwords + -1 run dwords) of any (column, tile)             */
+    uint32_t mean_run_dwords_x16; /* mean of the same, times 16, rounded up                               */
+    uint32_t reserved[42];
 } tl_layout_header;
 
 /* Bytes of the blob that tl_layout_build will write for these tiled-CSC arrays
@@ -171,7 +174,8 @@ int tl_layout_to_dense(const void* blob, int64_t blob_bytes, int32_t* w_out);
 /* ======================================================================== */
 
 /* Workspace bytes tl_spmm needs for M rows of x_dtype in x_layout (0 when none).
- * `header` is a host copy of the blob's first 256 bytes. */
+ * `header` is a host copy of the blob's first 256 bytes.  The workspace carries no
+ * state between calls; two calls that may run concurrently need different ones. */
 int tl_spmm_workspace(const tl_layout_header* header, int64_t M, int x_dtype, int x_layout,
                       int64_t* workspace_bytes);
 

@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(_DIR, "libternary_spmm.so")
 TL_F32, TL_F16 = 0, 1
 TL_X_ROW_MAJOR, TL_X_K_MAJOR = 0, 1
 TL_ACT_SILU_GATE = 1
-TL_LAYOUT_MAGIC = 0x32474C54
+TL_LAYOUT_MAGIC = 0x34474C54
 
 ERROR_NAMES = {
     -1: "TL_ERR_ARG", -2: "TL_ERR_SHAPE", -3: "TL_ERR_DTYPE", -4: "TL_ERR_ALIGN", -5: "TL_ERR_UNSUPPORTED",
@@ -29,12 +29,12 @@ class LayoutHeader(ctypes.Structure):
     _fields_ = [
         ("magic", ctypes.c_uint32), ("version", ctypes.c_uint32), ("inners", ctypes.c_uint32),
         ("columns", ctypes.c_uint32), ("tile_rows", ctypes.c_uint32), ("n_tiles", ctypes.c_uint32),
-        ("n_blocks", ctypes.c_uint32), ("reserved0", ctypes.c_uint32),
+        ("n_blocks", ctypes.c_uint32), ("max_chunk_dwords", ctypes.c_uint32),
         ("nnz_pos", ctypes.c_uint64), ("nnz_neg", ctypes.c_uint64),
-        ("off_blockstart", ctypes.c_uint64), ("off_desc", ctypes.c_uint64), ("off_idx", ctypes.c_uint64),
-        ("idx_bytes", ctypes.c_uint64), ("total_bytes", ctypes.c_uint64),
+        ("off_chunkstart", ctypes.c_uint64), ("off_stream", ctypes.c_uint64),
+        ("stream_bytes", ctypes.c_uint64), ("total_bytes", ctypes.c_uint64),
         ("max_run_dwords", ctypes.c_uint32), ("mean_run_dwords_x16", ctypes.c_uint32),
-        ("reserved", ctypes.c_uint32 * 40),
+        ("reserved", ctypes.c_uint32 * 42),
     ]
 
 

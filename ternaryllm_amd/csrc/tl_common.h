@@ -15,7 +15,7 @@ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline int64_t round_up(int64_t a, int64_t b) { return ceil_div(a, b) * b; }
 
 // Descriptor word of one (column, tile): bits 0-7 number of +1 rows, bits 8-15
-// number of -1 rows, bits 16-31 dword offset of the +1 run inside its 64-column block of the tile's
+// number of -1 rows, bits 16-31 dword offset of the +1 run from the start of its (block, tile) chunk of the
 // index stream (the -1 run follows the padded +1 run).
 inline uint32_t make_desc(uint32_t n_pos, uint32_t n_neg, uint32_t dword_off)
 {

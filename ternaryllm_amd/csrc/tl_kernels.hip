@@ -4,12 +4,12 @@
 // Two kernels replace the reference's pair
 // (ternaryLLM_GPU/csrc/ter_spmm_kernel.cuh:24-78 SpMV, :106-308 SpMM):
 //
-//   tl_spmm_small  M <= 48 (decode and small batches).  A group of LPC lanes owns
-//                  one output column and splits each (column, tile) run between its
-//                  lanes, one dword = four 8-bit row indices per lane; the
-//                  activation tiles sit in LDS as fp32 [slot][row]; every index is
-//                  one LDS gather and one fp32 add per activation row; the LPC
-//                  partial sums are folded with cross-lane shuffles.
+//   tl_spmm_block  M <= 48 (decode and small batches).  A workgroup owns a block of 16
+//                  columns over all of K and streams its chunks and the matching
+//                  activation rows through LDS; LPC lanes share a column and split
+//                  each run, four dwords = sixteen 8-bit row indices per lane; every
+//                  index is one LDS gather and one fp32 add per activation row; the
+//                  LPC partial sums are folded with cross-lane shuffles.
 //   tl_spmm_rows   larger M (prefill).  Lanes own activation rows, a wave owns C
 //                  output columns, so an index is wave-uniform: it is read through
 //                  the scalar path once and serves 64*R rows; the activation tile
@@ -38,9 +38,8 @@ __device__ __forceinline__ const_u32_ptr as_const(const uint32_t* p) { return (c
 #pragma clang diagnostic pop
 
 struct WeightPtrs {
-    const uint32_t* blockstart;  // [T * NB + 1]
-    const uint32_t* desc;        // [T][NB * 64]
-    const uint32_t* idx;         // dwords of four 8-bit rows
+    const uint32_t* chunkstart;  // [NB * T + 1], dword offsets into stream
+    const uint32_t* stream;      // chunks: 64 descriptors + runs of four 8-bit rows per dword
     const void* scale;           // per-column factor or null
 };
 
@@ -52,7 +51,8 @@ struct KernelArgs {
     long long ldx, ldy;
     int M, N, K, T, tile_rows, NB;
     int x_f16, x_kmajor, y_f16, scale_f16;
-    int tiles_per_stage;
+    int tiles_per_group;  // small-M kernel: activation tiles staged per pass
+    unsigned tile_magic;  // ceil(2^32 / tile_rows): k / tile_rows == (k * tile_magic) >> 32 for every k < 2^24
     float one;  // 1.0f, passed in so that the fp16 -> fp32 accumulate stays a single mixed-precision fma
 };
 
@@ -74,7 +74,7 @@ __device__ __forceinline__ int run_pos_dwords(uint32_t d) { return (int)(((d & 0
 __device__ __forceinline__ int run_neg_dwords(uint32_t d) { return (int)((((d >> 8) & 0xffu) + 3u) >> 2); }
 
 // ---------------------------------------------------------------------------
-// Small-M kernel.
+// Small-M kernel: one workgroup per (column block, range of tiles, block of rows).
 // ---------------------------------------------------------------------------
 template <int MT>
 __device__ __forceinline__ void gather_add(float (&acc)[MT], const float* __restrict__ xt, uint32_t word, float sign)
@@ -102,90 +102,161 @@ __device__ __forceinline__ void gather_add(float (&acc)[MT], const float* __rest
     }
 }
 
-template <int MT, int LPC>
-__global__ __launch_bounds__(256) void tl_spmm_small(KernelArgs a)
+constexpr int kSmallStreamBytes = 32 * 1024;  // LDS for the chunks of one group of tiles
+constexpr int kSmallXBytes = 32 * 1024;       // LDS for the activation rows of one group of tiles
+constexpr int kBlockThreads = 512;            // workgroup of the small-M kernel: 32 lanes for each of its 16 columns
+constexpr int kMaxChunkBytes = (TL_BLOCK_COLUMNS + TL_BLOCK_COLUMNS * 128) * 4;  // a chunk of all-non-zero columns
+
+// Sizes of one group of tiles for a workgroup of NT threads with MT activation rows: what one
+// thread keeps in registers while a group is in flight is bounded (256 bytes of stream and a
+// few 16-byte activation vectors), and the whole group fits the two LDS areas.
+template <int MT, int NT>
+struct BlockShape {
+    static constexpr int kStreamCap = (NT * 256 < kMaxChunkBytes ? kMaxChunkBytes + 240
+                                       : (NT * 256 > kSmallStreamBytes ? kSmallStreamBytes : NT * 256)) / 16 * 16;
+    static constexpr int kVectors = (kStreamCap / 16 + NT - 1) / NT;
+    static constexpr int kByLds = kSmallXBytes / (kTileSlots * MT * 4);
+    static constexpr int kTiles = kByLds < 32 ? kByLds : 32;                         // tiles per group at most
+    // 16-byte activation vectors per row of a group (fp32: 4 values each; +2 for the ragged ends)
+    static constexpr int kRowVectors = (kTiles * kMaxTileRows + 3) / 4 + 2;
+    static constexpr int kXVectors = MT * ((kRowVectors + NT - 1) / NT);             // per thread
+};
+
+// One workgroup owns one block of 16 columns (and MT activation rows) over all of K.
+// K is walked in groups of tiles.  For a group, the chunks are one contiguous piece of the
+// stream; it and the activation rows of the same tiles (contiguous in K) travel
+// global -> registers one group ahead as 16-byte vectors, all in flight before anything
+// waits, then registers -> LDS (activations as fp32 [slot][row]).
+// From LDS, 32 lanes share a column: TP tiles are worked on side by side, LW lanes per run,
+// one dword (four row indices) per lane and pass; an index is one LDS gather and one fp32
+// add per activation row.  The 32 partial sums of a column are folded with cross-lane
+// shuffles.  No workgroup depends on another.
+// X must be row-major with 16-byte aligned rows (the launcher repacks anything else).
+template <int MT, int LW, bool XF16>
+__global__ __launch_bounds__(kBlockThreads) void tl_spmm_block(KernelArgs a)
 {
-    // LDS: activation tiles as fp32 [tiles_per_stage * 256 slots][MT], then the
-    // descriptors of this workgroup's columns for every tile, then the block starts.
-    extern __shared__ __align__(16) float xs[];
-    constexpr int CPB = 256 / LPC;  // columns per workgroup; divides 64, so they share one column block
-    constexpr int TB = 16;          // tiles whose index loads are in flight together
-    uint32_t* dsc = reinterpret_cast<uint32_t*>(xs + (size_t)a.tiles_per_stage * kTileSlots * MT);
-    uint32_t* bst = dsc + (size_t)a.T * CPB;
-
+    extern __shared__ __align__(16) unsigned char lds[];
+    constexpr int NT = kBlockThreads;
+    constexpr int LPC = NT / TL_BLOCK_COLUMNS;  // lanes per column: TP tiles in parallel x LW lanes per run
+    constexpr int TP = LPC / LW;
+    using Shape = BlockShape<MT, NT>;
+    constexpr int NV = Shape::kVectors;    // 16-byte stream vectors per thread and group
+    constexpr int NXV = Shape::kXVectors;  // 16-byte activation vectors per thread and group
+    constexpr int VE = XF16 ? 8 : 4;       // activation values per vector
+    constexpr int XPR = NXV / MT;          // vectors per thread and row
     const int tid = threadIdx.x;
-    const int lig = tid % LPC, col = tid / LPC;
-    const int n_first = blockIdx.x * CPB;
-    const int n = n_first + col;
-    const int m0 = blockIdx.y * MT;
-    const int NP = a.NB * TL_BLOCK_COLUMNS;
-    const uint32_t* __restrict__ idx = a.w0.idx;
+    const int nb = blockIdx.x, m0 = blockIdx.y * MT;
+    const int TG = a.tiles_per_group;  // <= Shape::kTiles, and TG chunks fit Shape::kStreamCap
+    float* xs = reinterpret_cast<float*>(lds);                                   // [TG * 256 slots][MT]
+    uint32_t* buf = reinterpret_cast<uint32_t*>(lds + kSmallXBytes);             // chunk copy
+    uint32_t* cst = reinterpret_cast<uint32_t*>(lds + kSmallXBytes + kSmallStreamBytes);  // chunk starts inside buf
+    const_u32_ptr cs = as_const(a.w0.chunkstart) + (size_t)nb * a.T;
+    const unsigned char* Xb = static_cast<const unsigned char*>(a.X);
+    constexpr int ES = XF16 ? 2 : 4;
 
-    for (int e = tid; e < a.T * CPB; e += 256) dsc[e] = a.w0.desc[(size_t)(e / CPB) * NP + n_first + e % CPB];
-    for (int e = tid; e < a.T; e += 256) bst[e] = a.w0.blockstart[(size_t)e * a.NB + n_first / TL_BLOCK_COLUMNS];
-    __syncthreads();
+    // Slots that staging never writes (rows past the tile height, the sentinel slot) must read as zero.
+    for (int e = tid; e < kSmallXBytes / 16; e += NT) reinterpret_cast<u32x4*>(xs)[e] = u32x4{0u, 0u, 0u, 0u};
 
+    u32x4 cv[NV];
+    u32x4 xv[NXV];
+    // global -> registers for the tiles [t, t + nt)
+    auto prefetch = [&](int t, int nt) {
+        const uint32_t s_lo = cs[t];
+        const int nvec = (int)(cs[t + nt] - s_lo) / 4;
+        const u32x4* src = reinterpret_cast<const u32x4*>(a.w0.stream + s_lo);
+#pragma unroll
+        for (int i = 0; i < NV; ++i) cv[i] = src[min(tid + i * NT, nvec - 1)];  // past the end: last vector again, never stored
+        const int k_lo = t * a.tile_rows, k_hi = min(a.K, (t + nt) * a.tile_rows);
+        const int v_lo = k_lo / VE, v_hi = (k_hi + VE - 1) / VE;  // vectors [v_lo, v_hi) of a row cover the group
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            const int row = min(m0 + m, a.M - 1);  // rows past M re-read the last row; they are never stored to Y
+#pragma unroll
+            for (int i = 0; i < XPR; ++i) {
+                const int v = min(v_lo + tid + i * NT, v_hi - 1);
+                xv[m * XPR + i] = *reinterpret_cast<const u32x4*>(Xb + ((size_t)row * a.ldx + (size_t)v * VE) * ES);
+            }
+        }
+    };
+    // registers -> LDS
+    auto commit = [&](int t, int nt) {
+        const uint32_t s_lo = cs[t];
+        const int nvec = (int)(cs[t + nt] - s_lo) / 4;
+#pragma unroll
+        for (int i = 0; i < NV; ++i)
+            if (tid + i * NT < nvec) reinterpret_cast<u32x4*>(buf)[tid + i * NT] = cv[i];
+        const int k_lo = t * a.tile_rows, k_hi = min(a.K, (t + nt) * a.tile_rows);
+        const int v_lo = k_lo / VE, v_hi = (k_hi + VE - 1) / VE;
+#pragma unroll
+        for (int i = 0; i < XPR; ++i) {
+            const int v = v_lo + tid + i * NT;
+            if (v < v_hi) {
+                int k = v * VE;
+                int tile = (int)(((unsigned long long)(unsigned)k * a.tile_magic) >> 32);  // k / tile_rows
+                int r = k - tile * a.tile_rows;
+#pragma unroll
+                for (int e = 0; e < VE; ++e) {
+                    if (k >= k_lo && k < k_hi) {
+                        float* dst = xs + (size_t)((tile - t) * kTileSlots + r) * MT;
+#pragma unroll
+                        for (int m = 0; m < MT; ++m) {
+                            const uint32_t word = xv[m * XPR + i][XF16 ? e / 2 : e];
+                            dst[m] = XF16 ? __half2float(__ushort_as_half((unsigned short)(e % 2 ? word >> 16 : word & 0xffffu)))
+                                          : __uint_as_float(word);
+                        }
+                    }
+                    ++k;
+                    if (++r == a.tile_rows) { r = 0; ++tile; }
+                }
+            }
+        }
+        if (tid <= nt) cst[tid] = cs[t + tid] - s_lo;
+    };
+
+    const int col = tid / LPC, lig = tid % LPC;
+    const int tp = lig / LW, lw = lig % LW;
     float acc[MT];
 #pragma unroll
     for (int m = 0; m < MT; ++m) acc[m] = 0.f;
 
-    // One dword (four rows) per lane and tile; lanes past the run's end take an
-    // all-sentinel word, i.e. four gathers of the zero slot, so nothing branches.
-    auto fetch = [&](int tb, uint32_t(&w)[TB]) {
+    constexpr int TU = MT <= 2 ? 4 : (MT <= 8 ? 2 : 1);  // tiles of one lane whose LDS reads are issued together
+    prefetch(0, min(TG, a.T));
+    for (int t = 0; t < a.T; t += TG) {
+        const int nt = min(TG, a.T - t);
+        __syncthreads();  // the previous group has been consumed
+        commit(t, nt);
+        __syncthreads();
+        if (t + TG < a.T) prefetch(t + TG, min(TG, a.T - t - TG));
+        for (int tl0 = tp; tl0 < nt; tl0 += TP * TU) {
+            uint32_t d[TU], w[TU];
+            const uint32_t* run[TU];
 #pragma unroll
-        for (int u = 0; u < TB; ++u) {
-            const int t = tb + u;
-            uint32_t word = 0xffffffffu;
-            if (t < a.T) {
-                const uint32_t d = dsc[t * CPB + col];
-                if (lig < run_pos_dwords(d) + run_neg_dwords(d)) word = idx[bst[t] + (d >> 16) + lig];
+            for (int u = 0; u < TU; ++u) {
+                const int tl = tl0 + u * TP;
+                const uint32_t* chunk = buf + cst[min(tl, nt - 1)];
+                d[u] = tl < nt ? chunk[col] : 0u;  // tiles past the group: empty run
+                run[u] = chunk + (d[u] >> 16);
             }
-            w[u] = word;
-        }
-    };
-
-    uint32_t wn[TB];
-    fetch(0, wn);
-    for (int tb = 0; tb < a.T; tb += TB) {
-        uint32_t wc[TB];
 #pragma unroll
-        for (int u = 0; u < TB; ++u) wc[u] = wn[u];
-        if (tb + TB < a.T) fetch(tb + TB, wn);
+            for (int u = 0; u < TU; ++u)  // lanes past the run's end take an all-sentinel word: four gathers of zero
+                w[u] = lw < run_pos_dwords(d[u]) + run_neg_dwords(d[u]) ? run[u][lw] : 0xffffffffu;
 #pragma unroll
-        for (int u = 0; u < TB; ++u) {
-            const int t = tb + u;
-            if (t >= a.T) break;
-            if (t % a.tiles_per_stage == 0) {  // uniform: stage the next group of activation tiles
-                const int slots = min(a.tiles_per_stage, a.T - t) * kTileSlots;
-                __syncthreads();
-                for (int e = tid; e < slots * MT; e += 256) {
-                    const int slot = e % slots, m = e / slots;
-                    const int r = slot & (kTileSlots - 1);
-                    const long long k = (long long)(t + (slot >> 8)) * a.tile_rows + r;
-                    float v = 0.f;
-                    if (r < a.tile_rows && k < a.K && m0 + m < a.M) {
-                        const long long off = a.x_kmajor ? k * a.ldx + (m0 + m) : (long long)(m0 + m) * a.ldx + k;
-                        v = a.x_f16 ? __half2float(static_cast<const __half*>(a.X)[off]) : static_cast<const float*>(a.X)[off];
-                    }
-                    xs[slot * MT + m] = v;
-                }
-                __syncthreads();
+            for (int u = 0; u < TU; ++u) {
+                const int pd = run_pos_dwords(d[u]), tot = pd + run_neg_dwords(d[u]);
+                const float* xt = xs + (size_t)min(tl0 + u * TP, nt - 1) * kTileSlots * MT;
+                gather_add<MT>(acc, xt, w[u], lw < pd ? 1.0f : -1.0f);
+                for (int i = lw + LW; i < tot; i += LW)  // runs longer than the lane group
+                    gather_add<MT>(acc, xt, run[u][i], i < pd ? 1.0f : -1.0f);
             }
-            const uint32_t d = dsc[t * CPB + col];
-            const int pd = run_pos_dwords(d), tot = pd + run_neg_dwords(d);
-            const float* xt = xs + (size_t)(t % a.tiles_per_stage) * kTileSlots * MT;
-            gather_add<MT>(acc, xt, wc[u], lig < pd ? 1.0f : -1.0f);
-            for (int i = lig + LPC; i < tot; i += LPC)  // runs longer than the lane group: rare
-                gather_add<MT>(acc, xt, idx[bst[t] + (d >> 16) + i], i < pd ? 1.0f : -1.0f);
         }
     }
-
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
 #pragma unroll
         for (int off = LPC / 2; off > 0; off >>= 1) acc[m] += __shfl_xor(acc[m], off, 64);
     }
-    if (n < a.N && lig == 0) {
+    const int n = nb * TL_BLOCK_COLUMNS + col;
+    if (lig == 0 && n < a.N) {
         const float s = load_scale(a.w0.scale, a.scale_f16, n);
 #pragma unroll
         for (int m = 0; m < MT; ++m)
@@ -261,15 +332,16 @@ struct WaveRuns {
 };
 
 template <int C>
-__device__ __forceinline__ void fetch_runs(WaveRuns<C>& r, const WeightPtrs& w, int t, int NP, int NB, int n0, int lane)
+__device__ __forceinline__ void fetch_runs(WaveRuns<C>& r, const WeightPtrs& w, int t, int T, int n0, int lane)
 {
-    const_u32_ptr dp = as_const(w.desc) + (size_t)t * NP + n0;
+    const uint32_t chunk = as_const(w.chunkstart)[(size_t)(n0 / TL_BLOCK_COLUMNS) * T + t];
+    const_u32_ptr dp = as_const(w.stream) + chunk + n0 % TL_BLOCK_COLUMNS;
 #pragma unroll
     for (int c = 0; c < C; ++c) r.d[c] = dp[c];
-    r.base = as_const(w.blockstart)[(size_t)t * NB + n0 / TL_BLOCK_COLUMNS] + (r.d[0] >> 16);
+    r.base = chunk + (r.d[0] >> 16);
     // Reads past the wave's piece stay inside the blob (it ends with spare bytes) and are never used.
 #pragma unroll
-    for (int ch = 0; ch < NPRE; ++ch) r.pre[ch] = w.idx[r.base + ch * 64 + lane];
+    for (int ch = 0; ch < NPRE; ++ch) r.pre[ch] = w.stream[r.base + ch * 64 + lane];
 }
 
 template <typename XT, int R>
@@ -358,8 +430,7 @@ __global__ __launch_bounds__(WAVES * 64) void tl_spmm_rows(KernelArgs a)
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int m0 = blockIdx.y * MTILE;
     const int n0 = blockIdx.x * (WAVES * C) + wave * C;
-    const int NP = a.NB * TL_BLOCK_COLUMNS;
-    const bool wave_live = n0 < a.N;                                       // uniform; n0 < NP whenever true
+    const bool wave_live = n0 < a.N;                                       // uniform; then n0 lies inside a stored column block
     const unsigned char* __restrict__ XTr = static_cast<const unsigned char*>(a.X);  // [K][ldx] of XT, m contiguous
 
     float acc[C][R];
@@ -379,8 +450,8 @@ __global__ __launch_bounds__(WAVES * 64) void tl_spmm_rows(KernelArgs a)
     u32x4 pf[PER];
     WaveRuns<C> cur, nxt, cur2, nxt2;
     if (wave_live) {
-        fetch_runs<C>(nxt, a.w0, 0, NP, a.NB, n0, lane);
-        if constexpr (GATED) fetch_runs<C>(nxt2, a.w1, 0, NP, a.NB, n0, lane);
+        fetch_runs<C>(nxt, a.w0, 0, a.T, n0, lane);
+        if constexpr (GATED) fetch_runs<C>(nxt2, a.w1, 0, a.T, n0, lane);
     }
     tile_to_regs<XT, CHUNKS, NT, PER>(pf, XTr, a, 0, m0);
     const XT* tile_lane = tile + lane * R;
@@ -393,11 +464,11 @@ __global__ __launch_bounds__(WAVES * 64) void tl_spmm_rows(KernelArgs a)
             cur = nxt;
             if constexpr (GATED) cur2 = nxt2;
             if (t + 1 < a.T) {
-                fetch_runs<C>(nxt, a.w0, t + 1, NP, a.NB, n0, lane);
-                if constexpr (GATED) fetch_runs<C>(nxt2, a.w1, t + 1, NP, a.NB, n0, lane);
+                fetch_runs<C>(nxt, a.w0, t + 1, a.T, n0, lane);
+                if constexpr (GATED) fetch_runs<C>(nxt2, a.w1, t + 1, a.T, n0, lane);
             }
-            rows_consume<XT, R, C>(acc, cur, a.w0.idx, tile_lane, lane, a.one);
-            if constexpr (GATED) rows_consume<XT, R, C>(acc2, cur2, a.w1.idx, tile_lane, lane, a.one);
+            rows_consume<XT, R, C>(acc, cur, a.w0.stream, tile_lane, lane, a.one);
+            if constexpr (GATED) rows_consume<XT, R, C>(acc2, cur2, a.w1.stream, tile_lane, lane, a.one);
         }
     }
 
@@ -424,9 +495,10 @@ __global__ __launch_bounds__(WAVES * 64) void tl_spmm_rows(KernelArgs a)
 int check_header(const tl_layout_header* h)
 {
     if (!h) return fail(TL_ERR_ARG, "layout header is null");
-    if (h->magic != TL_LAYOUT_MAGIC || h->version != 2) return fail(TL_ERR_FORMAT, "bad layout magic/version");
+    if (h->magic != TL_LAYOUT_MAGIC || h->version != TL_LAYOUT_VERSION) return fail(TL_ERR_FORMAT, "bad layout magic/version");
     if (h->tile_rows == 0 || h->tile_rows > (uint32_t)kMaxTileRows || h->n_tiles != (uint32_t)ceil_div(h->inners, h->tile_rows) ||
-        h->n_blocks != (uint32_t)ceil_div(h->columns, TL_BLOCK_COLUMNS))
+        h->n_blocks != (uint32_t)ceil_div(h->columns, TL_BLOCK_COLUMNS) || h->max_chunk_dwords < TL_BLOCK_COLUMNS ||
+        (int64_t)h->max_chunk_dwords * 4 > kMaxChunkBytes + 16)
         return fail(TL_ERR_FORMAT, "layout header geometry is inconsistent");
     return TL_OK;
 }
@@ -453,46 +525,10 @@ WeightPtrs weight_ptrs(const tl_layout_header* h, const void* blob_dev, const vo
 {
     const unsigned char* b = static_cast<const unsigned char*>(blob_dev);
     WeightPtrs w;
-    w.blockstart = reinterpret_cast<const uint32_t*>(b + h->off_blockstart);
-    w.desc = reinterpret_cast<const uint32_t*>(b + h->off_desc);
-    w.idx = reinterpret_cast<const uint32_t*>(b + h->off_idx);
+    w.chunkstart = reinterpret_cast<const uint32_t*>(b + h->off_chunkstart);
+    w.stream = reinterpret_cast<const uint32_t*>(b + h->off_stream);
     w.scale = scale;
     return w;
-}
-
-template <int MT>
-int launch_small_lpc(const KernelArgs& a, int lpc, hipStream_t st)
-{
-    const size_t lds = (size_t)a.tiles_per_stage * kTileSlots * MT * sizeof(float) + ((size_t)a.T * (256 / lpc) + a.T) * sizeof(uint32_t);
-    dim3 grid((unsigned)ceil_div(a.N, 256 / lpc), (unsigned)ceil_div(a.M, MT));
-    switch (lpc) {
-        case 8: hipLaunchKernelGGL((tl_spmm_small<MT, 8>), grid, dim3(256), lds, st, a); break;
-        case 16: hipLaunchKernelGGL((tl_spmm_small<MT, 16>), grid, dim3(256), lds, st, a); break;
-        case 32: hipLaunchKernelGGL((tl_spmm_small<MT, 32>), grid, dim3(256), lds, st, a); break;
-        default: hipLaunchKernelGGL((tl_spmm_small<MT, 64>), grid, dim3(256), lds, st, a); break;
-    }
-    return TL_OK;
-}
-
-int launch_small(KernelArgs a, const tl_layout_header* h, hipStream_t st)
-{
-    int mt = 1;
-    while (mt < a.M && mt < 32) mt *= 2;
-    const double mean_run = h->mean_run_dwords_x16 / 16.0;
-    int lpc = 8;
-    while (lpc < 64 && lpc < mean_run * 1.1) lpc *= 2;
-    lpc = env_int("TL_LPC", lpc);
-    if (lpc != 8 && lpc != 16 && lpc != 32 && lpc != 64) return fail(TL_ERR_ARG, "TL_LPC=%d (8, 16, 32 or 64 expected)", lpc);
-    const int budget_slots = (48 * 1024) / (int)(mt * sizeof(float));
-    a.tiles_per_stage = (int)std::min<int64_t>(a.T, std::max(1, budget_slots / kTileSlots));
-    switch (mt) {
-        case 1: return launch_small_lpc<1>(a, lpc, st);
-        case 2: return launch_small_lpc<2>(a, lpc, st);
-        case 4: return launch_small_lpc<4>(a, lpc, st);
-        case 8: return launch_small_lpc<8>(a, lpc, st);
-        case 16: return launch_small_lpc<16>(a, lpc, st);
-        default: return launch_small_lpc<32>(a, lpc, st);
-    }
 }
 
 template <typename KernelT>
@@ -501,6 +537,103 @@ int raise_lds_limit(KernelT kernel, size_t bytes)
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
     if (e != hipSuccess) return fail(TL_ERR_LAUNCH, "hipFuncSetAttribute(%zu bytes of LDS): %s", bytes, hipGetErrorString(e));
     return TL_OK;
+}
+
+template <int MT, int LW, bool XF16>
+int launch_block_kernel(KernelArgs a, const tl_layout_header* h, hipStream_t st)
+{
+    using Shape = BlockShape<MT, kBlockThreads>;
+    const int by_stream = (int)(Shape::kStreamCap / ((int64_t)h->max_chunk_dwords * 4));
+    a.tiles_per_group = std::max(1, std::min(std::min(Shape::kTiles, by_stream), 255));
+    a.tile_magic = (unsigned)(((1ull << 32) + h->tile_rows - 1) / h->tile_rows);
+    const size_t lds = kSmallXBytes + kSmallStreamBytes + 1024;
+    auto kernel = tl_spmm_block<MT, LW, XF16>;
+    static bool raised = false;  // per instantiation; a repeated or racing call is harmless
+    if (!raised) {
+        if (int rc = raise_lds_limit(kernel, lds)) return rc;
+        raised = true;
+    }
+    dim3 grid((unsigned)a.NB, (unsigned)ceil_div(a.M, MT));
+    hipLaunchKernelGGL(kernel, grid, dim3(kBlockThreads), lds, st, a);
+    return TL_OK;
+}
+
+template <int MT>
+int launch_small_lpc(const KernelArgs& a, const tl_layout_header* h, int lpc, hipStream_t st)
+{
+    if (a.x_f16) {
+        switch (lpc) {
+            case 8: return launch_block_kernel<MT, 8, true>(a, h, st);
+            case 16: return launch_block_kernel<MT, 16, true>(a, h, st);
+            default: return launch_block_kernel<MT, 32, true>(a, h, st);
+        }
+    }
+    switch (lpc) {
+        case 8: return launch_block_kernel<MT, 8, false>(a, h, st);
+        case 16: return launch_block_kernel<MT, 16, false>(a, h, st);
+        default: return launch_block_kernel<MT, 32, false>(a, h, st);
+    }
+}
+
+// Row-major activations with 16-byte aligned rows are read in place; anything else
+// (K-major, odd leading dimension, odd base address) is first repacked into the workspace.
+inline bool small_needs_repack(const void* X, int x_dtype, int x_layout, int64_t ldx, int64_t K)
+{
+    const int es = x_dtype == TL_F16 ? 2 : 4;
+    // K must be whole vectors too: the kernel reads 16 bytes at a time and must not run past a row's end
+    return x_layout != TL_X_ROW_MAJOR || (ldx * es) % 16 != 0 || (K * es) % 16 != 0 || reinterpret_cast<uintptr_t>(X) % 16 != 0;
+}
+inline int64_t small_repack_bytes(const tl_layout_header* h, int64_t M, int x_dtype)
+{
+    // rows padded to a multiple of 8 values plus one spare vector: the kernel reads whole vectors
+    return M * (round_up(h->inners, 8) + 8) * (x_dtype == TL_F16 ? 2 : 4);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void tl_repack_rows(const T* __restrict__ X, long long ldx, int kmajor, T* __restrict__ out,
+                                                      long long ldo, int M, int K)
+{
+    const long long i = blockIdx.x * 256ll + threadIdx.x;
+    if (i >= (long long)M * ldo) return;
+    const int m = (int)(i / ldo), k = (int)(i % ldo);
+    out[i] = k < K ? (kmajor ? X[(long long)k * ldx + m] : X[(long long)m * ldx + k]) : T(0.0f);
+}
+
+int launch_small(KernelArgs a, const tl_layout_header* h, int x_dtype, void* workspace, int64_t workspace_bytes, hipStream_t st)
+{
+    int mt = 1;
+    while (mt < a.M && mt < 32) mt *= 2;
+    // lanes per run: one dword per lane should cover a typical run in one pass
+    const double mean_run = h->mean_run_dwords_x16 / 16.0;
+    int lpc = 8;
+    while (lpc < 32 && lpc < mean_run) lpc *= 2;
+    lpc = env_int("TL_LPC", lpc);
+    if (lpc != 8 && lpc != 16 && lpc != 32) return fail(TL_ERR_ARG, "TL_LPC=%d (8, 16 or 32 expected)", lpc);
+    if (small_needs_repack(a.X, x_dtype, a.x_kmajor ? TL_X_K_MAJOR : TL_X_ROW_MAJOR, a.ldx, a.K)) {
+        const int64_t need = small_repack_bytes(h, a.M, x_dtype);
+        if (!workspace || workspace_bytes < need)
+            return fail(TL_ERR_SIZE, "workspace has %lld bytes, %lld needed", (long long)workspace_bytes, (long long)need);
+        if (reinterpret_cast<uintptr_t>(workspace) % 16) return fail(TL_ERR_ALIGN, "workspace must be 16-byte aligned");
+        const long long ldo = round_up(a.K, 8) + 8;
+        const unsigned blocks = (unsigned)ceil_div((int64_t)a.M * ldo, 256);
+        if (x_dtype == TL_F16)
+            hipLaunchKernelGGL(tl_repack_rows<__half>, dim3(blocks), dim3(256), 0, st, static_cast<const __half*>(a.X), a.ldx,
+                               a.x_kmajor, static_cast<__half*>(workspace), ldo, a.M, a.K);
+        else
+            hipLaunchKernelGGL(tl_repack_rows<float>, dim3(blocks), dim3(256), 0, st, static_cast<const float*>(a.X), a.ldx,
+                               a.x_kmajor, static_cast<float*>(workspace), ldo, a.M, a.K);
+        a.X = workspace;
+        a.ldx = ldo;
+        a.x_kmajor = 0;
+    }
+    switch (mt) {
+        case 1: return launch_small_lpc<1>(a, h, lpc, st);
+        case 2: return launch_small_lpc<2>(a, h, lpc, st);
+        case 4: return launch_small_lpc<4>(a, h, lpc, st);
+        case 8: return launch_small_lpc<8>(a, h, lpc, st);
+        case 16: return launch_small_lpc<16>(a, h, lpc, st);
+        default: return launch_small_lpc<32>(a, h, lpc, st);
+    }
 }
 
 template <typename XT, int R, bool GATED>
@@ -570,13 +703,15 @@ int check_io(const void* blob_dev, const void* X, void* Y, int x_dtype, int x_la
 
 extern "C" int tl_spmm_workspace(const tl_layout_header* header, int64_t M, int x_dtype, int x_layout, int64_t* workspace_bytes)
 {
-    (void)x_layout;
     if (int rc = check_header(header)) return rc;
     if (int rc = check_dtype(x_dtype, "x")) return rc;
     if (!workspace_bytes) return fail(TL_ERR_ARG, "workspace_bytes is null");
     if (M <= 0) return fail(TL_ERR_SHAPE, "M=%lld must be positive", (long long)M);
     if (M <= kSmallMaxM) {
-        *workspace_bytes = 0;
+        // needed only when the activations have to be repacked (K-major or unaligned rows); whether the
+        // base address is aligned is not known here, so the room is always asked for
+        *workspace_bytes = small_repack_bytes(header, M, x_dtype);
+        (void)x_layout;
         return TL_OK;
     }
     *workspace_bytes = (int64_t)header->inners * round_up(M, rows_mtile(x_dtype)) * (x_dtype == TL_F16 ? 2 : 4);
@@ -601,7 +736,8 @@ extern "C" int tl_spmm(const tl_layout_header* header, const void* blob_dev,
     a.x_f16 = x_dtype == TL_F16; a.x_kmajor = x_layout == TL_X_K_MAJOR; a.y_f16 = y_dtype == TL_F16; a.scale_f16 = scale_dtype == TL_F16;
     a.one = 1.0f;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    int rc = (M <= kSmallMaxM) ? launch_small(a, header, st) : launch_rows(a, x_dtype, workspace, workspace_bytes, false, st);
+    int rc = (M <= kSmallMaxM) ? launch_small(a, header, x_dtype, workspace, workspace_bytes, st)
+                               : launch_rows(a, x_dtype, workspace, workspace_bytes, false, st);
     if (rc) return rc;
     return finish_launch();
 }

@@ -8,8 +8,9 @@
 //     byte value 255 can act as a padding sentinel;
 //   - pads every run to whole dwords so that a lane (or a broadcast word) always
 //     carries four indices;
-//   - orders the stream tile-major, so that the runs a wave needs for one tile --
-//     those of a few neighbouring columns -- are one contiguous piece of memory.
+//   - groups columns in blocks of 16 and stores, block-major, one self-describing chunk per
+//     (block, tile): 16 descriptors followed by the block's runs.  What a workgroup needs
+//     for a range of tiles is then a single contiguous piece of memory.
 #include <cstring>
 #include <vector>
 
@@ -40,24 +41,24 @@ int pick_geometry(int columns, int inners, int tile_rows, Geometry* g)
 }
 
 struct Sections {
-    int64_t off_blockstart, off_desc, off_idx, total;
+    int64_t off_chunkstart, off_stream, total;
 };
 
-Sections place_sections(const Geometry& g, int64_t idx_bytes)
+Sections place_sections(const Geometry& g, int64_t stream_bytes)
 {
     Sections s;
-    s.off_blockstart = 256;
-    s.off_desc = s.off_blockstart + round_up(((int64_t)g.n_tiles * g.n_blocks + 1) * 4, 256);
-    s.off_idx = s.off_desc + round_up((int64_t)g.n_tiles * g.n_blocks * kBlock * 4, 256);
-    // 512 spare bytes behind the indices: kernels fetch whole 64-dword vectors past a run's end.
-    s.total = s.off_idx + round_up(idx_bytes, 256) + 512;
+    s.off_chunkstart = 256;
+    s.off_stream = s.off_chunkstart + round_up(((int64_t)g.n_tiles * g.n_blocks + 1) * 4, 256);
+    // 512 spare bytes behind the stream: kernels fetch whole vectors past a chunk's end.
+    s.total = s.off_stream + round_up(stream_bytes, 256) + 512;
     return s;
 }
 
-int64_t idx_upper_bound(int64_t nnz, int columns, const Geometry& g)
+int64_t stream_upper_bound(int64_t nnz, int columns, const Geometry& g)
 {
-    // every run rounds up by at most 3 bytes; two runs per (column, tile)
-    return round_up(nnz + (int64_t)6 * columns * g.n_tiles, 4);
+    // per (column, tile): two runs that each round up by at most 3 bytes; per chunk:
+    // one descriptor dword per column of the block and up to 12 bytes of padding
+    return round_up(nnz + (int64_t)6 * columns * g.n_tiles + (int64_t)g.n_tiles * g.n_blocks * (kBlock * 4 + 12), 16);
 }
 
 // Per (device tile, column) counts from the tiled-CSC offsets and local rows.
@@ -97,7 +98,7 @@ extern "C" int tl_layout_size(const int32_t* neg_off_tiled, const int32_t* pos_o
     Geometry g;
     if (int rc = pick_geometry(columns, inners, tile_rows, &g)) return rc;
     const int64_t nnz = stream_length(neg_off_tiled, columns, inners, tile_k) + stream_length(pos_off_tiled, columns, inners, tile_k);
-    *blob_bytes = place_sections(g, idx_upper_bound(nnz, columns, g)).total;
+    *blob_bytes = place_sections(g, stream_upper_bound(nnz, columns, g)).total;
     return TL_OK;
 }
 
@@ -121,23 +122,24 @@ extern "C" int tl_layout_build(const int32_t* neg_row, const int32_t* neg_off_ti
     if (int rc = count_device_tiles(pos_row, pos_off_tiled, columns, inners, tile_k, g, &cp)) return rc;
     if (int rc = count_device_tiles(neg_row, neg_off_tiled, columns, inners, tile_k, g, &cn)) return rc;
 
-    const int T = g.n_tiles, NB = g.n_blocks, NP = NB * kBlock;
+    const int T = g.n_tiles, NB = g.n_blocks;
     const int Ta = (int)ceil_div(inners, tile_k);
-    const int64_t reserve = idx_upper_bound(n_pos + n_neg, columns, g);
+    const int64_t reserve = stream_upper_bound(n_pos + n_neg, columns, g);
     const Sections s = place_sections(g, reserve);
     std::memset(blob, 0, (size_t)blob_bytes);
     uint8_t* base = static_cast<uint8_t*>(blob);
-    uint32_t* blockstart = reinterpret_cast<uint32_t*>(base + s.off_blockstart);
-    uint32_t* desc = reinterpret_cast<uint32_t*>(base + s.off_desc);
-    uint8_t* idx = base + s.off_idx;
+    uint32_t* chunkstart = reinterpret_cast<uint32_t*>(base + s.off_chunkstart);
+    uint32_t* stream = reinterpret_cast<uint32_t*>(base + s.off_stream);
 
-    // Pass 1: descriptors and block starts, tile-major.
+    // Pass 1: chunk starts and descriptors, block-major.
     uint64_t dwords = 0, run_sum = 0;
-    uint32_t run_max = 0;
-    for (int t = 0; t < T; ++t)
-        for (int nb = 0; nb < NB; ++nb) {
-            blockstart[(size_t)t * NB + nb] = (uint32_t)dwords;
-            uint32_t in_block = 0;
+    uint32_t run_max = 0, chunk_max = 0;
+    for (int nb = 0; nb < NB; ++nb)
+        for (int t = 0; t < T; ++t) {
+            chunkstart[(size_t)nb * T + t] = (uint32_t)dwords;
+            if (dwords > 0xffffffffull - 16384) return fail(TL_ERR_UNSUPPORTED, "index stream does not fit 32-bit dword offsets");
+            uint32_t* desc = stream + dwords;
+            uint32_t in_chunk = kBlock;  // runs start behind the descriptors
             for (int j = 0; j < kBlock; ++j) {
                 const int y = nb * kBlock + j;
                 uint32_t p = 0, n = 0;
@@ -146,28 +148,37 @@ extern "C" int tl_layout_build(const int32_t* neg_row, const int32_t* neg_off_ti
                     n = cn[(size_t)t * columns + y];
                 }
                 if (p > 255 || n > 255) return fail(TL_ERR_FORMAT, "column %d tile %d holds %u/%u rows of one sign", y, t, p, n);
-                desc[(size_t)t * NP + y] = make_desc(p, n, in_block);
+                if ((dwords + j) * 4 >= (uint64_t)reserve) return fail(TL_ERR_SIZE, "stream reserve exceeded");
+                desc[j] = make_desc(p, n, in_chunk);
                 const uint32_t run = (p + 3) / 4 + (n + 3) / 4;
-                in_block += run;  // at most 64 * 128 dwords: always fits 16 bits
+                in_chunk += run;  // at most 16 + 16 * 128 dwords: always fits 16 bits
                 if (y < columns) {
                     run_sum += run;
                     if (run > run_max) run_max = run;
                 }
             }
-            dwords += in_block;
+            in_chunk = (uint32_t)round_up(in_chunk, 4);
+            if (in_chunk > chunk_max) chunk_max = in_chunk;
+            dwords += in_chunk;
+            if (dwords * 4 > (uint64_t)reserve) return fail(TL_ERR_SIZE, "stream reserve exceeded");
         }
-    blockstart[(size_t)T * NB] = (uint32_t)dwords;
-    if (dwords * 4 > (uint64_t)reserve || dwords > 0xffffffffull)
-        return fail(TL_ERR_UNSUPPORTED, "index stream of %llu dwords does not fit", (unsigned long long)dwords);
-    std::memset(idx, kSentinel, (size_t)dwords * 4);
+    chunkstart[(size_t)NB * T] = (uint32_t)dwords;
 
-    // Pass 2: scatter the rows.  Rows arrive ascending per column, so one cursor per
-    // (device tile, sign) of the current column fills every run in ascending order.
-    std::vector<uint64_t> cursor((size_t)T * 2);
-    for (int y = 0; y < columns; ++y) {
+    // Pass 2: sentinel-fill the runs, then scatter the rows.  Rows arrive ascending per
+    // column, so one cursor per (device tile, sign) of the current column fills every run in order.
+    for (int nb = 0; nb < NB; ++nb)
         for (int t = 0; t < T; ++t) {
-            const uint32_t d = desc[(size_t)t * NP + y];
-            const uint64_t start = ((uint64_t)blockstart[(size_t)t * NB + y / kBlock] + (d >> 16)) * 4;
+            const uint64_t c0 = chunkstart[(size_t)nb * T + t], c1 = chunkstart[(size_t)nb * T + t + 1];
+            std::memset(stream + c0 + kBlock, kSentinel, (size_t)(c1 - c0 - kBlock) * 4);
+        }
+    std::vector<uint64_t> cursor((size_t)T * 2);
+    uint8_t* bytes = reinterpret_cast<uint8_t*>(stream);
+    for (int y = 0; y < columns; ++y) {
+        const int nb = y / kBlock, j = y % kBlock;
+        for (int t = 0; t < T; ++t) {
+            const uint64_t c0 = chunkstart[(size_t)nb * T + t];
+            const uint32_t d = stream[c0 + j];
+            const uint64_t start = (c0 + (d >> 16)) * 4;
             cursor[2 * t] = start;
             cursor[2 * t + 1] = start + (((d & 0xff) + 3) / 4) * 4;
         }
@@ -177,7 +188,7 @@ extern "C" int tl_layout_build(const int32_t* neg_row, const int32_t* neg_off_ti
             for (int t = 0; t < Ta; ++t)
                 for (int32_t i = off[((size_t)y * Ta + t) * 2]; i < off[((size_t)y * Ta + t) * 2 + 1]; ++i) {
                     const int k = t * tile_k + row[i];
-                    idx[cursor[2 * (k / g.tile_rows) + sign]++] = (uint8_t)(k % g.tile_rows);
+                    bytes[cursor[2 * (k / g.tile_rows) + sign]++] = (uint8_t)(k % g.tile_rows);
                 }
         }
     }
@@ -186,18 +197,18 @@ extern "C" int tl_layout_build(const int32_t* neg_row, const int32_t* neg_off_ti
     std::memset(&h, 0, sizeof(h));
     static_assert(sizeof(tl_layout_header) == 256, "header must stay 256 bytes");
     h.magic = TL_LAYOUT_MAGIC;
-    h.version = 2;
+    h.version = TL_LAYOUT_VERSION;
     h.inners = (uint32_t)inners;
     h.columns = (uint32_t)columns;
     h.tile_rows = (uint32_t)g.tile_rows;
     h.n_tiles = (uint32_t)T;
     h.n_blocks = (uint32_t)NB;
+    h.max_chunk_dwords = chunk_max;
     h.nnz_pos = (uint64_t)n_pos;
     h.nnz_neg = (uint64_t)n_neg;
-    h.off_blockstart = (uint64_t)s.off_blockstart;
-    h.off_desc = (uint64_t)s.off_desc;
-    h.off_idx = (uint64_t)s.off_idx;
-    h.idx_bytes = dwords * 4;
+    h.off_chunkstart = (uint64_t)s.off_chunkstart;
+    h.off_stream = (uint64_t)s.off_stream;
+    h.stream_bytes = dwords * 4;
     // The blob handed in is sized by an upper bound; what the format occupies is smaller.
     h.total_bytes = (uint64_t)place_sections(g, (int64_t)dwords * 4).total;
     h.max_run_dwords = run_max;
@@ -240,38 +251,39 @@ extern "C" int tl_layout_validate(const void* blob, int64_t blob_bytes)
     if (blob_bytes < (int64_t)sizeof(tl_layout_header)) return fail(TL_ERR_FORMAT, "blob shorter than its header");
     tl_layout_header h;
     std::memcpy(&h, blob, sizeof(h));
-    if (h.magic != TL_LAYOUT_MAGIC || h.version != 2) return fail(TL_ERR_FORMAT, "bad magic/version %08x/%u", h.magic, h.version);
+    if (h.magic != TL_LAYOUT_MAGIC || h.version != TL_LAYOUT_VERSION) return fail(TL_ERR_FORMAT, "bad magic/version %08x/%u", h.magic, h.version);
     if (h.tile_rows == 0 || h.tile_rows > (uint32_t)kMaxTileRows || h.columns == 0 || h.inners == 0 ||
         h.n_tiles != (uint32_t)ceil_div(h.inners, h.tile_rows) || h.n_blocks != (uint32_t)ceil_div(h.columns, kBlock))
         return fail(TL_ERR_FORMAT, "inconsistent geometry K=%u N=%u rows=%u tiles=%u blocks=%u", h.inners, h.columns,
                     h.tile_rows, h.n_tiles, h.n_blocks);
     Geometry g{(int)h.tile_rows, (int)h.n_tiles, (int)h.n_blocks};
-    const Sections s = place_sections(g, (int64_t)h.idx_bytes);
-    if (h.off_blockstart != (uint64_t)s.off_blockstart || h.off_desc != (uint64_t)s.off_desc || h.off_idx != (uint64_t)s.off_idx ||
-        h.total_bytes != (uint64_t)s.total || h.total_bytes > (uint64_t)blob_bytes || (h.idx_bytes & 3))
+    const Sections s = place_sections(g, (int64_t)h.stream_bytes);
+    if (h.off_chunkstart != (uint64_t)s.off_chunkstart || h.off_stream != (uint64_t)s.off_stream ||
+        h.total_bytes != (uint64_t)s.total || h.total_bytes > (uint64_t)blob_bytes || (h.stream_bytes & 15))
         return fail(TL_ERR_FORMAT, "section table does not match the geometry");
     const uint8_t* base = static_cast<const uint8_t*>(blob);
-    const uint32_t* blockstart = reinterpret_cast<const uint32_t*>(base + h.off_blockstart);
-    const uint32_t* desc = reinterpret_cast<const uint32_t*>(base + h.off_desc);
-    const uint8_t* idx = base + h.off_idx;
-    const uint32_t T = h.n_tiles, NB = h.n_blocks, NP = NB * kBlock;
+    const uint32_t* chunkstart = reinterpret_cast<const uint32_t*>(base + h.off_chunkstart);
+    const uint32_t* stream = reinterpret_cast<const uint32_t*>(base + h.off_stream);
+    const uint32_t T = h.n_tiles, NB = h.n_blocks;
     uint64_t np = 0, nn = 0, expect_start = 0;
-    uint32_t run_max = 0;
-    for (uint32_t t = 0; t < T; ++t) {
-        const uint32_t rows_here = (t + 1 == T) ? h.inners - t * h.tile_rows : h.tile_rows;
-        for (uint32_t nb = 0; nb < NB; ++nb) {
-            if (blockstart[(size_t)t * NB + nb] != expect_start)
-                return fail(TL_ERR_FORMAT, "tile %u block %u: start %u, expected %llu", t, nb, blockstart[(size_t)t * NB + nb],
+    uint32_t run_max = 0, chunk_max = 0;
+    for (uint32_t nb = 0; nb < NB; ++nb)
+        for (uint32_t t = 0; t < T; ++t) {
+            const uint32_t rows_here = (t + 1 == T) ? h.inners - t * h.tile_rows : h.tile_rows;
+            if (chunkstart[(size_t)nb * T + t] != expect_start)
+                return fail(TL_ERR_FORMAT, "block %u tile %u: start %u, expected %llu", nb, t, chunkstart[(size_t)nb * T + t],
                             (unsigned long long)expect_start);
-            uint32_t expect = 0;
+            if ((expect_start + kBlock) * 4 > h.stream_bytes) return fail(TL_ERR_FORMAT, "block %u tile %u: chunk leaves the stream", nb, t);
+            const uint32_t* desc = stream + expect_start;
+            uint32_t expect = kBlock;
             for (uint32_t j = 0; j < (uint32_t)kBlock; ++j) {
                 const uint32_t y = nb * kBlock + j;
-                const uint32_t d = desc[(size_t)t * NP + y], p = d & 0xff, n = (d >> 8) & 0xff, off = d >> 16;
+                const uint32_t d = desc[j], p = d & 0xff, n = (d >> 8) & 0xff, off = d >> 16;
                 if (off != expect) return fail(TL_ERR_FORMAT, "tile %u column %u: run offset %u, expected %u", t, y, off, expect);
                 if (y >= h.columns && (p || n)) return fail(TL_ERR_FORMAT, "tile %u: padding column %u is not empty", t, y);
                 const uint32_t pd = (p + 3) / 4, nd = (n + 3) / 4;
-                if ((expect_start + off + pd + nd) * 4 > h.idx_bytes) return fail(TL_ERR_FORMAT, "tile %u column %u: run leaves the stream", t, y);
-                const uint8_t* run = idx + (expect_start + off) * 4;
+                if ((expect_start + off + pd + nd) * 4 > h.stream_bytes) return fail(TL_ERR_FORMAT, "tile %u column %u: run leaves the stream", t, y);
+                const uint8_t* run = reinterpret_cast<const uint8_t*>(stream + expect_start + off);
                 for (int sign = 0; sign < 2; ++sign) {
                     const uint8_t* r = sign ? run + 4 * pd : run;
                     const uint32_t cnt = sign ? n : p, padded = sign ? 4 * nd : 4 * pd;
@@ -289,12 +301,15 @@ extern "C" int tl_layout_validate(const void* blob, int64_t blob_bytes)
                 expect += pd + nd;
                 if (pd + nd > run_max) run_max = pd + nd;
             }
-            expect_start += expect;
+            const uint32_t padded_chunk = (uint32_t)round_up(expect, 4);
+            for (uint32_t i = expect; i < padded_chunk; ++i)
+                if (stream[expect_start + i] != 0xffffffffu) return fail(TL_ERR_FORMAT, "block %u tile %u: chunk padding is not the sentinel", nb, t);
+            if (padded_chunk > chunk_max) chunk_max = padded_chunk;
+            expect_start += padded_chunk;
         }
-    }
-    if (blockstart[(size_t)T * NB] != expect_start || expect_start * 4 != h.idx_bytes)
-        return fail(TL_ERR_FORMAT, "stream length does not match the block table");
-    if (np != h.nnz_pos || nn != h.nnz_neg || run_max != h.max_run_dwords)
+    if (chunkstart[(size_t)T * NB] != expect_start || expect_start * 4 != h.stream_bytes)
+        return fail(TL_ERR_FORMAT, "stream length does not match the chunk table");
+    if (np != h.nnz_pos || nn != h.nnz_neg || run_max != h.max_run_dwords || chunk_max != h.max_chunk_dwords)
         return fail(TL_ERR_FORMAT, "header totals do not match the streams");
     return TL_OK;
 }
@@ -306,15 +321,14 @@ extern "C" int tl_layout_to_dense(const void* blob, int64_t blob_bytes, int32_t*
     tl_layout_header h;
     std::memcpy(&h, blob, sizeof(h));
     const uint8_t* base = static_cast<const uint8_t*>(blob);
-    const uint32_t* blockstart = reinterpret_cast<const uint32_t*>(base + h.off_blockstart);
-    const uint32_t* desc = reinterpret_cast<const uint32_t*>(base + h.off_desc);
-    const uint8_t* idx = base + h.off_idx;
-    const uint32_t NB = h.n_blocks, NP = NB * kBlock;
+    const uint32_t* chunkstart = reinterpret_cast<const uint32_t*>(base + h.off_chunkstart);
+    const uint32_t* stream = reinterpret_cast<const uint32_t*>(base + h.off_stream);
     std::memset(w_out, 0, sizeof(int32_t) * (size_t)h.inners * h.columns);
-    for (uint32_t t = 0; t < h.n_tiles; ++t)
-        for (uint32_t y = 0; y < h.columns; ++y) {
-            const uint32_t d = desc[(size_t)t * NP + y], p = d & 0xff, n = (d >> 8) & 0xff;
-            const uint8_t* run = idx + ((size_t)blockstart[(size_t)t * NB + y / kBlock] + (d >> 16)) * 4;
+    for (uint32_t y = 0; y < h.columns; ++y)
+        for (uint32_t t = 0; t < h.n_tiles; ++t) {
+            const uint32_t* chunk = stream + chunkstart[(size_t)(y / kBlock) * h.n_tiles + t];
+            const uint32_t d = chunk[y % kBlock], p = d & 0xff, n = (d >> 8) & 0xff;
+            const uint8_t* run = reinterpret_cast<const uint8_t*>(chunk + (d >> 16));
             for (uint32_t i = 0; i < p; ++i) w_out[((size_t)t * h.tile_rows + run[i]) * h.columns + y] = 1;
             run += ((p + 3) / 4) * 4;
             for (uint32_t i = 0; i < n; ++i) w_out[((size_t)t * h.tile_rows + run[i]) * h.columns + y] = -1;

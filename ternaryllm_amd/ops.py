@@ -78,13 +78,22 @@ def _x_geometry(x, K, x_layout):
     return x, M, x.stride(0) if x.shape[0] > 1 else max(x.shape[1], 1)
 
 
+_workspaces = {}
+
+
 def _workspace(header, M, x_code, x_layout, device):
+    """Scratch for one call: one buffer per (device, stream), kept and only replaced by a larger one
+    (work on one stream is ordered, so consecutive calls may share it)."""
     need = ctypes.c_int64(0)
     _lib.check(_lib.lib().tl_spmm_workspace(ctypes.byref(header), M, x_code, x_layout, ctypes.byref(need)))
     if need.value == 0:
         return None, 0
-    ws = torch.empty(need.value, dtype=torch.uint8, device=device)
-    return ws, need.value
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < need.value:
+        ws = torch.empty(max(need.value, 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws, ws.numel()
 
 
 def _scale_args(scale, N, device):
@@ -120,8 +129,6 @@ def spmm(weight, x, scale=None, out_dtype=None, x_layout=_lib.TL_X_ROW_MAJOR, ou
                                 y.data_ptr(), y_code, y.stride(0), scale.data_ptr() if scale is not None else None, s_code,
                                 ws.data_ptr() if ws is not None else None, ws_bytes, _stream_ptr(x.device))
     _lib.check(rc)
-    if ws is not None:
-        ws.record_stream(torch.cuda.current_stream(x.device))
     return y
 
 
@@ -150,8 +157,6 @@ def mlp_gate_up(gate, up, x, gate_scale=None, up_scale=None, out_dtype=None):
                                        us.data_ptr() if us is not None else None, s_code, _lib.TL_ACT_SILU_GATE,
                                        ws.data_ptr() if ws is not None else None, ws_bytes, _stream_ptr(x.device))
     _lib.check(rc)
-    if ws is not None:
-        ws.record_stream(torch.cuda.current_stream(x.device))
     return h
 
 

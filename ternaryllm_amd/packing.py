@@ -151,8 +151,8 @@ class PackedWeight:
         return w
 
     def algorithmic_bytes(self, M, x_bytes, y_bytes, scale_bytes=0):
-        """Bytes one product must move at least once: indices (padded, as stored), descriptors,
-        block table, X, Y and the optional scale."""
+        """Bytes one product must move at least once: the stream as stored (index bytes with their
+        padding and the embedded descriptors), the chunk table, X, Y and the optional scale."""
         h = self.header
-        meta = (h.n_tiles * h.n_blocks + 1) * 4 + h.n_tiles * h.n_blocks * 64 * 4
-        return int(h.idx_bytes + meta + M * h.inners * x_bytes + M * h.columns * y_bytes + h.columns * scale_bytes)
+        table = (h.n_tiles * h.n_blocks + 1) * 4
+        return int(h.stream_bytes + table + M * h.inners * x_bytes + M * h.columns * y_bytes + h.columns * scale_bytes)
