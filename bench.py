@@ -1,0 +1,186 @@
+#!/usr/bin/env python3
+"""Benchmark of the ternary SpMM hot path on one MI355X.
+
+Workload (BASELINE.json, "Llama-2-7B ternary MLP block", the shape the metric is quoted on):
+one step = one ternary SpMM of the gate projection: 8 x 128 = 1024 token rows, fp16 activations
+~N(0,1), W ternary [4096 -> 11008] at 80 % sparsity (10 % +1, 10 % -1, i.i.d., seeded), per-output
+fp16 scale ~U(0.5, 1.5), fp32 accumulation, fp16 output.  Inputs are resident in HBM before the
+timed region.  The value is algorithmic GB/s: bytes every operand must move at least once
+(index stream as stored, chunk table, X, Y, scale) divided by the step time.
+
+Prints ONE JSON line.  Besides the contract fields it carries
+  roofline      HBM roofline of the dominant kernel, timed with HIP events on the kernel's stream
+  cpu_baseline  the reference's CPU SIMD kernel on the same W and X, on this host's cores
+  extra         the other regimes of the path (decode SpMV, small batch, fused MLP block), add-rate
+                figures, and tokens/s
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+VALU_PEAK_GADDS = 39321.6      # 256 CU x 64 lanes x 2.4 GHz fp32 adds/s without packed-fp32 forms
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
+    return ap.parse_args()
+
+
+def weight_and_packed(K, N, sparsity, seed, device):
+    import torch
+    from ternaryllm_amd import ops
+    from ternaryllm_amd.linear import random_ternary_weights
+    from ternaryllm_amd.packing import PackedWeight
+    g = torch.Generator().manual_seed(seed)
+    w = random_ternary_weights((K, N), sparsity, generator=g)
+    pw = PackedWeight.from_dense(w)
+    return w, pw, ops.DeviceWeight(pw, device)
+
+
+def best_k_mean(samples, k):
+    s = sorted(samples)[:k]
+    return sum(s) / len(s)
+
+
+def time_spmm(dw, x, scale, steps, warmup, x_layout=0):
+    """Wall-clock ms per step (synchronise, K steps, synchronise) and event-timed ms per launch."""
+    import torch
+    from ternaryllm_amd import ops
+    for _ in range(warmup):
+        ops.spmm(dw, x, scale, x_layout=x_layout)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        ops.spmm(dw, x, scale, x_layout=x_layout)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    ev_ms, _ = ops.spmm_time(dw, x, steps, scale, x_layout=x_layout)
+    return wall_ms, ev_ms
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only; --gpus %d is not supported" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    import numpy as np
+    import torch
+    from ternaryllm_amd import _lib, ops
+    _lib.lib()  # no fallback: fail now if the HIP library is missing
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+
+    # ---- headline workload -------------------------------------------------
+    M, K, N, sparsity = 1024, 4096, 11008, 0.8
+    w, pw, dw = weight_and_packed(K, N, sparsity, 1237, dev)
+    g = torch.Generator().manual_seed(4242)
+    x = torch.randn((M, K), generator=g).to(torch.float16)
+    scale = (0.5 + torch.rand(N, generator=g)).to(torch.float16)
+    xd, sd = x.to(dev), scale.to(dev)
+    # the kernel's native activation layout ([K][M], M contiguous): the timed launch is then the SpMM kernel alone
+    xk = xd.t().contiguous()
+    wall_ms, ev_ms = time_spmm(dw, xk, sd, args.steps, args.warmup, x_layout=_lib.TL_X_K_MAJOR)
+    wall_rm_ms, ev_rm_ms = time_spmm(dw, xd, sd, args.steps, args.warmup)  # row-major input: adds the re-layout pre-pass
+    y = ops.spmm(dw, xk, sd, x_layout=_lib.TL_X_K_MAJOR)
+    ref = (x.double().numpy() @ w.double().numpy()) * scale.double().numpy()[None, :]
+    err = np.abs(y.float().cpu().numpy() - ref)
+    floor = np.linalg.norm(x.double().numpy(), axis=1, keepdims=True) * np.sqrt(1 - sparsity)
+    max_rel = float(np.max(err / np.maximum(np.abs(ref), floor)))
+    if max_rel > 2e-3:
+        print("bench.py: result differs from the exact product (max rel err %g)" % max_rel, file=sys.stderr)
+        sys.exit(1)
+    B = pw.algorithmic_bytes(M, 2, 2, 2)
+    nnz = pw.nnz
+    gbs = B / (wall_ms * 1e-3) / 1e9
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "spmm_rows_c3_gate_traffic.json")
+    if os.path.exists(tpath):
+        with open(tpath) as f:
+            traffic = json.load(f).get("hbm_bytes_per_launch")
+    out = {
+        "metric": "ternary SpMM GB/s (% HBM peak) + tokens/s, Llama-2-7B ternary MLP shape",
+        "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16 in / f32 accumulate / f16 out", "data": "synthetic",
+        "config": {"workload": "Llama-2-7B ternary MLP gate projection SpMM: M=1024 (8x128 tokens), K=4096, N=11008, "
+                               "80% sparsity, fp16 activations, per-output fp16 scale, u8 tile-local indices",
+                   "M": M, "K": K, "N": N, "sparsity": sparsity, "nnz": int(nnz), "algorithmic_bytes": int(B),
+                   "x_layout": "K-major [K][M]", "max_rel_err": max_rel},
+        "pct_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 3),
+        "tokens_per_s": round(M / (wall_ms * 1e-3), 1),
+        "roofline": {"bound": "hbm", "achieved": round(B / (ev_ms * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(B / (ev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 5), "traffic": traffic,
+                     "kernel": "tl_spmm_rows<__half, 4, 4, 16, false>", "kernel_ms": round(ev_ms, 5)},
+    }
+    extra = {
+        "gadd_per_s": round(M * nnz / (ev_ms * 1e-3) / 1e9, 1),
+        "valu_add_roofline_frac": round(M * nnz / (ev_ms * 1e-3) / 1e9 / VALU_PEAK_GADDS, 4),
+        "gop_equiv_per_s": round(2.0 * M * K * N / (ev_ms * 1e-3) / 1e9, 1),
+        "row_major_input_ms_per_step": round(wall_rm_ms, 5),
+    }
+
+    # ---- CPU baseline on the same W and X ------------------------------------
+    if not args.no_cpu:
+        try:
+            from oracle import cpu_baseline
+            r = cpu_baseline.time_gemm(w.numpy(), x.float().numpy(), runs=10)
+            idx_bytes = 2 * nnz + (N // (16 if r["kind"] == "reference" else 8)) * (34 if r["kind"] == "reference" else 18) * 4
+            Bc = idx_bytes + M * K * 4 + M * N * 4
+            out["cpu_baseline"] = {"value": round(Bc / r["seconds"] / 1e9, 3), "unit": "GB/s", "cores": r["threads"],
+                                   "kind": r["kind"], "sample": "the whole headline SpMM (same W, same X as fp32), mean of 10 runs",
+                                   "kernel": r["kernel"], "ms": round(r["seconds"] * 1e3, 3), "cpu": r["cpu"],
+                                   "tokens_per_s": round(M / r["seconds"], 1), "max_rel_err": r["max_rel_err"]}
+        except Exception as e:  # the baseline is reported, never required
+            out["cpu_baseline"] = {"value": None, "unit": "GB/s", "cores": 0, "kind": "port", "sample": "failed: %s" % e}
+
+    # ---- the other regimes of the path ---------------------------------------
+    if not args.no_extra:
+        def one(name, M2, K2, N2, s2, dt, seed):
+            w2, pw2, dw2 = weight_and_packed(K2, N2, s2, seed, dev)
+            x2 = torch.randn((M2, K2), generator=g).to(dt).to(dev)
+            wms, ems = time_spmm(dw2, x2, None, max(args.steps, 50), args.warmup)
+            B2 = pw2.algorithmic_bytes(M2, x2.element_size(), x2.element_size())
+            extra[name] = {"M": M2, "K": K2, "N": N2, "sparsity": s2, "dtype": str(dt).replace("torch.", ""),
+                           "kernel_ms": round(ems, 5), "GB_per_s": round(B2 / (ems * 1e-3) / 1e9, 1),
+                           "pct_hbm_peak": round(100 * B2 / (ems * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
+                           "tokens_per_s": round(M2 / (ems * 1e-3), 1)}
+        one("c1_spmm_m16_fp32", 16, 4096, 4096, 0.5, torch.float32, 1235)
+        one("c2_decode_spmv_m1_fp16", 1, 4096, 4096, 0.66, torch.float16, 1236)
+        one("decode_spmv_m1_fp16_n11008", 1, 4096, 11008, 0.66, torch.float16, 1239)
+        one("c3_down_m1024_fp16", 1024, 11008, 4096, 0.8, torch.float16, 1240)
+        one("c4_proj_m1024_fp16", 1024, 4096, 4096, 0.9, torch.float16, 1238)
+        # fused MLP block: gate+up+SiLU-gate in one kernel, then down
+        from ternaryllm_amd import TernaryConfig, LlamaTernaryMLP
+        cfg = TernaryConfig(sparsity=0.8)
+        gen = torch.Generator().manual_seed(1241)
+        sc = {k: (0.5 + torch.rand(n, generator=gen)).to(torch.float16) for k, n in (("gate", 11008), ("up", 11008), ("down", 4096))}
+        mlp = LlamaTernaryMLP(cfg, generator=gen, scales=sc, reference_buffers=False).to(dev)
+        xb = xd.reshape(8, 128, K)
+        for _ in range(3):
+            mlp(xb)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(10):
+            mlp(xb)
+        torch.cuda.synchronize()
+        mlp_ms = (time.perf_counter() - t0) * 1e3 / 10
+        extra["c3_mlp_block_fused"] = {"ms": round(mlp_ms, 4), "tokens_per_s": round(M / (mlp_ms * 1e-3), 1)}
+    out["extra"] = extra
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

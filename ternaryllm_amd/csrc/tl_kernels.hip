@@ -510,8 +510,8 @@ int check_dtype(int d, const char* what)
 }
 
 constexpr int kSmallMaxM = 48;       // above this the row-parallel kernel takes over
-constexpr int kRowsWaves = 8;
-constexpr int kRowsCols = 8;
+constexpr int kRowsWaves = 16;
+constexpr int kRowsCols = 4;
 
 inline int rows_mtile(int x_dtype) { return x_dtype == TL_F16 ? 256 : 128; }
 
@@ -652,25 +652,35 @@ int launch_rows_t(const KernelArgs& a, hipStream_t st)
     return TL_OK;
 }
 
-// Runs the re-layout pre-pass into `workspace`, then the row-parallel kernel.
-int launch_rows(KernelArgs a, int x_dtype, void* workspace, int64_t workspace_bytes, bool gated, hipStream_t st)
+// K-major activations whose leading dimension is a whole number of row tiles (and 16-byte aligned)
+// are what the row-parallel kernel reads directly; anything else goes through the re-layout pre-pass.
+inline bool rows_needs_relayout(const void* X, int x_dtype, int x_layout, int64_t ldx, int64_t M)
 {
     const int mtile = rows_mtile(x_dtype);
-    const int64_t ldm = round_up(a.M, mtile);
-    const int64_t need = (int64_t)a.K * ldm * (x_dtype == TL_F16 ? 2 : 4);
-    if (!workspace || workspace_bytes < need)
-        return fail(TL_ERR_SIZE, "workspace has %lld bytes, %lld needed", (long long)workspace_bytes, (long long)need);
-    if (reinterpret_cast<uintptr_t>(workspace) % 16) return fail(TL_ERR_ALIGN, "workspace must be 16-byte aligned");
-    dim3 tgrid((unsigned)ceil_div(a.K, 64), (unsigned)(ldm / 64));
-    if (x_dtype == TL_F16)
-        hipLaunchKernelGGL(tl_relayout_x<__half>, tgrid, dim3(256), 0, st, static_cast<const __half*>(a.X), a.ldx, a.x_kmajor,
-                           static_cast<__half*>(workspace), ldm, a.M, a.K);
-    else
-        hipLaunchKernelGGL(tl_relayout_x<float>, tgrid, dim3(256), 0, st, static_cast<const float*>(a.X), a.ldx, a.x_kmajor,
-                           static_cast<float*>(workspace), ldm, a.M, a.K);
-    a.X = workspace;
-    a.ldx = ldm;
-    a.x_kmajor = 1;
+    return x_layout != TL_X_K_MAJOR || ldx % mtile != 0 || ldx < round_up(M, mtile) || reinterpret_cast<uintptr_t>(X) % 16 != 0;
+}
+
+// Runs the re-layout pre-pass into `workspace` when needed, then the row-parallel kernel.
+int launch_rows(KernelArgs a, int x_dtype, void* workspace, int64_t workspace_bytes, bool gated, hipStream_t st)
+{
+    if (rows_needs_relayout(a.X, x_dtype, a.x_kmajor ? TL_X_K_MAJOR : TL_X_ROW_MAJOR, a.ldx, a.M)) {
+        const int mtile = rows_mtile(x_dtype);
+        const int64_t ldm = round_up(a.M, mtile);
+        const int64_t need = (int64_t)a.K * ldm * (x_dtype == TL_F16 ? 2 : 4);
+        if (!workspace || workspace_bytes < need)
+            return fail(TL_ERR_SIZE, "workspace has %lld bytes, %lld needed", (long long)workspace_bytes, (long long)need);
+        if (reinterpret_cast<uintptr_t>(workspace) % 16) return fail(TL_ERR_ALIGN, "workspace must be 16-byte aligned");
+        dim3 tgrid((unsigned)ceil_div(a.K, 64), (unsigned)(ldm / 64));
+        if (x_dtype == TL_F16)
+            hipLaunchKernelGGL(tl_relayout_x<__half>, tgrid, dim3(256), 0, st, static_cast<const __half*>(a.X), a.ldx, a.x_kmajor,
+                               static_cast<__half*>(workspace), ldm, a.M, a.K);
+        else
+            hipLaunchKernelGGL(tl_relayout_x<float>, tgrid, dim3(256), 0, st, static_cast<const float*>(a.X), a.ldx, a.x_kmajor,
+                               static_cast<float*>(workspace), ldm, a.M, a.K);
+        a.X = workspace;
+        a.ldx = ldm;
+        a.x_kmajor = 1;
+    }
     if (x_dtype == TL_F16) return gated ? launch_rows_t<__half, 4, true>(a, st) : launch_rows_t<__half, 4, false>(a, st);
     return gated ? launch_rows_t<float, 2, true>(a, st) : launch_rows_t<float, 2, false>(a, st);
 }

@@ -160,20 +160,20 @@ def mlp_gate_up(gate, up, x, gate_scale=None, up_scale=None, out_dtype=None):
     return h
 
 
-def spmm_time(weight, x, iters, scale=None, out_dtype=None):
+def spmm_time(weight, x, iters, scale=None, out_dtype=None, x_layout=_lib.TL_X_ROW_MAJOR):
     """Mean milliseconds per tl_spmm call over `iters` back-to-back calls, timed with HIP events
-    recorded on the stream the kernels run on."""
+    recorded on the stream the kernels run on.  Returns (ms, y)."""
     x_code = _code(x.dtype, "x")
-    x, M, ldx = _x_geometry(x, weight.inners, _lib.TL_X_ROW_MAJOR)
+    x, M, ldx = _x_geometry(x, weight.inners, x_layout)
     N = weight.columns
     out_dtype = out_dtype or x.dtype
     y = torch.empty((M, N), dtype=out_dtype, device=x.device)
     scale, s_code = _scale_args(scale, N, x.device)
-    ws, ws_bytes = _workspace(weight.header, M, x_code, _lib.TL_X_ROW_MAJOR, x.device)
+    ws, ws_bytes = _workspace(weight.header, M, x_code, x_layout, x.device)
     ms = ctypes.c_float(0)
     with torch.cuda.device(x.device):
         rc = _lib.lib().tl_spmm_time(ctypes.byref(weight.header), weight.blob.data_ptr(), x.data_ptr(), x_code,
-                                     _lib.TL_X_ROW_MAJOR, ldx, M, y.data_ptr(), _code(out_dtype, "out_dtype"), y.stride(0),
+                                     x_layout, ldx, M, y.data_ptr(), _code(out_dtype, "out_dtype"), y.stride(0),
                                      scale.data_ptr() if scale is not None else None, s_code,
                                      ws.data_ptr() if ws is not None else None, ws_bytes, _stream_ptr(x.device), iters,
                                      ctypes.byref(ms))
