@@ -103,7 +103,7 @@ class TernaryLinear(nn.Module):
             weight = torch.as_tensor(weight).to("cpu", torch.int32).contiguous()
             if tuple(weight.shape) != (in_features, out_features):
                 raise ValueError(f"weight must be [{in_features}, {out_features}]")
-        self.ternary_weight = weight  # kept on the CPU as a plain attribute, as in the reference
+        self._dense = weight  # kept on the CPU, as the reference's `ternary_weight` attribute
         if reference_buffers:
             rows, offs, tiles = convert_ternary_weights(weight, padding=padding, padding_size=padding_size, device=device,
                                                         dtype=torch.int16)
@@ -129,6 +129,29 @@ class TernaryLinear(nn.Module):
         self.uniform = uniform
         self.padding = padding
         self._handle = None
+
+    @property
+    def ternary_weight(self):
+        """The dense int32 [K, N] weight on the CPU (decoded from the packed blob after a state_dict load)."""
+        if self._dense is None:
+            pw = packing.PackedWeight(self.w_packed.detach().cpu().numpy())
+            self._dense = torch.from_numpy(pw.to_dense())
+        return self._dense
+
+    def _load_from_state_dict(self, state_dict, prefix, *args, **kwargs):
+        # a packed weight has its own length: take the incoming blob's size before the generic copy
+        blob = state_dict.get(prefix + "w_packed")
+        if blob is not None:
+            pw = packing.PackedWeight(blob.detach().cpu().numpy())
+            if (pw.inners, pw.columns) != (self.in_features, self.out_features):
+                raise ValueError(f"packed weight is {pw.inners}x{pw.columns}, module is {self.in_features}x{self.out_features}")
+            pw.validate()
+            self.w_packed = torch.empty(blob.shape, dtype=torch.uint8, device=self.w_packed.device)
+            self._header = pw.header
+            self._packed_nnz = pw.nnz
+            self._dense = None
+            self._handle = None
+        super()._load_from_state_dict(state_dict, prefix, *args, **kwargs)
 
     def device_weight(self):
         """The DeviceWeight view of `w_packed` on its current device."""

@@ -81,6 +81,8 @@ def tiled_mcsc_to_dense(merged_row, merged_off, columns, inners, TILE_K):
     if merged_row.dtype not in (np.int16, np.int32):
         raise ValueError("merged_row must be int16 or int32")
     merged_off = np.ascontiguousarray(merged_off, dtype=np.int32)
+    if TILE_K <= 0 or merged_off.size != columns * (-(-inners // TILE_K)) * 4:
+        raise ValueError("merged_off must hold columns * ceil(inners / TILE_K) * 4 entries")
     w = np.zeros((inners, columns), np.int32)
     _lib.check(_lib.lib().tl_tiled_mcsc_to_dense(merged_row.ctypes.data, merged_row.dtype.itemsize, merged_row.size,
                                                   _lib.i32p(merged_off), columns, inners, TILE_K, _lib.i32p(w)))
