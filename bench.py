@@ -34,6 +34,8 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run one plain 256 MiB device copy (reference for scaling rocprof's FETCH_SIZE / WRITE_SIZE)")
     return ap.parse_args()
 
 
@@ -82,6 +84,13 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(2)
     dev = torch.device("cuda:0")
+
+    if args.copy_probe:
+        src = torch.ones(256 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---- headline workload -------------------------------------------------
     M, K, N, sparsity = 1024, 4096, 11008, 0.8

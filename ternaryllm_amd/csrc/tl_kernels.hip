@@ -428,8 +428,17 @@ __global__ __launch_bounds__(WAVES * 64) void tl_spmm_rows(KernelArgs a)
     XT* tile = reinterpret_cast<XT*>(smem);                              // [256 slots][MTILE]
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int m0 = blockIdx.y * MTILE;
-    const int n0 = blockIdx.x * (WAVES * C) + wave * C;
+    // Workgroups are dealt to the 8 XCDs round-robin by linear id, and every XCD has its own L2.
+    // The id is therefore re-read so that XCD x works through one contiguous eighth of the
+    // (row tile, column tile) list, row tile major: the workgroups that share an L2 then share
+    // the same few row tiles of the activations instead of all of them.
+    const int n_col_tiles = (a.N + WAVES * C - 1) / (WAVES * C);
+    const int total = (int)gridDim.x;
+    int id = (int)blockIdx.x;
+    const int per_xcd = total / 8;
+    if (id < per_xcd * 8) id = (id & 7) * per_xcd + (id >> 3);
+    const int m0 = (id / n_col_tiles) * MTILE;
+    const int n0 = (id % n_col_tiles) * (WAVES * C) + wave * C;
     const bool wave_live = n0 < a.N;                                       // uniform; then n0 lies inside a stored column block
     const unsigned char* __restrict__ XTr = static_cast<const unsigned char*>(a.X);  // [K][ldx] of XT, m contiguous
 
@@ -647,7 +656,7 @@ int launch_rows_t(const KernelArgs& a, hipStream_t st)
         if (int rc = raise_lds_limit(kernel, lds)) return rc;
         raised = true;
     }
-    dim3 grid((unsigned)ceil_div(a.N, kRowsWaves * kRowsCols), (unsigned)ceil_div(a.M, MTILE));
+    dim3 grid((unsigned)(ceil_div(a.N, kRowsWaves * kRowsCols) * ceil_div(a.M, MTILE)));  // 1-D: the kernel maps ids to tiles
     hipLaunchKernelGGL(kernel, grid, dim3(kRowsWaves * 64), lds, st, a);
     return TL_OK;
 }
