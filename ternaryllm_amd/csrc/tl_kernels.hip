@@ -296,30 +296,6 @@ __global__ __launch_bounds__(256) void tl_relayout_x(const T* __restrict__ X, lo
 // ---------------------------------------------------------------------------
 // Row-parallel kernel.
 // ---------------------------------------------------------------------------
-template <typename XT, int R>
-struct RowVec;
-template <>
-struct RowVec<__half, 4> {
-    using type = uint2;
-    static __device__ __forceinline__ void add(float (&acc)[4], uint2 v, float sgn_one)
-    {
-        const __half2 lo = *reinterpret_cast<const __half2*>(&v.x), hi = *reinterpret_cast<const __half2*>(&v.y);
-        acc[0] = fmaf(__low2float(lo), sgn_one, acc[0]);
-        acc[1] = fmaf(__high2float(lo), sgn_one, acc[1]);
-        acc[2] = fmaf(__low2float(hi), sgn_one, acc[2]);
-        acc[3] = fmaf(__high2float(hi), sgn_one, acc[3]);
-    }
-};
-template <>
-struct RowVec<float, 2> {
-    using type = float2;
-    static __device__ __forceinline__ void add(float (&acc)[2], float2 v, float sgn_one)
-    {
-        acc[0] = fmaf(v.x, sgn_one, acc[0]);
-        acc[1] = fmaf(v.y, sgn_one, acc[1]);
-    }
-};
-
 // The runs of one wave (C neighbouring columns) for one tile: descriptors, the
 // dword where the wave's piece of the stream starts, and its first NPRE * 64 dwords
 // (one per lane and chunk), fetched one tile ahead of their use.
@@ -344,15 +320,106 @@ __device__ __forceinline__ void fetch_runs(WaveRuns<C>& r, const WeightPtrs& w, 
     for (int ch = 0; ch < NPRE; ++ch) r.pre[ch] = w.stream[r.base + ch * 64 + lane];
 }
 
+// The inner loop of the row-parallel kernel, written out in assembly.
+//
+// A slot of the staged tile is 512 bytes for both activation types (256 fp16 rows / 128 fp32 rows).
+// Its two halves are fetched with LDS "add-TID" reads: address = M0 + offset + 4 * lane, with
+// M0 = slot * 512 set on the scalar unit, so no vector instruction is spent on addressing.  Lane l thus holds, for fp16, rows {2l, 2l+1} and {128+2l, 129+2l} of the row tile;
+// for fp32, rows l and 64+l.  Per dword of four indices: one v_readlane (the dword sits in a lane of
+// the chunk vector), scalar byte extraction, eight LDS reads, and 16 (fp16) or 8 (fp32) accumulating
+// vector ops.  Two register sets alternate so that the reads of dword i + 1 are in flight while
+// dword i is accumulated; LDS reads complete in issue order, so "lgkmcnt(8)" means everything but
+// the eight reads issued last has arrived.
+// The tile starts at LDS address 0 (the kernel has no other LDS; the launcher checks it), so
+// M0 = slot * 512 = the index byte moved to bits 9..16: one shift and one mask per index.  The scalar
+// op that prepares the next index sits between each write of M0 and the reads that use it (one wait
+// state is required there); the last gap is filled by the loop counter's increment.
+#define TL_ISSUE(W, X0, Y0, X1, Y1, X2, Y2, X3, Y3)                 \
+    "s_lshl_b32 %[t], " W ", 9\n\t"                                  \
+    "s_and_b32 m0, %[t], %[mk]\n\t"                                  \
+    "s_lshl_b32 %[t], " W ", 1\n\t"                                  \
+    "ds_read_addtid_b32 " X0 " offset:0\n\t"                         \
+    "ds_read_addtid_b32 " Y0 " offset:256\n\t"                       \
+    "s_and_b32 m0, %[t], %[mk]\n\t"                                  \
+    "s_lshr_b32 %[t], " W ", 7\n\t"                                  \
+    "ds_read_addtid_b32 " X1 " offset:0\n\t"                         \
+    "ds_read_addtid_b32 " Y1 " offset:256\n\t"                       \
+    "s_and_b32 m0, %[t], %[mk]\n\t"                                  \
+    "s_lshr_b32 %[t], " W ", 15\n\t"                                 \
+    "ds_read_addtid_b32 " X2 " offset:0\n\t"                         \
+    "ds_read_addtid_b32 " Y2 " offset:256\n\t"                       \
+    "s_and_b32 m0, %[t], %[mk]\n\t"                                  \
+    "s_add_u32 %[i], %[i], 1\n\t"                                    \
+    "ds_read_addtid_b32 " X3 " offset:0\n\t"                         \
+    "ds_read_addtid_b32 " Y3 " offset:256\n\t"
+
+// fp16: a dword holds two rows; the mixed-precision fma converts and accumulates in one op
+#define TL_FMA_H(X, Y)                                                                   \
+    "v_fma_mix_f32 %[c0], " X ", %[sg], %[c0] op_sel_hi:[1,0,0]\n\t"                      \
+    "v_fma_mix_f32 %[c1], " X ", %[sg], %[c1] op_sel:[1,0,0] op_sel_hi:[1,0,0]\n\t"       \
+    "v_fma_mix_f32 %[c2], " Y ", %[sg], %[c2] op_sel_hi:[1,0,0]\n\t"                      \
+    "v_fma_mix_f32 %[c3], " Y ", %[sg], %[c3] op_sel:[1,0,0] op_sel_hi:[1,0,0]\n\t"
+#define TL_FMA_F(X, Y)                              \
+    "v_fma_f32 %[c0], " X ", %[sg], %[c0]\n\t"       \
+    "v_fma_f32 %[c1], " Y ", %[sg], %[c1]\n\t"
+
+#define TL_SET_A "%[a0]", "%[b0]", "%[a1]", "%[b1]", "%[a2]", "%[b2]", "%[a3]", "%[b3]"
+#define TL_SET_B "%[p0]", "%[q0]", "%[p1]", "%[q1]", "%[p2]", "%[q2]", "%[p3]", "%[q3]"
+#define TL_ISSUE_SET(W, ...) TL_ISSUE(W, __VA_ARGS__)
+#define TL_ACC_A(F) F("%[a0]", "%[b0]") F("%[a1]", "%[b1]") F("%[a2]", "%[b2]") F("%[a3]", "%[b3]")
+#define TL_ACC_B(F) F("%[p0]", "%[q0]") F("%[p1]", "%[q1]") F("%[p2]", "%[q2]") F("%[p3]", "%[q3]")
+
+#define TL_RUN_LOOP(F)                                   \
+    "v_readlane_b32 %[w], %[v], %[i]\n\t"                \
+    TL_ISSUE_SET("%[w]", TL_SET_A)                       \
+    "Ltl_loop%=:\n\t"                                    \
+    "s_cmp_lt_u32 %[i], %[hi]\n\t"                       \
+    "s_cbranch_scc0 Ltl_lastA%=\n\t"                     \
+    "v_readlane_b32 %[w], %[v], %[i]\n\t"                \
+    TL_ISSUE_SET("%[w]", TL_SET_B)                       \
+    "s_waitcnt lgkmcnt(8)\n\t"                           \
+    TL_ACC_A(F)                                          \
+    "s_cmp_lt_u32 %[i], %[hi]\n\t"                       \
+    "s_cbranch_scc0 Ltl_lastB%=\n\t"                     \
+    "v_readlane_b32 %[w], %[v], %[i]\n\t"                \
+    TL_ISSUE_SET("%[w]", TL_SET_A)                       \
+    "s_waitcnt lgkmcnt(8)\n\t"                           \
+    TL_ACC_B(F)                                          \
+    "s_branch Ltl_loop%=\n\t"                            \
+    "Ltl_lastA%=:\n\t"                                   \
+    "s_waitcnt lgkmcnt(0)\n\t"                           \
+    TL_ACC_A(F)                                          \
+    "s_branch Ltl_end%=\n\t"                             \
+    "Ltl_lastB%=:\n\t"                                   \
+    "s_waitcnt lgkmcnt(0)\n\t"                           \
+    TL_ACC_B(F)                                          \
+    "Ltl_end%=:"
+
+// The dwords [lo, hi) of the chunk vector `v` (dword i sits in lane i), all of one column and one
+// sign: acc += sgn * (rows of the tile at each index).  lo < hi.
 template <typename XT, int R>
-__device__ __forceinline__ void rows_add4(float (&acc)[R], const XT* __restrict__ tile_lane, uint32_t word, float sgn_one)
+__device__ __forceinline__ void rows_run(float (&acc)[R], uint32_t v, int lo, int hi, float sgn_one)
 {
-    using V = typename RowVec<XT, R>::type;
-    constexpr int MTILE = 64 * R;
-#pragma unroll
-    for (int b = 0; b < 4; ++b) {
-        const uint32_t r = (word >> (8 * b)) & 0xffu;
-        RowVec<XT, R>::add(acc, *reinterpret_cast<const V*>(tile_lane + r * MTILE), sgn_one);
+    uint32_t a0, b0, a1, b1, a2, b2, a3, b3, p0, q0, p1, q1, p2, q2, p3, q3, w, t;
+    uint32_t i = (uint32_t)lo;
+    if constexpr (sizeof(XT) == 2) {
+        static_assert(R == 4, "fp16 row tiles hold 4 rows per lane");
+        asm volatile(TL_RUN_LOOP(TL_FMA_H)
+                     : [c0] "+v"(acc[0]), [c1] "+v"(acc[1]), [c2] "+v"(acc[2]), [c3] "+v"(acc[3]), [i] "+s"(i),
+                       [a0] "=&v"(a0), [b0] "=&v"(b0), [a1] "=&v"(a1), [b1] "=&v"(b1), [a2] "=&v"(a2), [b2] "=&v"(b2),
+                       [a3] "=&v"(a3), [b3] "=&v"(b3), [p0] "=&v"(p0), [q0] "=&v"(q0), [p1] "=&v"(p1), [q1] "=&v"(q1),
+                       [p2] "=&v"(p2), [q2] "=&v"(q2), [p3] "=&v"(p3), [q3] "=&v"(q3), [w] "=&s"(w), [t] "=&s"(t)
+                     : [v] "v"(v), [hi] "s"((uint32_t)hi), [mk] "s"(0x1fe00u), [sg] "s"(sgn_one)
+                     : "m0", "scc", "memory");
+    } else {
+        static_assert(R == 2, "fp32 row tiles hold 2 rows per lane");
+        asm volatile(TL_RUN_LOOP(TL_FMA_F)
+                     : [c0] "+v"(acc[0]), [c1] "+v"(acc[1]), [i] "+s"(i),
+                       [a0] "=&v"(a0), [b0] "=&v"(b0), [a1] "=&v"(a1), [b1] "=&v"(b1), [a2] "=&v"(a2), [b2] "=&v"(b2),
+                       [a3] "=&v"(a3), [b3] "=&v"(b3), [p0] "=&v"(p0), [q0] "=&v"(q0), [p1] "=&v"(p1), [q1] "=&v"(q1),
+                       [p2] "=&v"(p2), [q2] "=&v"(q2), [p3] "=&v"(p3), [q3] "=&v"(q3), [w] "=&s"(w), [t] "=&s"(t)
+                     : [v] "v"(v), [hi] "s"((uint32_t)hi), [mk] "s"(0x1fe00u), [sg] "s"(sgn_one)
+                     : "m0", "scc", "memory");
     }
 }
 
@@ -360,20 +427,21 @@ __device__ __forceinline__ void rows_add4(float (&acc)[R], const XT* __restrict_
 // and is broadcast from there, so its four row indices are wave-uniform.
 template <typename XT, int R, int C>
 __device__ __forceinline__ void rows_chunk(float (&acc)[C][R], const int (&pb)[C], const int (&pe)[C], const int (&ne)[C],
-                                           uint32_t v, int cb, const XT* __restrict__ tile_lane, float one)
+                                           uint32_t v, int cb, float one)
 {
 #pragma unroll
     for (int c = 0; c < C; ++c) {
-        for (int i = max(pb[c], cb); i < min(pe[c], cb + 64); ++i)
-            rows_add4<XT, R>(acc[c], tile_lane, (uint32_t)__builtin_amdgcn_readlane((int)v, i - cb), one);
-        for (int i = max(pe[c], cb); i < min(ne[c], cb + 64); ++i)
-            rows_add4<XT, R>(acc[c], tile_lane, (uint32_t)__builtin_amdgcn_readlane((int)v, i - cb), -one);
+        int lo = max(pb[c], cb) - cb, hi = min(pe[c], cb + 64) - cb;
+        if (lo < hi) rows_run<XT, R>(acc[c], v, lo, hi, one);
+        lo = max(pe[c], cb) - cb;
+        hi = min(ne[c], cb + 64) - cb;
+        if (lo < hi) rows_run<XT, R>(acc[c], v, lo, hi, -one);
     }
 }
 
 template <typename XT, int R, int C>
 __device__ __forceinline__ void rows_consume(float (&acc)[C][R], const WaveRuns<C>& r, const uint32_t* __restrict__ idx,
-                                             const XT* __restrict__ tile_lane, int lane, float one)
+                                             int lane, float one)
 {
     int pb[C], pe[C], ne[C];
 #pragma unroll
@@ -385,9 +453,9 @@ __device__ __forceinline__ void rows_consume(float (&acc)[C][R], const WaveRuns<
     const int total = ne[C - 1];
 #pragma unroll
     for (int ch = 0; ch < NPRE; ++ch)
-        if (ch * 64 < total) rows_chunk<XT, R, C>(acc, pb, pe, ne, r.pre[ch], ch * 64, tile_lane, one);
+        if (ch * 64 < total) rows_chunk<XT, R, C>(acc, pb, pe, ne, r.pre[ch], ch * 64, one);
     for (int cb = NPRE * 64; cb < total; cb += 64)  // pieces longer than the prefetch window: fetched on demand
-        rows_chunk<XT, R, C>(acc, pb, pe, ne, idx[r.base + cb + lane], cb, tile_lane, one);
+        rows_chunk<XT, R, C>(acc, pb, pe, ne, idx[r.base + cb + lane], cb, one);
 }
 
 // Staging of one activation tile in two halves: global -> registers (issued a tile
@@ -463,7 +531,6 @@ __global__ __launch_bounds__(WAVES * 64) void tl_spmm_rows(KernelArgs a)
         if constexpr (GATED) fetch_runs<C>(nxt2, a.w1, 0, a.T, n0, lane);
     }
     tile_to_regs<XT, CHUNKS, NT, PER>(pf, XTr, a, 0, m0);
-    const XT* tile_lane = tile + lane * R;
     for (int t = 0; t < a.T; ++t) {
         __syncthreads();  // every wave is done with the previous tile
         regs_to_lds<CHUNKS, NT, PER>(pf, smem, a, t);
@@ -476,8 +543,8 @@ __global__ __launch_bounds__(WAVES * 64) void tl_spmm_rows(KernelArgs a)
                 fetch_runs<C>(nxt, a.w0, t + 1, a.T, n0, lane);
                 if constexpr (GATED) fetch_runs<C>(nxt2, a.w1, t + 1, a.T, n0, lane);
             }
-            rows_consume<XT, R, C>(acc, cur, a.w0.stream, tile_lane, lane, a.one);
-            if constexpr (GATED) rows_consume<XT, R, C>(acc2, cur2, a.w1.stream, tile_lane, lane, a.one);
+            rows_consume<XT, R, C>(acc, cur, a.w0.stream, lane, a.one);
+            if constexpr (GATED) rows_consume<XT, R, C>(acc2, cur2, a.w1.stream, lane, a.one);
         }
     }
 
@@ -489,7 +556,8 @@ __global__ __launch_bounds__(WAVES * 64) void tl_spmm_rows(KernelArgs a)
         const float s2 = GATED ? load_scale(a.w1.scale, a.scale_f16, n) : 1.0f;
 #pragma unroll
         for (int j = 0; j < R; ++j) {
-            const int m = m0 + lane * R + j;
+            // rows of a lane: see rows_add4
+            const int m = m0 + (sizeof(XT) == 2 ? (j >> 1) * 128 + 2 * lane + (j & 1) : j * 64 + lane);
             if (m >= a.M) continue;
             float v = acc[c][j] * s;
             if constexpr (GATED) v = silu(v) * (acc2[GATED ? c : 0][j] * s2);
@@ -653,6 +721,10 @@ int launch_rows_t(const KernelArgs& a, hipStream_t st)
     auto kernel = tl_spmm_rows<XT, R, kRowsCols, kRowsWaves, GATED>;
     static bool raised = false;  // per instantiation; a repeated call is harmless
     if (!raised) {
+        // the kernel addresses its activation tile from LDS offset 0: it must own no static LDS
+        hipFuncAttributes attr;
+        if (hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(kernel)) != hipSuccess || attr.sharedSizeBytes != 0)
+            return fail(TL_ERR_LAUNCH, "row kernel was built with static LDS; its tile would not start at offset 0");
         if (int rc = raise_lds_limit(kernel, lds)) return rc;
         raised = true;
     }
