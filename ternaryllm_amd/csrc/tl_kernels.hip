@@ -307,18 +307,68 @@ struct WaveRuns {
     uint32_t pre[NPRE];
 };
 
+// The three dependent reads behind a wave's runs (chunk offset -> descriptors -> index dwords) are
+// spread over three tiles, so that none of them is waited for in the tile that issues it: while tile t
+// is consumed, the index dwords of tile t + 1, the descriptors of tile t + 2 and the chunk offset of
+// tile t + 3 are in flight.
 template <int C>
-__device__ __forceinline__ void fetch_runs(WaveRuns<C>& r, const WeightPtrs& w, int t, int T, int n0, int lane)
-{
-    const uint32_t chunk = as_const(w.chunkstart)[(size_t)(n0 / TL_BLOCK_COLUMNS) * T + t];
-    const_u32_ptr dp = as_const(w.stream) + chunk + n0 % TL_BLOCK_COLUMNS;
+struct RunFetcher {
+    WaveRuns<C> cur, nxt;   // runs of the tile being consumed / of the next one
+    uint32_t d1[C];         // descriptors one tile further on
+    uint32_t chunk1;        // chunk offset that goes with d1
+    uint32_t chunk2;        // chunk offset one tile further still
+    const_u32_ptr chunkstart, stream_c;
+    const uint32_t* stream;
+    int sub, lane;
+
+    __device__ __forceinline__ void descriptors(uint32_t (&d)[C], uint32_t chunk) const
+    {
+        const_u32_ptr dp = stream_c + chunk + sub;
 #pragma unroll
-    for (int c = 0; c < C; ++c) r.d[c] = dp[c];
-    r.base = chunk + (r.d[0] >> 16);
+        for (int c = 0; c < C; ++c) d[c] = dp[c];
+    }
     // Reads past the wave's piece stay inside the blob (it ends with spare bytes) and are never used.
+    __device__ __forceinline__ void indices(WaveRuns<C>& r, uint32_t chunk) const
+    {
+        r.base = chunk + (r.d[0] >> 16);
 #pragma unroll
-    for (int ch = 0; ch < NPRE; ++ch) r.pre[ch] = w.stream[r.base + ch * 64 + lane];
-}
+        for (int ch = 0; ch < NPRE; ++ch) r.pre[ch] = stream[r.base + ch * 64 + lane];
+    }
+    __device__ __forceinline__ void prime(const WeightPtrs& w, int T, int n0, int lane_)
+    {
+        chunkstart = as_const(w.chunkstart) + (size_t)(n0 / TL_BLOCK_COLUMNS) * T;
+        stream_c = as_const(w.stream);
+        stream = w.stream;
+        sub = n0 % TL_BLOCK_COLUMNS;
+        lane = lane_;
+        const uint32_t chunk0 = chunkstart[0];
+        descriptors(nxt.d, chunk0);
+        indices(nxt, chunk0);
+        chunk1 = chunk2 = 0;
+#pragma unroll
+        for (int c = 0; c < C; ++c) d1[c] = 0;
+        if (T > 1) {
+            chunk1 = chunkstart[1];
+            descriptors(d1, chunk1);
+        }
+        if (T > 2) chunk2 = chunkstart[2];
+    }
+    // Call at the start of tile t: afterwards `cur` holds tile t's runs.
+    __device__ __forceinline__ void advance(int t, int T)
+    {
+        cur = nxt;
+        if (t + 1 < T) {
+#pragma unroll
+            for (int c = 0; c < C; ++c) nxt.d[c] = d1[c];
+            indices(nxt, chunk1);
+        }
+        if (t + 2 < T) {
+            descriptors(d1, chunk2);
+            chunk1 = chunk2;
+        }
+        if (t + 3 < T) chunk2 = chunkstart[t + 3];
+    }
+};
 
 // The inner loop of the row-parallel kernel, written out in assembly.
 //
@@ -458,19 +508,28 @@ __device__ __forceinline__ void rows_consume(float (&acc)[C][R], const WaveRuns<
         rows_chunk<XT, R, C>(acc, pb, pe, ne, idx[r.base + cb + lane], cb, one);
 }
 
-// Staging of one activation tile in two halves: global -> registers (issued a tile
-// ahead), registers -> LDS.  A thread owns the same 16-byte chunks in both halves.
+// Staging of one activation tile: global -> registers (issued a tile ahead), registers -> LDS.
+// A thread owns the 16-byte chunks threadIdx.x + i * NT of the tile.  Their byte offsets from the tile's first
+// row are the same for every full tile, so they are computed once (stage_offsets) and a tile's loads
+// take only a wave-uniform base on top; the last tile, when it is shorter, gets offsets of its own.
 template <typename XT, int CHUNKS, int NT, int PER>
-__device__ __forceinline__ void tile_to_regs(u32x4 (&pf)[PER], const unsigned char* __restrict__ XTr, const KernelArgs& a, int t, int m0)
+__device__ __forceinline__ void stage_offsets(uint32_t (&voff)[PER], const KernelArgs& a, int rows)
 {
-    const int n_chunks = min(a.tile_rows, a.K - t * a.tile_rows) * CHUNKS;
+    const int n_chunks = rows * CHUNKS;
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
         // Chunks past the tile's end re-read its last chunk (never stored): the load stays unconditional.
         const int e = min((int)threadIdx.x + i * NT, n_chunks - 1);
         const int r = e / CHUNKS, ch = e % CHUNKS;
-        pf[i] = *reinterpret_cast<const u32x4*>(XTr + ((size_t)(t * a.tile_rows + r) * a.ldx + m0) * sizeof(XT) + ch * 16);
+        voff[i] = (uint32_t)r * (uint32_t)a.ldx * (uint32_t)sizeof(XT) + (uint32_t)ch * 16u;
     }
+}
+
+template <int PER>
+__device__ __forceinline__ void tile_to_regs(u32x4 (&pf)[PER], const unsigned char* __restrict__ tile_base, const uint32_t (&voff)[PER])
+{
+#pragma unroll
+    for (int i = 0; i < PER; ++i) pf[i] = *reinterpret_cast<const u32x4*>(tile_base + voff[i]);
 }
 
 template <int CHUNKS, int NT, int PER>
@@ -525,26 +584,30 @@ __global__ __launch_bounds__(WAVES * 64) void tl_spmm_rows(KernelArgs a)
 
     // The next activation tile travels global -> registers while the current one is consumed.
     u32x4 pf[PER];
-    WaveRuns<C> cur, nxt, cur2, nxt2;
+    RunFetcher<C> f0, f1;
     if (wave_live) {
-        fetch_runs<C>(nxt, a.w0, 0, a.T, n0, lane);
-        if constexpr (GATED) fetch_runs<C>(nxt2, a.w1, 0, a.T, n0, lane);
+        f0.prime(a.w0, a.T, n0, lane);
+        if constexpr (GATED) f1.prime(a.w1, a.T, n0, lane);
     }
-    tile_to_regs<XT, CHUNKS, NT, PER>(pf, XTr, a, 0, m0);
+    uint32_t voff[PER];
+    const int last_rows = a.K - (a.T - 1) * a.tile_rows;
+    const size_t tile_stride = (size_t)a.tile_rows * a.ldx * sizeof(XT);  // bytes between the first rows of two tiles
+    const unsigned char* __restrict__ col0 = XTr + (size_t)m0 * sizeof(XT);
+    stage_offsets<XT, CHUNKS, NT, PER>(voff, a, a.T > 1 ? a.tile_rows : last_rows);
+    tile_to_regs<PER>(pf, col0, voff);
     for (int t = 0; t < a.T; ++t) {
         __syncthreads();  // every wave is done with the previous tile
         regs_to_lds<CHUNKS, NT, PER>(pf, smem, a, t);
         __syncthreads();
-        if (t + 1 < a.T) tile_to_regs<XT, CHUNKS, NT, PER>(pf, XTr, a, t + 1, m0);
+        if (t + 1 < a.T) {
+            if (t + 2 == a.T && last_rows != a.tile_rows) stage_offsets<XT, CHUNKS, NT, PER>(voff, a, last_rows);
+            tile_to_regs<PER>(pf, col0 + (size_t)(t + 1) * tile_stride, voff);
+        }
         if (wave_live) {
-            cur = nxt;
-            if constexpr (GATED) cur2 = nxt2;
-            if (t + 1 < a.T) {
-                fetch_runs<C>(nxt, a.w0, t + 1, a.T, n0, lane);
-                if constexpr (GATED) fetch_runs<C>(nxt2, a.w1, t + 1, a.T, n0, lane);
-            }
-            rows_consume<XT, R, C>(acc, cur, a.w0.stream, lane, a.one);
-            if constexpr (GATED) rows_consume<XT, R, C>(acc2, cur2, a.w1.stream, lane, a.one);
+            f0.advance(t, a.T);
+            if constexpr (GATED) f1.advance(t, a.T);
+            rows_consume<XT, R, C>(acc, f0.cur, a.w0.stream, lane, a.one);
+            if constexpr (GATED) rows_consume<XT, R, C>(acc2, f1.cur, a.w1.stream, lane, a.one);
         }
     }
 
@@ -762,6 +825,9 @@ int launch_rows(KernelArgs a, int x_dtype, void* workspace, int64_t workspace_by
         a.ldx = ldm;
         a.x_kmajor = 1;
     }
+    // the kernel keeps a thread's byte offsets inside one activation tile in 32 bits
+    if ((int64_t)kTileSlots * a.ldx * (x_dtype == TL_F16 ? 2 : 4) >= (int64_t)1 << 32)
+        return fail(TL_ERR_ARG, "activation leading dimension %lld is too large for one call; split the rows", (long long)a.ldx);
     if (x_dtype == TL_F16) return gated ? launch_rows_t<__half, 4, true>(a, st) : launch_rows_t<__half, 4, false>(a, st);
     return gated ? launch_rows_t<float, 2, true>(a, st) : launch_rows_t<float, 2, false>(a, st);
 }
