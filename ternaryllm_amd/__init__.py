@@ -6,6 +6,7 @@ from .config import TernaryConfig
 from .linear import TernaryLinear, random_ternary_weights, convert_ternary_weights, MapKSizeToTileSize
 from .mlp import LlamaTernaryMLP
 from .attention import LlamaTernaryAttention
+from .llama import TernaryLlamaDecoder
 
-__all__ = ["TernaryLinear", "LlamaTernaryMLP", "LlamaTernaryAttention", "TernaryConfig",
+__all__ = ["TernaryLinear", "LlamaTernaryMLP", "LlamaTernaryAttention", "TernaryConfig", "TernaryLlamaDecoder",
            "random_ternary_weights", "convert_ternary_weights", "MapKSizeToTileSize"]

@@ -130,6 +130,35 @@ class TernaryLinear(nn.Module):
         self.padding = padding
         self._handle = None
 
+    @classmethod
+    def from_packed(cls, packed, scale=None, device=None):
+        """A module around an existing PackedWeight: no random draw, no dense copy kept, no bias and
+        none of the reference's merged arrays (`ternary_weight` decodes the blob on demand)."""
+        self = cls.__new__(cls)
+        nn.Module.__init__(self)
+        self.register_parameter("bias", None)
+        empty16 = torch.zeros(0, dtype=torch.int16, device=device)
+        self.register_buffer("w_row_indices", empty16, False)
+        self.register_buffer("w_col_offsets", torch.zeros(0, dtype=torch.int32, device=device), False)
+        self.register_buffer("w_col_tile_indices", empty16.clone(), False)
+        self._dense = None
+        self._header = packed.header
+        self._packed_nnz = packed.nnz
+        self.register_buffer("w_packed", torch.from_numpy(packed.blob).to(device), True)
+        if scale is not None:
+            scale = torch.as_tensor(scale).reshape(-1)
+            if scale.numel() != packed.columns:
+                raise ValueError("scale must have out_features elements")
+            self.register_buffer("w_scale", scale.to(device).contiguous(), True)
+        else:
+            self.w_scale = None
+        self.in_features = packed.inners
+        self.out_features = packed.columns
+        self.uniform = False
+        self.padding = False
+        self._handle = None
+        return self
+
     @property
     def ternary_weight(self):
         """The dense int32 [K, N] weight on the CPU (decoded from the packed blob after a state_dict load)."""

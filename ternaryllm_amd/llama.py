@@ -1,0 +1,264 @@
+"""A minimal Llama-shaped decoder whose linear layers are all ternary: RMSNorm, rotary embedding,
+a preallocated KV cache, causal softmax attention, the SiLU-gated MLP, and a greedy generation loop.
+
+It stands where the reference patches a Hugging Face Llama with its ternary modules
+(ternaryLLM_GPU/TernaryLLM/TernaryLlama.py:69-75) and drives it with `generate`
+(ternaryLLM_GPU/benchmark_ternary_llama.py:81-105); the CPU twin of the same structure is
+ternaryLLM_CPU/src/LlamaModel.hpp:457-527.  Weights are random ternary matrices, drawn as the
+reference draws them; every product runs in libternary_spmm.so.  Normalisation, rotary embedding
+and attention are torch operators.
+
+The decode step has static shapes (the cache has its full length, a mask hides what is not
+written yet, position and token live in device tensors), so it can be captured once in a HIP graph
+and replayed for every generated token.
+"""
+import math
+from concurrent.futures import ThreadPoolExecutor
+
+import numpy as np
+import torch
+from torch import nn
+
+from . import ops, packing
+from .linear import TernaryLinear
+
+
+def _draw_ternary(K, N, sparsity, generator, device):
+    """The reference's i.i.d. rule (TernaryLinear.py:79-83) evaluated on `device`: r < s -> 0,
+    s <= r < (s + 1) / 2 -> -1, else +1.  Returns an int32 [K, N] tensor on the CPU."""
+    r = torch.rand((K, N), generator=generator, device=device)
+    w = (r >= (sparsity + 1) / 2).to(torch.int32) - ((r >= sparsity) & (r < (sparsity + 1) / 2)).to(torch.int32)
+    return w.cpu()
+
+
+class RMSNorm(nn.Module):
+    def __init__(self, size, eps, dtype, device):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(size, dtype=dtype, device=device), requires_grad=False)
+        self.eps = eps
+
+    def forward(self, x):
+        return torch.nn.functional.rms_norm(x, (x.shape[-1],), self.weight, self.eps)
+
+
+class DecoderLayer(nn.Module):
+    """One block.  q, k and v share their input, so their weights are packed side by side as one
+    [hidden, 3 * hidden] matrix and run as one product; gate and up stay two blobs (the fused
+    gate/up/SiLU kernel takes them as a pair)."""
+
+    def __init__(self, config, linears, dtype, device):
+        super().__init__()
+        self.qkv_proj, self.o_proj, self.gate_proj, self.up_proj, self.down_proj = linears
+        self.input_layernorm = RMSNorm(config.hidden_size, config.rms_norm_eps, dtype, device)
+        self.post_attention_layernorm = RMSNorm(config.hidden_size, config.rms_norm_eps, dtype, device)
+
+
+class TernaryLlamaDecoder(nn.Module):
+    """config: TernaryConfig (or any object with its attributes).  `sparsity` of the config applies to
+    every linear layer, the output head included.  Each linear carries a per-output-channel scale
+    1 / sqrt(non-zeros per column) so that activations keep their magnitude through the stack."""
+
+    LINEARS = ("qkv", "o", "gate", "up", "down")
+
+    def __init__(self, config, *, seed=0, device="cuda", dtype=torch.float16, max_seq_len=None, pack_threads=8):
+        super().__init__()
+        if config.num_key_value_heads != config.num_attention_heads:
+            raise ValueError("grouped-query attention is not supported by this decoder")
+        self.config = config
+        self.dtype = dtype
+        self.max_seq_len = int(max_seq_len or config.max_position_embeddings)
+        H, I, V = config.hidden_size, config.intermediate_size, config.vocab_size
+        dev = torch.device(device)
+        gen = torch.Generator(device=dev if dev.type == "cuda" else "cpu")
+        gen.manual_seed(seed)
+        draw_dev = dev if dev.type == "cuda" else "cpu"
+
+        shapes = {"qkv": (H, 3 * H), "o": (H, H), "gate": (H, I), "up": (H, I), "down": (I, H)}
+
+        def make(shape):
+            K, N = shape
+            w = _draw_ternary(K, N, config.sparsity, gen, draw_dev)
+            return w.numpy()
+
+        def pack(w):
+            K, N = w.shape
+            pw = packing.PackedWeight.from_dense(w)
+            nnz_col = np.maximum(np.count_nonzero(w, axis=0), 1)
+            return pw, torch.from_numpy((1.0 / np.sqrt(nnz_col)).astype(np.float16))
+
+        # Draw in layer order (so the seed fixes the model) and pack on worker threads: the packers run
+        # outside the interpreter lock.  Only a few dense matrices are alive at a time.
+        todo = [(li, name) for li in range(config.num_hidden_layers) for name in self.LINEARS] + [(-1, "head")]
+        shapes["head"] = (H, V)
+        done = {}
+        with ThreadPoolExecutor(max_workers=max(1, pack_threads)) as pool:
+            pending = []
+            for key in todo:
+                pending.append((key, pool.submit(pack, make(shapes[key[1]]))))
+                if len(pending) >= 2 * max(1, pack_threads):
+                    k0, job = pending.pop(0)
+                    done[k0] = TernaryLinear.from_packed(*job.result(), device=dev)
+            for k0, job in pending:
+                done[k0] = TernaryLinear.from_packed(*job.result(), device=dev)
+        layers = [DecoderLayer(config, [done[(li, name)] for name in self.LINEARS], dtype, dev)
+                  for li in range(config.num_hidden_layers)]
+        self.lm_head = done[(-1, "head")]
+        self.layers = nn.ModuleList(layers)
+        cpu_gen = torch.Generator().manual_seed(seed + 1)
+        self.embed_tokens = nn.Parameter((0.02 * torch.randn((V, H), generator=cpu_gen)).to(dev, dtype), requires_grad=False)
+        for layer in self.layers:
+            for norm in (layer.input_layernorm, layer.post_attention_layernorm):
+                norm.weight.copy_((1.0 + 0.02 * torch.randn(H, generator=cpu_gen)).to(dev, dtype))
+        self.norm = RMSNorm(H, config.rms_norm_eps, dtype, dev)
+        hd = config.head_dim
+        inv = 1.0 / (config.rope_theta ** (torch.arange(0, hd, 2, dtype=torch.float32) / hd))
+        ang = torch.arange(self.max_seq_len, dtype=torch.float32)[:, None] * inv[None, :]
+        ang = torch.cat([ang, ang], dim=-1)
+        self.register_buffer("rope_cos", ang.cos().to(dev, dtype), False)
+        self.register_buffer("rope_sin", ang.sin().to(dev, dtype), False)
+        self._cache = None
+        self._graph = None
+
+    # -- pieces ------------------------------------------------------------------------------
+    @staticmethod
+    def _rope(x, cos, sin):
+        half = x.shape[-1] // 2
+        rot = torch.cat([-x[..., half:], x[..., :half]], dim=-1)
+        return x * cos + rot * sin
+
+    def _mlp(self, layer, x2):
+        h = ops.mlp_gate_up(layer.gate_proj.device_weight(), layer.up_proj.device_weight(), x2, layer.gate_proj.w_scale,
+                            layer.up_proj.w_scale)
+        return layer.down_proj(h)
+
+    def allocate_cache(self, batch):
+        c = self.config
+        shape = (c.num_hidden_layers, 2, batch, c.num_attention_heads, self.max_seq_len, c.head_dim)
+        self._cache = torch.zeros(shape, dtype=self.dtype, device=self.embed_tokens.device)
+        self._graph = None
+        return self._cache
+
+    def _block(self, layer, li, x, cos, sin, write_pos, attend):
+        """x: [B, S, H]; cos/sin: [S, head_dim]; write_pos: LongTensor [S] of cache slots;
+        attend(q, k_cache, v_cache) -> [B, heads, S, head_dim]."""
+        c = self.config
+        B, S, H = x.shape
+        nh, hd = c.num_attention_heads, c.head_dim
+        h = layer.input_layernorm(x)
+        qkv = layer.qkv_proj(h.reshape(B * S, H)).view(B, S, 3, nh, hd)
+        q = self._rope(qkv[:, :, 0].transpose(1, 2), cos, sin)
+        k = self._rope(qkv[:, :, 1].transpose(1, 2), cos, sin)
+        v = qkv[:, :, 2].transpose(1, 2)
+        kc, vc = self._cache[li, 0], self._cache[li, 1]
+        kc.index_copy_(2, write_pos, k)
+        vc.index_copy_(2, write_pos, v)
+        a = attend(q, kc, vc).transpose(1, 2).reshape(B * S, H)
+        x = x + layer.o_proj(a).view(B, S, H)
+        h = layer.post_attention_layernorm(x)
+        return x + self._mlp(layer, h.reshape(B * S, H)).view(B, S, H)
+
+    # -- prefill -----------------------------------------------------------------------------
+    @torch.no_grad()
+    def prefill(self, tokens):
+        """tokens: LongTensor [B, S].  Fills the cache slots [0, S) and returns the logits of the last
+        position, [B, vocab]."""
+        B, S = tokens.shape
+        if S > self.max_seq_len:
+            raise ValueError("prompt longer than the cache")
+        if self._cache is None or self._cache.shape[2] != B:
+            self.allocate_cache(B)
+        x = self.embed_tokens[tokens]
+        pos = torch.arange(S, device=x.device)
+        cos, sin = self.rope_cos[:S], self.rope_sin[:S]
+
+        def attend(q, kc, vc):
+            return torch.nn.functional.scaled_dot_product_attention(q, kc[:, :, :S], vc[:, :, :S], is_causal=True)
+
+        for li, layer in enumerate(self.layers):
+            x = self._block(layer, li, x, cos, sin, pos, attend)
+        last = self.norm(x[:, -1])
+        return self.lm_head(last)
+
+    # -- decode ------------------------------------------------------------------------------
+    def _decode_step(self, token, pos, mask):
+        """token: LongTensor [B]; pos: LongTensor [1] (cache slot to write); mask: bool [1, 1, 1, max_seq]
+        true on slots <= pos.  Static shapes throughout.  Returns logits [B, vocab]."""
+        x = self.embed_tokens[token][:, None]
+        cos, sin = self.rope_cos.index_select(0, pos), self.rope_sin.index_select(0, pos)
+
+        def attend(q, kc, vc):
+            return torch.nn.functional.scaled_dot_product_attention(q, kc, vc, attn_mask=mask)
+
+        for li, layer in enumerate(self.layers):
+            x = self._block(layer, li, x, cos, sin, pos, attend)
+        return self.lm_head(self.norm(x[:, 0]))
+
+    @torch.no_grad()
+    def generate(self, tokens, new_tokens, use_graph=True):
+        """Greedy decoding: prefill `tokens` [B, S], then `new_tokens` steps.  Returns LongTensor
+        [B, new_tokens].  With use_graph the decode step is captured once and replayed."""
+        B, S = tokens.shape
+        if S + new_tokens > self.max_seq_len:
+            raise ValueError("prompt plus new tokens exceed the cache")
+        dev = self.embed_tokens.device
+        logits = self.prefill(tokens)
+        out = torch.empty((B, new_tokens), dtype=torch.long, device=dev)
+        st = self._decode_state(B)
+        st["token"].copy_(logits.argmax(-1))
+        st["pos"].fill_(S)
+        st["mask"].copy_((torch.arange(self.max_seq_len, device=dev) <= S)[None, None, None])
+        for i in range(new_tokens):
+            out[:, i] = st["token"]
+            if i + 1 == new_tokens:
+                break
+            self.decode_once(st, use_graph)
+        return out
+
+    def _decode_state(self, B):
+        dev = self.embed_tokens.device
+        st = getattr(self, "_state", None)
+        if st is None or st["token"].shape[0] != B:
+            st = {"token": torch.zeros(B, dtype=torch.long, device=dev), "pos": torch.zeros(1, dtype=torch.long, device=dev),
+                  "mask": torch.zeros((1, 1, 1, self.max_seq_len), dtype=torch.bool, device=dev)}
+            self._state = st
+            self._graph = None
+        return st
+
+    def _advance(self, st):
+        logits = self._decode_step(st["token"], st["pos"], st["mask"])
+        st["token"].copy_(logits.argmax(-1))
+        st["pos"].add_(1)
+        st["mask"].index_fill_(3, st["pos"], True)
+
+    @torch.no_grad()
+    def decode_once(self, st, use_graph=True):
+        """One greedy step on the state tensors (token, pos, mask), in place."""
+        if not use_graph:
+            self._advance(st)
+            return
+        if self._graph is None:
+            # warm-up on a side stream (first calls set kernel attributes and grow workspaces), with the
+            # state restored afterwards; then capture
+            keep = {k: v.clone() for k, v in st.items()}
+            cache_keep = None
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                for _ in range(2):
+                    for k, v in keep.items():
+                        st[k].copy_(v)
+                    self._advance(st)
+            torch.cuda.current_stream().wait_stream(side)
+            for k, v in keep.items():
+                st[k].copy_(v)
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                self._advance(st)
+            for k, v in keep.items():
+                st[k].copy_(v)
+            self._graph = g
+            del cache_keep
+        self._graph.replay()
+
+
+__all__ = ["TernaryLlamaDecoder", "RMSNorm", "DecoderLayer"]
