@@ -22,6 +22,7 @@
 
 #include <cstdlib>
 #include <cstring>
+#include <type_traits>
 
 #include "tl_common.h"
 
@@ -52,7 +53,12 @@ struct KernelArgs {
     int M, N, K, T, tile_rows, NB;
     int x_f16, x_kmajor, y_f16, scale_f16;
     int tiles_per_group;  // small-M kernel: activation tiles staged per pass
+    int block_set;        // small-M kernel: column blocks per workgroup (1, 2 or 4)
+    int lpc_shift, lw_shift;  // small-M kernel: log2 of lanes per column and of lanes per run
+    int xs_bytes, buf_bytes;  // small-M kernel: LDS for the staged activations / for the chunk copies
+    int x_mode;           // small-M kernel: how activations are staged (kStageElements / kStageSlotVectors / kStageRowVectors)
     unsigned tile_magic;  // ceil(2^32 / tile_rows): k / tile_rows == (k * tile_magic) >> 32 for every k < 2^24
+    long long x_sm, x_sk; // small-M kernel: element strides of the activations along M and along K
     float one;  // 1.0f, passed in so that the fp16 -> fp32 accumulate stays a single mixed-precision fma
 };
 
@@ -74,147 +80,288 @@ __device__ __forceinline__ int run_pos_dwords(uint32_t d) { return (int)(((d & 0
 __device__ __forceinline__ int run_neg_dwords(uint32_t d) { return (int)((((d >> 8) & 0xffu) + 3u) >> 2); }
 
 // ---------------------------------------------------------------------------
-// Small-M kernel: one workgroup per (column block, range of tiles, block of rows).
+// Small-M kernel: one workgroup per (set of column blocks, block of MT rows).
 // ---------------------------------------------------------------------------
-template <int MT>
-__device__ __forceinline__ void gather_add(float (&acc)[MT], const float* __restrict__ xt, uint32_t word, float sign)
+// acc[m] += sign * x[slot][m] for the four slots named by the bytes of `word`.  `xt` is the staged
+// tile, [slot][MT] in the activations' own type; a slot's MT values are fetched with the widest
+// LDS reads that fit, fp16 values are widened inside the accumulating fma.
+template <int MT, typename XT>
+__device__ __forceinline__ void gather_add(float (&acc)[MT], const XT* __restrict__ xt, uint32_t word, float sign)
 {
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
         const uint32_t r = (word >> (8 * b)) & 0xffu;
-        const float* row = xt + r * MT;
-        if constexpr (MT % 4 == 0) {
+        const XT* row = xt + r * MT;
+        if constexpr (sizeof(XT) == 4) {
+            if constexpr (MT % 4 == 0) {
 #pragma unroll
-            for (int m = 0; m < MT; m += 4) {
-                const float4 v = *reinterpret_cast<const float4*>(row + m);
-                acc[m + 0] = fmaf(v.x, sign, acc[m + 0]);
-                acc[m + 1] = fmaf(v.y, sign, acc[m + 1]);
-                acc[m + 2] = fmaf(v.z, sign, acc[m + 2]);
-                acc[m + 3] = fmaf(v.w, sign, acc[m + 3]);
+                for (int m = 0; m < MT; m += 4) {
+                    const float4 v = *reinterpret_cast<const float4*>(row + m);
+                    acc[m + 0] = fmaf(v.x, sign, acc[m + 0]);
+                    acc[m + 1] = fmaf(v.y, sign, acc[m + 1]);
+                    acc[m + 2] = fmaf(v.z, sign, acc[m + 2]);
+                    acc[m + 3] = fmaf(v.w, sign, acc[m + 3]);
+                }
+            } else if constexpr (MT == 2) {
+                const float2 v = *reinterpret_cast<const float2*>(row);
+                acc[0] = fmaf(v.x, sign, acc[0]);
+                acc[1] = fmaf(v.y, sign, acc[1]);
+            } else {
+                acc[0] = fmaf(row[0], sign, acc[0]);
             }
-        } else if constexpr (MT == 2) {
-            const float2 v = *reinterpret_cast<const float2*>(row);
-            acc[0] = fmaf(v.x, sign, acc[0]);
-            acc[1] = fmaf(v.y, sign, acc[1]);
         } else {
-            acc[0] = fmaf(row[0], sign, acc[0]);
+            if constexpr (MT >= 8) {
+#pragma unroll
+                for (int m = 0; m < MT; m += 8) {
+                    const u32x4 v = *reinterpret_cast<const u32x4*>(row + m);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        acc[m + 2 * j] = fmaf(__half2float(__ushort_as_half((unsigned short)(v[j] & 0xffffu))), sign, acc[m + 2 * j]);
+                        acc[m + 2 * j + 1] = fmaf(__half2float(__ushort_as_half((unsigned short)(v[j] >> 16))), sign, acc[m + 2 * j + 1]);
+                    }
+                }
+            } else if constexpr (MT == 4) {
+                const uint2 v = *reinterpret_cast<const uint2*>(row);
+                acc[0] = fmaf(__half2float(__ushort_as_half((unsigned short)(v.x & 0xffffu))), sign, acc[0]);
+                acc[1] = fmaf(__half2float(__ushort_as_half((unsigned short)(v.x >> 16))), sign, acc[1]);
+                acc[2] = fmaf(__half2float(__ushort_as_half((unsigned short)(v.y & 0xffffu))), sign, acc[2]);
+                acc[3] = fmaf(__half2float(__ushort_as_half((unsigned short)(v.y >> 16))), sign, acc[3]);
+            } else if constexpr (MT == 2) {
+                const uint32_t v = *reinterpret_cast<const uint32_t*>(row);
+                acc[0] = fmaf(__half2float(__ushort_as_half((unsigned short)(v & 0xffffu))), sign, acc[0]);
+                acc[1] = fmaf(__half2float(__ushort_as_half((unsigned short)(v >> 16))), sign, acc[1]);
+            } else {
+                acc[0] = fmaf(__half2float(row[0]), sign, acc[0]);
+            }
         }
     }
 }
 
+constexpr int kBlockThreads = 512;            // workgroup of the small-M kernel
+// Staging of the activations by the small-M kernel:
+constexpr int kStageElements = 0;     // a thread owns slots and reads their MT values one by one (any layout)
+constexpr int kStageSlotVectors = 1;  // K-major, aligned: a thread owns slots and reads each as 16-byte vectors
+constexpr int kStageRowVectors = 2;   // row-major, aligned, MT <= 4: a thread owns 16-byte pieces of the rows
+constexpr int kMaxBlockSet = 4;               // column blocks one workgroup may own
 constexpr int kSmallStreamBytes = 32 * 1024;  // LDS for the chunks of one group of tiles
-constexpr int kSmallXBytes = 32 * 1024;       // LDS for the activation rows of one group of tiles
-constexpr int kBlockThreads = 512;            // workgroup of the small-M kernel: 32 lanes for each of its 16 columns
 constexpr int kMaxChunkBytes = (TL_BLOCK_COLUMNS + TL_BLOCK_COLUMNS * 128) * 4;  // a chunk of all-non-zero columns
 
-// Sizes of one group of tiles for a workgroup of NT threads with MT activation rows: what one
-// thread keeps in registers while a group is in flight is bounded (256 bytes of stream and a
-// few 16-byte activation vectors), and the whole group fits the two LDS areas.
-template <int MT, int NT>
+// What one thread keeps in registers while a group of tiles is in flight: kVectors 16-byte pieces of
+// the stream and, for kSlots slots of the staged tiles, kSlotRegs dwords of activations each.
+// Slots of 8 rows and more are only ever staged as whole vectors (MT * ES / 4 dwords), narrower ones
+// also element by element (one dword per value).
+template <int MT, int ES, int NT>
 struct BlockShape {
     static constexpr int kStreamCap = (NT * 256 < kMaxChunkBytes ? kMaxChunkBytes + 240
                                        : (NT * 256 > kSmallStreamBytes ? kSmallStreamBytes : NT * 256)) / 16 * 16;
     static constexpr int kVectors = (kStreamCap / 16 + NT - 1) / NT;
-    static constexpr int kByLds = kSmallXBytes / (kTileSlots * MT * 4);
-    static constexpr int kTiles = kByLds < 32 ? kByLds : 32;                         // tiles per group at most
-    // 16-byte activation vectors per row of a group (fp32: 4 values each; +2 for the ragged ends)
-    static constexpr int kRowVectors = (kTiles * kMaxTileRows + 3) / 4 + 2;
-    static constexpr int kXVectors = MT * ((kRowVectors + NT - 1) / NT);             // per thread
+    static constexpr int kSlotRegs = MT >= 8 ? MT * ES / 4 : MT;
+    static constexpr int kSlots = 72 / kSlotRegs > 16 ? 16 : 72 / kSlotRegs;  // per thread
+    static constexpr int kTiles = kSlots * NT / kTileSlots;                   // tiles per group at most
 };
 
-// One workgroup owns one block of 16 columns (and MT activation rows) over all of K.
-// K is walked in groups of tiles.  For a group, the chunks are one contiguous piece of the
-// stream; it and the activation rows of the same tiles (contiguous in K) travel
-// global -> registers one group ahead as 16-byte vectors, all in flight before anything
-// waits, then registers -> LDS (activations as fp32 [slot][row]).
-// From LDS, 32 lanes share a column: TP tiles are worked on side by side, LW lanes per run,
-// one dword (four row indices) per lane and pass; an index is one LDS gather and one fp32
-// add per activation row.  The 32 partial sums of a column are folded with cross-lane
-// shuffles.  No workgroup depends on another.
-// X must be row-major with 16-byte aligned rows (the launcher repacks anything else).
-template <int MT, int LW, bool XF16>
+// A workgroup owns BS neighbouring blocks of 16 columns and MT activation rows over all of K.
+// K is walked in groups of tiles.  For a group, the chunks of each block are one contiguous piece
+// of the stream: the pieces travel global -> registers as 16-byte vectors one group ahead, all in
+// flight before anything waits, then registers -> LDS.  The activation rows of the same tiles are
+// staged by slot: a thread owns slots of the [tile][slot][MT] LDS image, reads the slot's MT values
+// (strided element reads from row-major activations, whole vectors from K-major ones), and
+// writes them side by side, so that the gather of an index is one contiguous LDS read of MT values.
+// Slots past a tile's height, the sentinel slot among them, are written as zeros.
+// From LDS, LPC = 32 / BS lanes share a column: TP tiles are worked on side by side, LW lanes per run,
+// one dword (four row indices) per lane and pass; an index is one LDS read and MT accumulating
+// ops.  The LPC partial sums of a column are folded with cross-lane shuffles.  No workgroup depends
+// on another.
+template <int MT, bool XF16>
 __global__ __launch_bounds__(kBlockThreads) void tl_spmm_block(KernelArgs a)
 {
     extern __shared__ __align__(16) unsigned char lds[];
+    using XT = typename std::conditional<XF16, __half, float>::type;
     constexpr int NT = kBlockThreads;
-    constexpr int LPC = NT / TL_BLOCK_COLUMNS;  // lanes per column: TP tiles in parallel x LW lanes per run
-    constexpr int TP = LPC / LW;
-    using Shape = BlockShape<MT, NT>;
-    constexpr int NV = Shape::kVectors;    // 16-byte stream vectors per thread and group
-    constexpr int NXV = Shape::kXVectors;  // 16-byte activation vectors per thread and group
-    constexpr int VE = XF16 ? 8 : 4;       // activation values per vector
-    constexpr int XPR = NXV / MT;          // vectors per thread and row
+    constexpr int ES = (int)sizeof(XT);
+    using Shape = BlockShape<MT, ES, NT>;
+    constexpr int NV = Shape::kVectors;  // 16-byte stream vectors per thread and group
+    constexpr int SPT = Shape::kSlots;   // staged slots per thread and group
+    constexpr int RPS = Shape::kSlotRegs;
+    constexpr int VPS = MT * ES / 16;    // 16-byte vectors per slot (0: slots are never read as vectors)
+    constexpr int VE = 16 / ES;          // activation values per 16-byte vector
+    // row-vector staging: vectors per thread and row that cover a group of Shape::kTiles tiles (+2 for the ragged ends)
+    constexpr int XPR = ((Shape::kTiles * kMaxTileRows + VE - 1) / VE + 2 + NT - 1) / NT;
+    static_assert(MT > 4 || MT * XPR * 4 <= SPT * RPS, "row vectors must fit the staging registers");
     const int tid = threadIdx.x;
-    const int nb = blockIdx.x, m0 = blockIdx.y * MT;
-    const int TG = a.tiles_per_group;  // <= Shape::kTiles, and TG chunks fit Shape::kStreamCap
-    float* xs = reinterpret_cast<float*>(lds);                                   // [TG * 256 slots][MT]
-    uint32_t* buf = reinterpret_cast<uint32_t*>(lds + kSmallXBytes);             // chunk copy
-    uint32_t* cst = reinterpret_cast<uint32_t*>(lds + kSmallXBytes + kSmallStreamBytes);  // chunk starts inside buf
-    const_u32_ptr cs = as_const(a.w0.chunkstart) + (size_t)nb * a.T;
+    const int BS = a.block_set, TG = a.tiles_per_group;
+    const int nb0 = blockIdx.x * BS, m0 = blockIdx.y * MT;
+    const int bs = min(BS, a.NB - nb0);  // blocks this workgroup really has
+    XT* xs = reinterpret_cast<XT*>(lds);                                           // [TG][256 slots][MT]
+    uint32_t* buf = reinterpret_cast<uint32_t*>(lds + a.xs_bytes);                 // chunk copies, block after block
+    uint32_t* cst = reinterpret_cast<uint32_t*>(lds + a.xs_bytes + a.buf_bytes);   // [BS][TG + 1] chunk starts inside buf
+    const_u32_ptr cs = as_const(a.w0.chunkstart) + (size_t)nb0 * a.T;
     const unsigned char* Xb = static_cast<const unsigned char*>(a.X);
-    constexpr int ES = XF16 ? 2 : 4;
-
-    // Slots that staging never writes (rows past the tile height, the sentinel slot) must read as zero.
-    for (int e = tid; e < kSmallXBytes / 16; e += NT) reinterpret_cast<u32x4*>(xs)[e] = u32x4{0u, 0u, 0u, 0u};
 
     u32x4 cv[NV];
-    u32x4 xv[NXV];
+    uint32_t xr[SPT][RPS];  // raw bits: one value per entry (element staging) or whole vectors
     // global -> registers for the tiles [t, t + nt)
     auto prefetch = [&](int t, int nt) {
-        const uint32_t s_lo = cs[t];
-        const int nvec = (int)(cs[t + nt] - s_lo) / 4;
-        const u32x4* src = reinterpret_cast<const u32x4*>(a.w0.stream + s_lo);
+        uint32_t lo[kMaxBlockSet], pre[kMaxBlockSet + 1];
+        pre[0] = 0;
 #pragma unroll
-        for (int i = 0; i < NV; ++i) cv[i] = src[min(tid + i * NT, nvec - 1)];  // past the end: last vector again, never stored
-        const int k_lo = t * a.tile_rows, k_hi = min(a.K, (t + nt) * a.tile_rows);
-        const int v_lo = k_lo / VE, v_hi = (k_hi + VE - 1) / VE;  // vectors [v_lo, v_hi) of a row cover the group
+        for (int j = 0; j < kMaxBlockSet; ++j) {
+            const bool live = j < bs;
+            lo[j] = live ? cs[(size_t)j * a.T + t] : 0u;
+            pre[j + 1] = pre[j] + (live ? (cs[(size_t)j * a.T + t + nt] - lo[j]) / 4 : 0u);
+        }
 #pragma unroll
-        for (int m = 0; m < MT; ++m) {
-            const int row = min(m0 + m, a.M - 1);  // rows past M re-read the last row; they are never stored to Y
+        for (int i = 0; i < NV; ++i) {
+            const uint32_t g = min((uint32_t)(tid + i * NT), pre[kMaxBlockSet] - 1);  // past the end: last vector again, never stored
+            uint32_t base = lo[0], first = 0;
 #pragma unroll
-            for (int i = 0; i < XPR; ++i) {
-                const int v = min(v_lo + tid + i * NT, v_hi - 1);
-                xv[m * XPR + i] = *reinterpret_cast<const u32x4*>(Xb + ((size_t)row * a.ldx + (size_t)v * VE) * ES);
+            for (int j = 1; j < kMaxBlockSet; ++j)
+                if (g >= pre[j]) { base = lo[j]; first = pre[j]; }
+            cv[i] = *reinterpret_cast<const u32x4*>(a.w0.stream + base + (size_t)(g - first) * 4);
+        }
+        if constexpr (MT <= 4) {
+            if (a.x_mode == kStageRowVectors) {
+                // vectors [v_lo, v_hi) of a row cover the group's k range
+                const int k_lo = t * a.tile_rows, k_hi = min(a.K, (t + nt) * a.tile_rows);
+                const int v_lo = k_lo / VE, v_hi = (k_hi + VE - 1) / VE;
+#pragma unroll
+                for (int m = 0; m < MT; ++m) {
+                    const int row = min(m0 + m, a.M - 1);  // rows past M re-read the last row; they are never stored to Y
+#pragma unroll
+                    for (int i = 0; i < XPR; ++i) {
+                        const int v = min(v_lo + tid + i * NT, v_hi - 1);
+                        const u32x4 q = *reinterpret_cast<const u32x4*>(Xb + ((size_t)row * a.ldx + (size_t)v * VE) * ES);
+                        const int f = (m * XPR + i) * 4;
+                        xr[f / RPS][f % RPS] = q[0]; xr[(f + 1) / RPS][(f + 1) % RPS] = q[1];
+                        xr[(f + 2) / RPS][(f + 2) % RPS] = q[2]; xr[(f + 3) / RPS][(f + 3) % RPS] = q[3];
+                    }
+                }
+                return;
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < SPT; ++s) {
+            const int e = tid + s * NT;  // slot of the group's LDS image
+            const int tile = e >> 8, r = e & 255;
+            // slots that hold no row re-read a valid element; they are stored as zeros
+            const int k = min((t + min(tile, nt - 1)) * a.tile_rows + min(r, a.tile_rows - 1), a.K - 1);
+            if (MT >= 8 || a.x_mode == kStageSlotVectors) {
+                if constexpr (VPS > 0) {
+                    const unsigned char* src = Xb + ((size_t)k * a.ldx + m0) * ES;
+#pragma unroll
+                    for (int v = 0; v < VPS; ++v) {
+                        const u32x4 q = *reinterpret_cast<const u32x4*>(src + v * 16);
+                        xr[s][4 * v + 0] = q[0]; xr[s][4 * v + 1] = q[1]; xr[s][4 * v + 2] = q[2]; xr[s][4 * v + 3] = q[3];
+                    }
+                }
+            } else if constexpr (MT <= 4) {
+                const unsigned char* src = Xb + (size_t)k * a.x_sk * ES;
+#pragma unroll
+                for (int m = 0; m < MT; ++m) {
+                    const unsigned char* p = src + (size_t)min(m0 + m, a.M - 1) * a.x_sm * ES;  // rows past M re-read the last row
+                    if constexpr (XF16) xr[s][m] = *reinterpret_cast<const unsigned short*>(p);
+                    else xr[s][m] = *reinterpret_cast<const uint32_t*>(p);
+                }
             }
         }
     };
     // registers -> LDS
     auto commit = [&](int t, int nt) {
-        const uint32_t s_lo = cs[t];
-        const int nvec = (int)(cs[t + nt] - s_lo) / 4;
+        uint32_t lo[kMaxBlockSet], pre[kMaxBlockSet + 1];
+        pre[0] = 0;
+#pragma unroll
+        for (int j = 0; j < kMaxBlockSet; ++j) {
+            const bool live = j < bs;
+            lo[j] = live ? cs[(size_t)j * a.T + t] : 0u;
+            pre[j + 1] = pre[j] + (live ? (cs[(size_t)j * a.T + t + nt] - lo[j]) / 4 : 0u);
+        }
 #pragma unroll
         for (int i = 0; i < NV; ++i)
-            if (tid + i * NT < nvec) reinterpret_cast<u32x4*>(buf)[tid + i * NT] = cv[i];
-        const int k_lo = t * a.tile_rows, k_hi = min(a.K, (t + nt) * a.tile_rows);
-        const int v_lo = k_lo / VE, v_hi = (k_hi + VE - 1) / VE;
+            if ((uint32_t)(tid + i * NT) < pre[kMaxBlockSet]) reinterpret_cast<u32x4*>(buf)[tid + i * NT] = cv[i];
+        if (tid < kMaxBlockSet * (TG + 1)) {
+            const int j = tid / (TG + 1), tl = tid % (TG + 1);
+            if (j < bs && tl <= nt) cst[tid] = pre[j] * 4 + cs[(size_t)j * a.T + t + tl] - lo[j];
+        }
+        if constexpr (MT <= 4) {
+            if (a.x_mode == kStageRowVectors) {
+                // slots the rows do not cover (past a tile's height, the sentinel slot) must read as zero
+                for (int e = tid; e < nt * kTileSlots; e += NT)
+                    if ((e & 255) >= min(a.tile_rows, a.K - (t + (e >> 8)) * a.tile_rows)) {
 #pragma unroll
-        for (int i = 0; i < XPR; ++i) {
-            const int v = v_lo + tid + i * NT;
-            if (v < v_hi) {
-                int k = v * VE;
-                int tile = (int)(((unsigned long long)(unsigned)k * a.tile_magic) >> 32);  // k / tile_rows
-                int r = k - tile * a.tile_rows;
+                        for (int m = 0; m < MT; ++m) xs[(size_t)e * MT + m] = XT(0.0f);
+                    }
+                const int k_lo = t * a.tile_rows, k_hi = min(a.K, (t + nt) * a.tile_rows);
+                const int v_lo = k_lo / VE, v_hi = (k_hi + VE - 1) / VE;
 #pragma unroll
-                for (int e = 0; e < VE; ++e) {
-                    if (k >= k_lo && k < k_hi) {
-                        float* dst = xs + (size_t)((tile - t) * kTileSlots + r) * MT;
+                for (int i = 0; i < XPR; ++i) {
+                    const int v = v_lo + tid + i * NT;
+                    if (v < v_hi) {
+                        int k = v * VE;
+                        int tile = (int)(((unsigned long long)(unsigned)k * a.tile_magic) >> 32);  // k / tile_rows
+                        int r = k - tile * a.tile_rows;
 #pragma unroll
-                        for (int m = 0; m < MT; ++m) {
-                            const uint32_t word = xv[m * XPR + i][XF16 ? e / 2 : e];
-                            dst[m] = XF16 ? __half2float(__ushort_as_half((unsigned short)(e % 2 ? word >> 16 : word & 0xffffu)))
-                                          : __uint_as_float(word);
+                        for (int el = 0; el < VE; ++el) {
+                            if (k >= k_lo && k < k_hi) {
+                                XT* dst = xs + (size_t)((tile - t) * kTileSlots + r) * MT;
+#pragma unroll
+                                for (int m = 0; m < MT; ++m) {
+                                    const int f = (m * XPR + i) * 4 + (XF16 ? el / 2 : el);
+                                    const uint32_t word = xr[f / RPS][f % RPS];
+                                    if constexpr (XF16) dst[m] = __ushort_as_half((unsigned short)(el % 2 ? word >> 16 : word & 0xffffu));
+                                    else dst[m] = __uint_as_float(word);
+                                }
+                            }
+                            ++k;
+                            if (++r == a.tile_rows) { r = 0; ++tile; }
                         }
                     }
-                    ++k;
-                    if (++r == a.tile_rows) { r = 0; ++tile; }
+                }
+                return;
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < SPT; ++s) {
+            const int e = tid + s * NT;
+            const int tile = e >> 8, r = e & 255;
+            if (tile < nt) {
+                const bool real = r < min(a.tile_rows, a.K - (t + tile) * a.tile_rows);
+                uint32_t packed[MT * ES / 4 > 0 ? MT * ES / 4 : 1];
+                if constexpr (MT >= 8) {
+#pragma unroll
+                    for (int d = 0; d < MT * ES / 4; ++d) packed[d] = real ? xr[s][d] : 0u;
+                } else if (a.x_mode == kStageSlotVectors && VPS > 0) {
+#pragma unroll
+                    for (int d = 0; d < MT * ES / 4; ++d) packed[d] = real ? xr[s][d] : 0u;
+                } else if constexpr (XF16) {
+                    if constexpr (MT == 1) packed[0] = real ? xr[s][0] : 0u;
+#pragma unroll
+                    for (int d = 0; d < MT / 2; ++d) packed[d] = real ? (xr[s][2 * d] | (xr[s][2 * d + 1] << 16)) : 0u;
+                } else {
+#pragma unroll
+                    for (int d = 0; d < MT; ++d) packed[d] = real ? xr[s][d] : 0u;
+                }
+                unsigned char* dst = reinterpret_cast<unsigned char*>(xs) + (size_t)e * MT * ES;
+                if constexpr (MT * ES >= 16) {
+#pragma unroll
+                    for (int v = 0; v < MT * ES / 16; ++v)
+                        reinterpret_cast<u32x4*>(dst)[v] = u32x4{packed[4 * v], packed[4 * v + 1], packed[4 * v + 2], packed[4 * v + 3]};
+                } else if constexpr (MT * ES == 8) {
+                    *reinterpret_cast<uint2*>(dst) = make_uint2(packed[0], packed[1]);
+                } else if constexpr (MT * ES == 4) {
+                    *reinterpret_cast<uint32_t*>(dst) = packed[0];
+                } else {
+                    *reinterpret_cast<unsigned short*>(dst) = (unsigned short)packed[0];
                 }
             }
         }
-        if (tid <= nt) cst[tid] = cs[t + tid] - s_lo;
     };
 
-    const int col = tid / LPC, lig = tid % LPC;
-    const int tp = lig / LW, lw = lig % LW;
+    const int lpc_shift = a.lpc_shift, lw_shift = a.lw_shift;
+    const int LPC = 1 << lpc_shift, LW = 1 << lw_shift, TP = LPC >> lw_shift;
+    const int col = tid >> lpc_shift, lig = tid & (LPC - 1);
+    const int blk = col >> 4, c16 = col & 15;
+    const int tp = lig >> lw_shift, lw = lig & (LW - 1);
+    const uint32_t* my_cst = cst + blk * (TG + 1);
     float acc[MT];
 #pragma unroll
     for (int m = 0; m < MT; ++m) acc[m] = 0.f;
@@ -227,36 +374,41 @@ __global__ __launch_bounds__(kBlockThreads) void tl_spmm_block(KernelArgs a)
         commit(t, nt);
         __syncthreads();
         if (t + TG < a.T) prefetch(t + TG, min(TG, a.T - t - TG));
-        for (int tl0 = tp; tl0 < nt; tl0 += TP * TU) {
-            uint32_t d[TU], w[TU];
-            const uint32_t* run[TU];
+        if (blk < bs) {
+            for (int tl0 = tp; tl0 < nt; tl0 += TP * TU) {
+                uint32_t d[TU];
+                const uint32_t* run[TU];
 #pragma unroll
-            for (int u = 0; u < TU; ++u) {
-                const int tl = tl0 + u * TP;
-                const uint32_t* chunk = buf + cst[min(tl, nt - 1)];
-                d[u] = tl < nt ? chunk[col] : 0u;  // tiles past the group: empty run
-                run[u] = chunk + (d[u] >> 16);
-            }
+                for (int u = 0; u < TU; ++u) {
+                    const int tl = tl0 + u * TP;
+                    const uint32_t* chunk = buf + my_cst[min(tl, nt - 1)];
+                    d[u] = tl < nt ? chunk[c16] : 0u;  // tiles past the group: empty run
+                    run[u] = chunk + (d[u] >> 16);
+                }
+                uint32_t w[TU];
 #pragma unroll
-            for (int u = 0; u < TU; ++u)  // lanes past the run's end take an all-sentinel word: four gathers of zero
-                w[u] = lw < run_pos_dwords(d[u]) + run_neg_dwords(d[u]) ? run[u][lw] : 0xffffffffu;
+                for (int u = 0; u < TU; ++u)  // lanes past the run's end take an all-sentinel word: four gathers of zero
+                    w[u] = lw < run_pos_dwords(d[u]) + run_neg_dwords(d[u]) ? run[u][lw] : 0xffffffffu;
 #pragma unroll
-            for (int u = 0; u < TU; ++u) {
-                const int pd = run_pos_dwords(d[u]), tot = pd + run_neg_dwords(d[u]);
-                const float* xt = xs + (size_t)min(tl0 + u * TP, nt - 1) * kTileSlots * MT;
-                gather_add<MT>(acc, xt, w[u], lw < pd ? 1.0f : -1.0f);
-                for (int i = lw + LW; i < tot; i += LW)  // runs longer than the lane group
-                    gather_add<MT>(acc, xt, run[u][i], i < pd ? 1.0f : -1.0f);
+                for (int u = 0; u < TU; ++u) {
+                    const int pd = run_pos_dwords(d[u]), tot = pd + run_neg_dwords(d[u]);
+                    if (u > 0 && __builtin_amdgcn_ballot_w64(tot > 0) == 0) continue;  // no lane of the wave has this tile
+                    const XT* xt = xs + (size_t)min(tl0 + u * TP, nt - 1) * kTileSlots * MT;
+                    gather_add<MT, XT>(acc, xt, w[u], lw < pd ? 1.0f : -1.0f);
+                    for (int i = lw + LW; i < tot; i += LW)  // runs longer than the lane group
+                        gather_add<MT, XT>(acc, xt, run[u][i], i < pd ? 1.0f : -1.0f);
+                }
             }
         }
     }
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
 #pragma unroll
-        for (int off = LPC / 2; off > 0; off >>= 1) acc[m] += __shfl_xor(acc[m], off, 64);
+        for (int off = 16; off > 0; off >>= 1)
+            if (off < LPC) acc[m] += __shfl_xor(acc[m], off, 64);
     }
-    const int n = nb * TL_BLOCK_COLUMNS + col;
-    if (lig == 0 && n < a.N) {
+    const int n = (nb0 + blk) * TL_BLOCK_COLUMNS + c16;
+    if (lig == 0 && blk < bs && n < a.N) {
         const float s = load_scale(a.w0.scale, a.scale_f16, n);
 #pragma unroll
         for (int m = 0; m < MT; ++m)
@@ -679,100 +831,154 @@ int raise_lds_limit(KernelT kernel, size_t bytes)
     return TL_OK;
 }
 
-template <int MT, int LW, bool XF16>
+// out[k][m] = x(m, k) for m < M, zero for M <= m < ldo (ldo <= 48), from activations of any layout
+// (element strides sm, sk): the aligned K-major image the small-M kernel copies as vectors.
+// A workgroup moves 64 values of k.
+template <typename T>
+__global__ __launch_bounds__(256) void tl_to_kmajor(const T* __restrict__ X, long long sm, long long sk, T* __restrict__ out, int ldo, int M, int K)
+{
+    __shared__ T tile[48][65];
+    const int k0 = blockIdx.x * 64;
+    T v[12];
+#pragma unroll
+    for (int i = 0; i < 12; ++i) {
+        const int idx = threadIdx.x + i * 256, m = idx >> 6, k = k0 + (idx & 63);
+        v[i] = (m < M && k < K) ? X[(size_t)m * sm + (size_t)k * sk] : T(0.0f);
+    }
+#pragma unroll
+    for (int i = 0; i < 12; ++i) {
+        const int idx = threadIdx.x + i * 256, m = idx >> 6;
+        if (m < ldo) tile[m][idx & 63] = v[i];
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < 64 * ldo; idx += 256) {
+        const int kk = idx / ldo, m = idx - kk * ldo;
+        if (k0 + kk < K) out[(size_t)(k0 + kk) * ldo + m] = tile[m][kk];
+    }
+}
+
+inline int64_t small_kmajor_bytes(const tl_layout_header* h, int64_t M, int x_dtype)
+{
+    return M > 4 ? (int64_t)h->inners * round_up(M, 16) * (x_dtype == TL_F16 ? 2 : 4) : 0;
+}
+
+// LDS one workgroup of the small-M kernel may use: two workgroups fit a compute unit's 160 KB; a launch
+// with no more workgroups than compute units lets each have (nearly) all of it.
+constexpr int kSmallLdsShared = 78 * 1024;
+constexpr int kSmallLdsAlone = 158 * 1024;
+constexpr int kComputeUnits = 256;
+
+template <int MT, bool XF16>
 int launch_block_kernel(KernelArgs a, const tl_layout_header* h, hipStream_t st)
 {
-    using Shape = BlockShape<MT, kBlockThreads>;
-    const int by_stream = (int)(Shape::kStreamCap / ((int64_t)h->max_chunk_dwords * 4));
-    a.tiles_per_group = std::max(1, std::min(std::min(Shape::kTiles, by_stream), 255));
-    a.tile_magic = (unsigned)(((1ull << 32) + h->tile_rows - 1) / h->tile_rows);
-    const size_t lds = kSmallXBytes + kSmallStreamBytes + 1024;
-    auto kernel = tl_spmm_block<MT, LW, XF16>;
+    constexpr int es = XF16 ? 2 : 4;
+    using Shape = BlockShape<MT, es, kBlockThreads>;
+    const int tile_bytes = kTileSlots * MT * es;
+    const int64_t chunk_bytes = (int64_t)h->max_chunk_dwords * 4;
+    if (chunk_bytes * a.block_set > Shape::kStreamCap) return fail(TL_ERR_UNSUPPORTED, "a tile's chunks do not fit the staging registers");
+    const unsigned gx = (unsigned)ceil_div(a.NB, a.block_set), gy = (unsigned)ceil_div(a.M, MT);
+    const int budget = env_int("TL_SMALL_LDS", (int64_t)gx * gy <= kComputeUnits ? kSmallLdsAlone : kSmallLdsShared);
+    // tiles per group: bounded by the registers of the staging (Shape), by the LDS budget shared between
+    // the activation image and the chunk copies, and by the stream bytes one group may hold
+    const int per_tile = tile_bytes + (int)chunk_bytes * a.block_set;
+    int tg = std::min(Shape::kTiles, (budget - 1024) / per_tile);
+    tg = std::min(tg, (int)(Shape::kStreamCap / (chunk_bytes * a.block_set)));
+    tg = std::max(1, std::min(std::min(tg, a.T), 255));
+    tg = (int)ceil_div(a.T, ceil_div(a.T, tg));  // same number of groups, evened out
+    a.tiles_per_group = tg;
+    a.xs_bytes = tg * tile_bytes;
+    a.buf_bytes = (int)round_up(std::min<int64_t>(chunk_bytes * a.block_set * tg, Shape::kStreamCap), 16);
+    const size_t lds = (size_t)a.xs_bytes + a.buf_bytes + (size_t)kMaxBlockSet * (tg + 1) * 4;
+    if (lds > 160 * 1024) return fail(TL_ERR_UNSUPPORTED, "one tile of %d rows needs %zu bytes of LDS", MT, lds);
+    auto kernel = tl_spmm_block<MT, XF16>;
     static bool raised = false;  // per instantiation; a repeated or racing call is harmless
     if (!raised) {
-        if (int rc = raise_lds_limit(kernel, lds)) return rc;
+        if (int rc = raise_lds_limit(kernel, 160 * 1024)) return rc;
         raised = true;
     }
-    dim3 grid((unsigned)a.NB, (unsigned)ceil_div(a.M, MT));
-    hipLaunchKernelGGL(kernel, grid, dim3(kBlockThreads), lds, st, a);
+    hipLaunchKernelGGL(kernel, dim3(gx, gy), dim3(kBlockThreads), lds, st, a);
     return TL_OK;
 }
 
 template <int MT>
-int launch_small_lpc(const KernelArgs& a, const tl_layout_header* h, int lpc, hipStream_t st)
+int launch_small_mt(const KernelArgs& a, const tl_layout_header* h, hipStream_t st)
 {
-    if (a.x_f16) {
-        switch (lpc) {
-            case 8: return launch_block_kernel<MT, 8, true>(a, h, st);
-            case 16: return launch_block_kernel<MT, 16, true>(a, h, st);
-            default: return launch_block_kernel<MT, 32, true>(a, h, st);
-        }
-    }
-    switch (lpc) {
-        case 8: return launch_block_kernel<MT, 8, false>(a, h, st);
-        case 16: return launch_block_kernel<MT, 16, false>(a, h, st);
-        default: return launch_block_kernel<MT, 32, false>(a, h, st);
-    }
+    return a.x_f16 ? launch_block_kernel<MT, true>(a, h, st) : launch_block_kernel<MT, false>(a, h, st);
 }
 
-// Row-major activations with 16-byte aligned rows are read in place; anything else
-// (K-major, odd leading dimension, odd base address) is first repacked into the workspace.
-inline bool small_needs_repack(const void* X, int x_dtype, int x_layout, int64_t ldx, int64_t K)
+inline int log2_exact(int v)
 {
-    const int es = x_dtype == TL_F16 ? 2 : 4;
-    // K must be whole vectors too: the kernel reads 16 bytes at a time and must not run past a row's end
-    return x_layout != TL_X_ROW_MAJOR || (ldx * es) % 16 != 0 || (K * es) % 16 != 0 || reinterpret_cast<uintptr_t>(X) % 16 != 0;
-}
-inline int64_t small_repack_bytes(const tl_layout_header* h, int64_t M, int x_dtype)
-{
-    // rows padded to a multiple of 8 values plus one spare vector: the kernel reads whole vectors
-    return M * (round_up(h->inners, 8) + 8) * (x_dtype == TL_F16 ? 2 : 4);
-}
-
-template <typename T>
-__global__ __launch_bounds__(256) void tl_repack_rows(const T* __restrict__ X, long long ldx, int kmajor, T* __restrict__ out,
-                                                      long long ldo, int M, int K)
-{
-    const long long i = blockIdx.x * 256ll + threadIdx.x;
-    if (i >= (long long)M * ldo) return;
-    const int m = (int)(i / ldo), k = (int)(i % ldo);
-    out[i] = k < K ? (kmajor ? X[(long long)k * ldx + m] : X[(long long)m * ldx + k]) : T(0.0f);
+    int s = 0;
+    while ((1 << s) < v) ++s;
+    return s;
 }
 
 int launch_small(KernelArgs a, const tl_layout_header* h, int x_dtype, void* workspace, int64_t workspace_bytes, hipStream_t st)
 {
     int mt = 1;
-    while (mt < a.M && mt < 32) mt *= 2;
-    // lanes per run: one dword per lane should cover a typical run in one pass
-    const double mean_run = h->mean_run_dwords_x16 / 16.0;
-    int lpc = 8;
-    while (lpc < 32 && lpc < mean_run) lpc *= 2;
-    lpc = env_int("TL_LPC", lpc);
-    if (lpc != 8 && lpc != 16 && lpc != 32) return fail(TL_ERR_ARG, "TL_LPC=%d (8, 16 or 32 expected)", lpc);
-    if (small_needs_repack(a.X, x_dtype, a.x_kmajor ? TL_X_K_MAJOR : TL_X_ROW_MAJOR, a.ldx, a.K)) {
-        const int64_t need = small_repack_bytes(h, a.M, x_dtype);
+    while (mt < a.M && mt < 16) mt *= 2;
+    const int es = x_dtype == TL_F16 ? 2 : 4;
+    a.x_sm = a.x_kmajor ? 1 : a.ldx;
+    a.x_sk = a.x_kmajor ? a.ldx : 1;
+    bool aligned = (a.ldx * es) % 16 == 0 && reinterpret_cast<uintptr_t>(a.X) % 16 == 0;
+    // Slots of 8 rows and more are staged as whole vectors from an aligned K-major image; activations
+    // that are not one already are brought into that form in the workspace first.
+    if (mt >= 8 && !(a.x_kmajor && aligned && a.ldx >= round_up(a.M, mt))) {
+        const int64_t need = small_kmajor_bytes(h, a.M, x_dtype);
         if (!workspace || workspace_bytes < need)
             return fail(TL_ERR_SIZE, "workspace has %lld bytes, %lld needed", (long long)workspace_bytes, (long long)need);
         if (reinterpret_cast<uintptr_t>(workspace) % 16) return fail(TL_ERR_ALIGN, "workspace must be 16-byte aligned");
-        const long long ldo = round_up(a.K, 8) + 8;
-        const unsigned blocks = (unsigned)ceil_div((int64_t)a.M * ldo, 256);
+        const int ldo = (int)round_up(a.M, 16);
+        const unsigned blocks = (unsigned)ceil_div(a.K, 64);
         if (x_dtype == TL_F16)
-            hipLaunchKernelGGL(tl_repack_rows<__half>, dim3(blocks), dim3(256), 0, st, static_cast<const __half*>(a.X), a.ldx,
-                               a.x_kmajor, static_cast<__half*>(workspace), ldo, a.M, a.K);
+            hipLaunchKernelGGL(tl_to_kmajor<__half>, dim3(blocks), dim3(256), 0, st, static_cast<const __half*>(a.X), a.x_sm, a.x_sk,
+                               static_cast<__half*>(workspace), ldo, a.M, a.K);
         else
-            hipLaunchKernelGGL(tl_repack_rows<float>, dim3(blocks), dim3(256), 0, st, static_cast<const float*>(a.X), a.ldx,
-                               a.x_kmajor, static_cast<float*>(workspace), ldo, a.M, a.K);
+            hipLaunchKernelGGL(tl_to_kmajor<float>, dim3(blocks), dim3(256), 0, st, static_cast<const float*>(a.X), a.x_sm, a.x_sk,
+                               static_cast<float*>(workspace), ldo, a.M, a.K);
         a.X = workspace;
         a.ldx = ldo;
-        a.x_kmajor = 0;
+        a.x_kmajor = 1;
+        a.x_sm = 1;
+        a.x_sk = ldo;
+        aligned = true;
     }
+    // Column blocks per workgroup.  A compute unit works through ceil(workgroups / 256) workgroups of
+    // `set` blocks each; among the sets that keep that product smallest, wider ones re-read the
+    // activations less often, which pays once a slot holds many rows.
+    int set = 1;
+    {
+        int64_t best = -1;
+        for (int cand = 1; cand <= kMaxBlockSet; cand *= 2) {
+            if ((int64_t)h->max_chunk_dwords * 4 * cand > BlockShape<1, 2, kBlockThreads>::kStreamCap) break;
+            const int64_t cost = ceil_div(ceil_div(a.NB, cand), kComputeUnits) * cand;
+            if (best < 0 || cost < best || (cost == best && mt >= 8)) { best = cost; set = cand; }
+        }
+    }
+    set = env_int("TL_BLOCK_SET", set);
+    if (set != 1 && set != 2 && set != 4) return fail(TL_ERR_ARG, "TL_BLOCK_SET=%d (1, 2 or 4 expected)", set);
+    a.block_set = set;
+    const int lpc = kBlockThreads / (TL_BLOCK_COLUMNS * set);
+    // lanes per run: one dword per lane should cover a typical run in a whole number of passes with
+    // few idle lanes; runs hold mean_run dwords (+1 and -1 parts together)
+    const double mean_run = h->mean_run_dwords_x16 / 16.0;
+    int lw = 4;
+    while (lw < lpc && lw * 3 < mean_run) lw *= 2;
+    lw = std::min(env_int("TL_LW", lw), lpc);
+    if (lw != 1 && lw != 2 && lw != 4 && lw != 8 && lw != 16 && lw != 32) return fail(TL_ERR_ARG, "TL_LW=%d (a power of two up to 32 expected)", lw);
+    a.lpc_shift = log2_exact(lpc);
+    a.lw_shift = log2_exact(lw);
+    a.x_mode = kStageElements;
+    if (a.x_kmajor && mt * es >= 16 && aligned && a.ldx >= round_up(a.M, mt)) a.x_mode = kStageSlotVectors;
+    // whole vectors of a row are read: K must be whole vectors too, so that none runs past a row's end
+    if (!a.x_kmajor && mt <= 4 && aligned && ((int64_t)a.K * es) % 16 == 0) a.x_mode = kStageRowVectors;
+    a.tile_magic = (unsigned)(((1ull << 32) + h->tile_rows - 1) / h->tile_rows);
     switch (mt) {
-        case 1: return launch_small_lpc<1>(a, h, lpc, st);
-        case 2: return launch_small_lpc<2>(a, h, lpc, st);
-        case 4: return launch_small_lpc<4>(a, h, lpc, st);
-        case 8: return launch_small_lpc<8>(a, h, lpc, st);
-        case 16: return launch_small_lpc<16>(a, h, lpc, st);
-        default: return launch_small_lpc<32>(a, h, lpc, st);
+        case 1: return launch_small_mt<1>(a, h, st);
+        case 2: return launch_small_mt<2>(a, h, st);
+        case 4: return launch_small_mt<4>(a, h, st);
+        case 8: return launch_small_mt<8>(a, h, st);
+        default: return launch_small_mt<16>(a, h, st);
     }
 }
 
@@ -864,11 +1070,9 @@ extern "C" int tl_spmm_workspace(const tl_layout_header* header, int64_t M, int 
     if (int rc = check_dtype(x_dtype, "x")) return rc;
     if (!workspace_bytes) return fail(TL_ERR_ARG, "workspace_bytes is null");
     if (M <= 0) return fail(TL_ERR_SHAPE, "M=%lld must be positive", (long long)M);
-    if (M <= kSmallMaxM) {
-        // needed only when the activations have to be repacked (K-major or unaligned rows); whether the
-        // base address is aligned is not known here, so the room is always asked for
-        *workspace_bytes = small_repack_bytes(header, M, x_dtype);
-        (void)x_layout;
+    if (M <= kSmallMaxM) {  // room for the aligned K-major image of the activations (more than 4 rows)
+        (void)x_layout;  // K-major activations need it too when they are not aligned vectors
+        *workspace_bytes = small_kmajor_bytes(header, M, x_dtype);
         return TL_OK;
     }
     *workspace_bytes = (int64_t)header->inners * round_up(M, rows_mtile(x_dtype)) * (x_dtype == TL_F16 ? 2 : 4);
