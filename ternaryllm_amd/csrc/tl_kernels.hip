@@ -401,11 +401,16 @@ __global__ __launch_bounds__(kBlockThreads) void tl_spmm_block(KernelArgs a)
             }
         }
     }
+    // fold the LPC partial sums of a column; per step the MT exchanges are independent of each other
 #pragma unroll
-    for (int m = 0; m < MT; ++m) {
+    for (int off = 16; off > 0; off >>= 1) {
+        if (off < LPC) {
+            float other[MT];
 #pragma unroll
-        for (int off = 16; off > 0; off >>= 1)
-            if (off < LPC) acc[m] += __shfl_xor(acc[m], off, 64);
+            for (int m = 0; m < MT; ++m) other[m] = __shfl_xor(acc[m], off, 64);
+#pragma unroll
+            for (int m = 0; m < MT; ++m) acc[m] += other[m];
+        }
     }
     const int n = (nb0 + blk) * TL_BLOCK_COLUMNS + c16;
     if (lig == 0 && blk < bs && n < a.N) {
