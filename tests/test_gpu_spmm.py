@@ -115,3 +115,29 @@ def test_k_major_input_and_tile_heights(cuda, oracle):
             assert np.array_equal(y.astype(np.float64), ref), (M, tile_rows)
             yk = ops.spmm(dw, x.t().contiguous().to(cuda), x_layout=1).cpu().numpy()
             assert np.array_equal(yk.astype(np.float64), ref), (M, tile_rows, "k-major")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("M", [1, 3, 4, 9, 16, 40])
+def test_small_m_activation_layouts(cuda, oracle, M, dtype):
+    """Every way the small-M kernel stages activations: whole row vectors, single elements (odd leading
+    dimension, odd K), K-major vectors, and the K-major pre-pass for 8 rows and more."""
+    from ternaryllm_amd import ops
+    from ternaryllm_amd.packing import PackedWeight
+    for K, N in ((1024, 96), (777, 50)):
+        w = ternary_weight(K, N, 0.7, 41 + K)
+        dw = ops.DeviceWeight(PackedWeight.from_dense(w), cuda)
+        x = activations(M, K, 42 + M, dtype, integer=True)
+        ref = oracle.fast_product(x.double().numpy(), w)
+        xd = x.to(cuda)
+        cases = {"row-major": (xd, 0), "k-major": (xd.t().contiguous(), 1)}
+        wide = torch.zeros((M, K + 3), dtype=dtype, device=cuda)           # rows with an odd leading dimension
+        wide[:, :K] = xd
+        cases["row-major, strided"] = (wide[:, :K], 0)
+        widek = torch.zeros((K, M + 5), dtype=dtype, device=cuda)          # K-major with an odd leading dimension
+        widek[:, :M] = xd.t()
+        cases["k-major, strided"] = (widek[:, :M], 1)
+        for name, (xin, layout) in cases.items():
+            print(f"case M={M} K={K} dtype={dtype} {name}", flush=True)
+            y = ops.spmm(dw, xin, x_layout=layout).float().cpu().numpy()
+            assert np.array_equal(y.astype(np.float64), ref), (M, K, name)
