@@ -34,6 +34,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
+    ap.add_argument("--no-decoder", action="store_true", help="skip the 32-layer decoder (prefill 512 + 128 greedy steps)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one plain 256 MiB device copy (reference for scaling rocprof's FETCH_SIZE / WRITE_SIZE)")
     return ap.parse_args()
@@ -69,6 +70,48 @@ def time_spmm(dw, x, scale, steps, warmup, x_layout=0):
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
     ev_ms, _ = ops.spmm_time(dw, x, steps, scale, x_layout=x_layout)
     return wall_ms, ev_ms
+
+
+def decoder_leg(dev, prompt=512, new_tokens=128):
+    """Llama-2-7B-shaped ternary decoder on random weights: prefill of `prompt` random ids, then
+    `new_tokens` greedy steps (the step captured once in a HIP graph), at batch 1 and 16."""
+    import torch
+    from ternaryllm_amd import TernaryConfig, TernaryLlamaDecoder
+    cfg = TernaryConfig(sparsity=0.66, max_position_embeddings=prompt + new_tokens)
+    t0 = time.perf_counter()
+    model = TernaryLlamaDecoder(cfg, seed=1242, device=dev, pack_threads=16)
+    torch.cuda.synchronize()
+    res = {"layers": cfg.num_hidden_layers, "hidden": cfg.hidden_size, "ffn": cfg.intermediate_size, "vocab": cfg.vocab_size,
+           "sparsity": cfg.sparsity, "build_s": round(time.perf_counter() - t0, 1),
+           "weights_GB": round(sum(b.numel() for n, b in model.named_buffers() if n.endswith("w_packed")) / 1e9, 3)}
+    g = torch.Generator().manual_seed(1243)
+    for B in (1, 16):
+        tokens = torch.randint(0, cfg.vocab_size, (B, prompt), generator=g).to(dev)
+        model.allocate_cache(B)
+        model.prefill(tokens)  # warm-up: kernel attributes, workspaces
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        logits = model.prefill(tokens)
+        torch.cuda.synchronize()
+        t_prefill = time.perf_counter() - t0
+        st = model._decode_state(B)
+        st["token"].copy_(logits.argmax(-1))
+        st["pos"].fill_(prompt)
+        st["mask"].copy_((torch.arange(model.max_seq_len, device=dev) <= prompt)[None, None, None])
+        model.decode_once(st, True)  # captures the graph; counts as the first of the new tokens' steps
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(new_tokens - 1):
+            model.decode_once(st, True)
+        torch.cuda.synchronize()
+        t_decode = (time.perf_counter() - t0) * new_tokens / (new_tokens - 1)
+        res["batch_%d" % B] = {"prefill_ms": round(t_prefill * 1e3, 2), "prefill_tokens_per_s": round(B * prompt / t_prefill, 1),
+                               "decode_ms_per_step": round(t_decode * 1e3 / new_tokens, 4),
+                               "decode_tokens_per_s": round(B * new_tokens / t_decode, 1),
+                               "end_to_end_tokens_per_s": round(B * (prompt + new_tokens) / (t_prefill + t_decode), 1)}
+    del model
+    torch.cuda.empty_cache()
+    return res
 
 
 def main():
@@ -187,6 +230,9 @@ def main():
         torch.cuda.synchronize()
         mlp_ms = (time.perf_counter() - t0) * 1e3 / 10
         extra["c3_mlp_block_fused"] = {"ms": round(mlp_ms, 4), "tokens_per_s": round(M / (mlp_ms * 1e-3), 1)}
+    # ---- whole decoder: 32 layers, every linear ternary at 66 % sparsity -------
+    if not args.no_extra and not args.no_decoder:
+        extra["c5_decoder"] = decoder_leg(dev)
     out["extra"] = extra
     print(json.dumps(out))
 

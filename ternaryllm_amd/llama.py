@@ -227,7 +227,9 @@ class TernaryLlamaDecoder(nn.Module):
     def _advance(self, st):
         logits = self._decode_step(st["token"], st["pos"], st["mask"])
         st["token"].copy_(logits.argmax(-1))
-        st["pos"].add_(1)
+        # positions stay inside the cache even if a caller steps past its end (the results are then
+        # meaningless, but nothing is written out of bounds; generate() checks the length up front)
+        st["pos"].add_(1).clamp_(max=self.max_seq_len - 1)
         st["mask"].index_fill_(3, st["pos"], True)
 
     @torch.no_grad()
