@@ -7,6 +7,9 @@ from .linear import TernaryLinear, random_ternary_weights, convert_ternary_weigh
 from .mlp import LlamaTernaryMLP
 from .attention import LlamaTernaryAttention
 from .llama import TernaryLlamaDecoder
+from .surgery import (collect_linear_layers, replace_linear_layers, prepare_ternary_model, add_padding_to_token,
+                      collect_attn_linear_layers)
 
-__all__ = ["TernaryLinear", "LlamaTernaryMLP", "LlamaTernaryAttention", "TernaryConfig", "TernaryLlamaDecoder",
+__all__ = ["TernaryLinear", "LlamaTernaryMLP", "LlamaTernaryAttention", "TernaryConfig", "TernaryLlamaDecoder", "collect_linear_layers", "replace_linear_layers",
+           "prepare_ternary_model", "add_padding_to_token", "collect_attn_linear_layers",
            "random_ternary_weights", "convert_ternary_weights", "MapKSizeToTileSize"]

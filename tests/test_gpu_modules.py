@@ -150,3 +150,34 @@ def test_full_size_properties(cuda):
     # decode shape (M = 1) on the same weight
     y1 = ops.spmm(dw, xa[:1].to(cuda), out_dtype=torch.float32)
     assert torch.equal(y1, ya[:1])
+
+
+def test_surgery_on_a_hugging_face_llama(cuda):
+    """prepare_ternary_model on a small transformers Llama built from a local config (no download):
+    the patched model's logits equal those of the same model with dense linears holding the ternary
+    weights."""
+    transformers = pytest.importorskip("transformers")
+    import copy
+    from ternaryllm_amd import TernaryConfig, TernaryLinear, prepare_ternary_model
+    torch.manual_seed(11)
+    hf_cfg = transformers.LlamaConfig(hidden_size=128, intermediate_size=256, num_hidden_layers=2, num_attention_heads=4,
+                                      num_key_value_heads=4, vocab_size=120, max_position_embeddings=64)
+    model = transformers.LlamaForCausalLM(hf_cfg).eval()
+    cfg = TernaryConfig(sparsity=0.7)
+    model = prepare_ternary_model(model, cfg, device=cuda, generator=torch.Generator().manual_seed(12))
+    replaced = [m for m in model.modules() if isinstance(m, TernaryLinear)]
+    assert len(replaced) == 2 * 7
+    dense = copy.deepcopy(model).to("cpu")
+    for name, mod in list(dense.named_modules()):
+        if isinstance(mod, TernaryLinear):
+            lin = torch.nn.Linear(mod.in_features, mod.out_features, bias=False)
+            lin.weight.data = mod.ternary_weight.t().float().contiguous()
+            parent, _, leaf = name.rpartition(".")
+            setattr(dense.get_submodule(parent), leaf, lin)
+    dense = dense.to(cuda)
+    ids = torch.randint(0, 120, (2, 24), generator=torch.Generator().manual_seed(13)).to(cuda)
+    with torch.no_grad():
+        got = model(ids).logits.float()
+        ref = dense(ids).logits.float()
+    assert torch.isfinite(ref).all()
+    assert (got - ref).abs().max().item() <= 1e-3 * ref.abs().max().item()
