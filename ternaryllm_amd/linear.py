@@ -25,6 +25,28 @@ def ternarize_weights(w):
     raise NotImplementedError("ternarize_weights not implement")  # as in the reference, TernaryLinear.py:19-20
 
 
+def ternarize_threshold(w, sparsity=None):
+    """Ternarises a float weight [K, N] column by column: an entry becomes sign(w) where |w| exceeds the
+    column's threshold, else 0, and each column gets the scale that minimises the squared error for that
+    support, mean |w| over the kept entries.  The threshold is 0.7 * mean |w| of the column (the classic
+    ternary-weight rule) or, with `sparsity` given, the column's `sparsity` quantile of |w|, so that about
+    that fraction of each column is zero.  Returns (int32 [K, N] in {-1, 0, 1}, float32 scale [N]).
+    The reference has no counterpart (its ternarize_weights raises); random weights stay the default."""
+    w = torch.as_tensor(w, dtype=torch.float32)
+    mag = w.abs()
+    if sparsity is None:
+        thr = 0.7 * mag.mean(dim=0, keepdim=True)
+    else:
+        if not 0.0 <= sparsity < 1.0:
+            raise ValueError("sparsity must be in [0, 1)")
+        thr = torch.quantile(mag, sparsity, dim=0, keepdim=True)
+    keep = mag > thr
+    t = (torch.sign(w) * keep).to(torch.int32)
+    kept = keep.sum(dim=0).clamp(min=1)
+    scale = (mag * keep).sum(dim=0) / kept
+    return t, scale
+
+
 def random_ternary_weights(size, sparsity=0.8, uniform=False, block_size=512, generator=None):
     """Random ternary [K, N] int32 matrix, distributed as the reference's generator
     (TernaryLinear.py:23-85).  i.i.d. mode: r ~ U[0,1); r < s -> 0, s <= r < (s+1)/2 -> -1, else +1.
@@ -131,6 +153,15 @@ class TernaryLinear(nn.Module):
         self._handle = None
 
     @classmethod
+    def from_float(cls, weight, sparsity=None, device=None, scale_dtype=torch.float32):
+        """A module that approximates x @ weight for a float weight [K, N] (note: nn.Linear stores the
+        transpose): ternarised by ternarize_threshold, with its per-column scale."""
+        t, scale = ternarize_threshold(weight, sparsity)
+        self = cls.from_packed(packing.PackedWeight.from_dense(t), scale.to(scale_dtype), device=device)
+        self._dense = t
+        return self
+
+    @classmethod
     def from_packed(cls, packed, scale=None, device=None):
         """A module around an existing PackedWeight: no random draw, no dense copy kept, no bias and
         none of the reference's merged arrays (`ternary_weight` decodes the blob on demand)."""
@@ -218,4 +249,5 @@ class TernaryLinear(nn.Module):
         return f"in_features={self.in_features}, out_features={self.out_features}, nnz={self._packed_nnz}"
 
 
-__all__ = ["TernaryLinear", "random_ternary_weights", "convert_ternary_weights", "MapKSizeToTileSize"]
+__all__ = ["TernaryLinear", "random_ternary_weights", "convert_ternary_weights", "MapKSizeToTileSize",
+           "ternarize_weights", "ternarize_threshold"]

@@ -35,14 +35,23 @@ def collect_linear_layers(model, config):
     return picked
 
 
-def replace_linear_layers(layers, model, config, *, generator=None, reference_buffers=False, verbose=False):
+def replace_linear_layers(layers, model, config, *, generator=None, reference_buffers=False, verbose=False,
+                          from_weights=False):
     """Puts a TernaryLinear of the same shape in the place of each listed layer (TernaryLlama.py:21-36).
-    `generator` seeds the random weights; `reference_buffers` also builds the reference's merged arrays."""
+    `generator` seeds the random weights; `reference_buffers` also builds the reference's merged arrays.
+    With `from_weights` the layer's own weight is ternarised instead (threshold at the configured
+    sparsity's quantile per output channel, with the matching per-channel scale); the bias is dropped
+    either way, as in the reference."""
     for name, module in layers:
         parent_name, _, leaf = name.rpartition(".")
         parent = model.get_submodule(parent_name) if parent_name else model
         if verbose:
             print(f"replacing {name}: {module.in_features} -> {module.out_features}")
+        if from_weights:
+            scale_dtype = module.weight.dtype if module.weight.dtype in (torch.float16, torch.float32) else torch.float32
+            setattr(parent, leaf, TernaryLinear.from_float(module.weight.detach().t().float().cpu(), config.sparsity,
+                                                           scale_dtype=scale_dtype))
+            continue
         ternary = TernaryLinear(module.in_features, module.out_features, sparsity=config.sparsity,
                                 uniform=config.uniform_sparsity, uniform_blk_size=config.uniform_sparsity_block_size,
                                 padding=False, bias=False, device="cpu", generator=generator,

@@ -68,3 +68,29 @@ def test_add_padding_to_token():
     class Tok:
         pad_token, eos_token, pad_token_id = None, "</s>", 2
     assert surgery.add_padding_to_token(ids, Tok(), 4, "cpu")[0, -1] == 2
+
+
+def test_ternarize_threshold_and_from_weights():
+    from ternaryllm_amd.linear import ternarize_threshold
+    g = torch.Generator().manual_seed(3)
+    w = torch.randn(200, 30, generator=g)
+    t, scale = ternarize_threshold(w, sparsity=0.6)
+    assert t.dtype == torch.int32 and set(t.unique().tolist()) <= {-1, 0, 1}
+    assert (t == 0).float().mean(dim=0).sub(0.6).abs().max() < 0.02          # per column
+    assert torch.equal(t[t != 0].sign(), w[t != 0].sign().to(torch.int32))
+    # the scale is the least-squares one for the chosen support: <w, t> / <t, t> per column
+    ls = (w * t).sum(0) / (t * t).sum(0).clamp(min=1)
+    assert torch.allclose(scale, ls, atol=1e-6)
+    # kept entries are the largest ones
+    assert (w.abs() * (t == 0)).max(dim=0).values.le((w.abs() * (t != 0) + 1e9 * (t == 0)).min(dim=0).values).all()
+    t2, _ = ternarize_threshold(w)                                           # 0.7 * mean |w| rule
+    assert ((w.abs() > 0.7 * w.abs().mean(0, keepdim=True)) == (t2 != 0)).all()
+    m = _Toy()
+    cfg = TernaryConfig(sparsity=0.5)
+    ref_w = m.layers[0].mlp.down_proj.weight.detach().clone()
+    surgery.replace_linear_layers(surgery.collect_linear_layers(m, cfg), m, cfg, from_weights=True)
+    mod = m.layers[0].mlp.down_proj
+    assert isinstance(mod, TernaryLinear) and mod.w_scale is not None
+    approx = mod.ternary_weight.float() * mod.w_scale[None, :]
+    err = (approx - ref_w.t()).norm() / ref_w.norm()
+    assert err < 0.6                                                          # a ternary fit of uniform weights, not noise
