@@ -218,6 +218,33 @@ int tl_spmm_time(const tl_layout_header* header, const void* blob_dev,
                  void* workspace, int64_t workspace_bytes, void* stream,
                  int iters, float* mean_ms);
 
+/* ======================================================================== */
+/* Around the products of a single-token decode step.                       */
+/* ======================================================================== */
+
+/* Rotary embedding of q and k fused with the KV-cache update -- stands where the
+ * reference's attention calls apply_rotary_pos_emb and Cache.update of the
+ * transformers package (TernaryLLM/TernaryAttn.py:93-98).
+ *   qkv        device [batch][3][heads][head_dim]: q, k, v of one token per batch row
+ *   cos_table, sin_table  device [max_seq][head_dim], rotate-half form (both halves of a row alike)
+ *   pos_dev    device pointer to one int64: the token's position = the cache row written
+ *   q_out      device [batch][heads][head_dim]
+ *   k_cache, v_cache      device [batch][heads][max_seq][head_dim]
+ * A position outside [0, max_seq) writes nothing. */
+int tl_rope_cache_update(const void* qkv, int dtype, int64_t batch, int heads, int head_dim,
+                         const void* cos_table, const void* sin_table, const int64_t* pos_dev,
+                         void* q_out, void* k_cache, void* v_cache, int64_t max_seq, void* stream);
+
+/* Softmax attention of one query per (batch row, head) over cache rows [0, *pos_dev] --
+ * the reference's eager matmul / softmax / matmul for q_len == 1
+ * (TernaryLLM/TernaryAttn.py:100-113), scores and softmax in fp32.
+ *   q          device [batch][heads][head_dim]
+ *   out        device [batch][heads * head_dim]
+ * head_dim 64, 128 or 256; max_seq * 4 bytes of scores must fit 120 KB of LDS. */
+int tl_decode_attention(const void* q, const void* k_cache, const void* v_cache, int dtype,
+                        int64_t batch, int heads, int head_dim, int64_t max_seq,
+                        const int64_t* pos_dev, void* out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,226 @@
+// Two small kernels around the ternary products of a single-token decode step:
+// rotary embedding fused with the KV-cache update, and softmax attention of one query per head over
+// the cache.  They stand where the reference calls into the transformers package
+// (ternaryLLM_GPU/TernaryLLM/TernaryAttn.py:93-113: apply_rotary_pos_emb, Cache.update, the eager
+// matmul / softmax / matmul) -- a handful of tiny launches per layer there, two here.  Position and
+// valid length are read from device memory, so a captured HIP graph of the step can be replayed for
+// every token.
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+
+#include "tl_common.h"
+
+using namespace tl;
+
+namespace {
+
+template <typename T> __device__ __forceinline__ float to_f(T v);
+template <> __device__ __forceinline__ float to_f<float>(float v) { return v; }
+template <> __device__ __forceinline__ float to_f<__half>(__half v) { return __half2float(v); }
+template <typename T> __device__ __forceinline__ T from_f(float v);
+template <> __device__ __forceinline__ float from_f<float>(float v) { return v; }
+template <> __device__ __forceinline__ __half from_f<__half>(float v) { return __float2half(v); }
+
+// qkv: [batch][3][heads][head_dim] (q, k, v of one token per batch row, as the fused projection
+// writes them).  Rotate-half form: out[d] = x[d] * cos[d] - x[d + h/2] * sin[d] for d < h/2,
+// out[d] = x[d] * cos[d] + x[d - h/2] * sin[d] above.  q goes to q_out [batch][heads][head_dim];
+// rotated k and plain v go to row `pos` of the caches [batch][heads][max_seq][head_dim].
+template <typename T>
+__global__ __launch_bounds__(256) void tl_rope_cache(const T* __restrict__ qkv, const T* __restrict__ cos_t,
+                                                     const T* __restrict__ sin_t, const long long* __restrict__ pos_p,
+                                                     T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                                     int batch, int heads, int head_dim, long long max_seq)
+{
+    const long long pos = *pos_p;
+    const int half = head_dim / 2;
+    const long long i = blockIdx.x * 256ll + threadIdx.x;  // over batch * heads * head_dim
+    if (i >= (long long)batch * heads * head_dim || pos < 0 || pos >= max_seq) return;
+    const int d = (int)(i % head_dim);
+    const long long bh = i / head_dim;
+    const int h = (int)(bh % heads);
+    const long long b = bh / heads;
+    const T* base = qkv + (size_t)b * 3 * heads * head_dim + (size_t)h * head_dim;
+    const size_t plane = (size_t)heads * head_dim;
+    const float c = to_f(cos_t[(size_t)pos * head_dim + d]), s = to_f(sin_t[(size_t)pos * head_dim + d]);
+    const int partner = d < half ? d + half : d - half;
+    const float sgn = d < half ? -1.0f : 1.0f;
+    const float q = to_f(base[d]) * c + sgn * to_f(base[partner]) * s;
+    const float k = to_f(base[plane + d]) * c + sgn * to_f(base[plane + partner]) * s;
+    q_out[i] = from_f<T>(q);
+    const size_t row = ((size_t)bh * max_seq + pos) * head_dim + d;
+    k_cache[row] = from_f<T>(k);
+    v_cache[row] = base[2 * plane + d];
+}
+
+// One workgroup per (batch row, head): scores of the query against cache rows [0, pos], softmax in
+// fp32, weighted sum of the value rows.  out is [batch][heads * head_dim], the layout the output
+// projection multiplies.  Threads first own cache rows (a score is one thread's dot product over the
+// row's contiguous head_dim values), then own output dimensions (reads of a value row are contiguous
+// across threads); the two halves of the workgroup split the rows of the second pass.
+constexpr int kAttnThreads = 256;
+
+template <typename T, int HD>
+__global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restrict__ q, const T* __restrict__ k_cache,
+                                                               const T* __restrict__ v_cache, const long long* __restrict__ pos_p,
+                                                               T* __restrict__ out, int heads, long long max_seq, float scale)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    float* score = reinterpret_cast<float*>(smem);            // [n]
+    __shared__ float qs[HD];
+    __shared__ float red[kAttnThreads / 64];
+    __shared__ float partial[kAttnThreads / HD > 0 ? kAttnThreads / HD : 1][HD];
+    const int tid = threadIdx.x;
+    const long long bh = blockIdx.x;
+    long long n = *pos_p + 1;  // valid rows
+    if (n > max_seq) n = max_seq;
+    if (n < 1) n = 1;
+    const T* kc = k_cache + (size_t)bh * max_seq * HD;
+    const T* vc = v_cache + (size_t)bh * max_seq * HD;
+    for (int d = tid; d < HD; d += kAttnThreads) qs[d] = to_f(q[(size_t)bh * HD + d]) * scale;
+    __syncthreads();
+
+    float local_max = -INFINITY;
+    for (long long j = tid; j < n; j += kAttnThreads) {
+        const T* row = kc + (size_t)j * HD;
+        float acc = 0.f;
+        if constexpr (sizeof(T) == 2) {
+#pragma unroll 4
+            for (int d = 0; d < HD; d += 8) {
+                const uint4 v = *reinterpret_cast<const uint4*>(row + d);
+                const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    acc = fmaf(__half2float(__ushort_as_half((unsigned short)(w[e] & 0xffffu))), qs[d + 2 * e], acc);
+                    acc = fmaf(__half2float(__ushort_as_half((unsigned short)(w[e] >> 16))), qs[d + 2 * e + 1], acc);
+                }
+            }
+        } else {
+#pragma unroll 4
+            for (int d = 0; d < HD; d += 4) {
+                const float4 v = *reinterpret_cast<const float4*>(row + d);
+                acc = fmaf(v.x, qs[d], acc); acc = fmaf(v.y, qs[d + 1], acc);
+                acc = fmaf(v.z, qs[d + 2], acc); acc = fmaf(v.w, qs[d + 3], acc);
+            }
+        }
+        score[j] = acc;
+        local_max = fmaxf(local_max, acc);
+    }
+    // block maximum
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) local_max = fmaxf(local_max, __shfl_xor(local_max, off, 64));
+    if ((tid & 63) == 0) red[tid >> 6] = local_max;
+    __syncthreads();
+    float m = red[0];
+#pragma unroll
+    for (int w = 1; w < kAttnThreads / 64; ++w) m = fmaxf(m, red[w]);
+    __syncthreads();
+    float local_sum = 0.f;
+    for (long long j = tid; j < n; j += kAttnThreads) {
+        const float e = __expf(score[j] - m);
+        score[j] = e;
+        local_sum += e;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) local_sum += __shfl_xor(local_sum, off, 64);
+    if ((tid & 63) == 0) red[tid >> 6] = local_sum;
+    __syncthreads();
+    float total = 0.f;
+#pragma unroll
+    for (int w = 0; w < kAttnThreads / 64; ++w) total += red[w];
+
+    // weighted sum of value rows: thread -> (slice of the rows, output dimension)
+    constexpr int SLICES = kAttnThreads / HD > 0 ? kAttnThreads / HD : 1;
+    const int d = tid % HD, slice = tid / HD;
+    if (slice < SLICES) {
+        float acc = 0.f;
+        for (long long j = slice; j < n; j += SLICES) acc = fmaf(score[j], to_f(vc[(size_t)j * HD + d]), acc);
+        partial[slice][d] = acc;
+    }
+    __syncthreads();
+    if (tid < HD) {
+        float acc = 0.f;
+#pragma unroll
+        for (int s = 0; s < SLICES; ++s) acc += partial[s][tid];
+        const long long b = bh / heads;
+        const int h = (int)(bh % heads);
+        out[((size_t)b * heads + h) * HD + tid] = from_f<T>(acc / total);
+    }
+}
+
+int check_common(int dtype, int64_t batch, int heads, int head_dim, int64_t max_seq, const void* pos_dev)
+{
+    if (dtype != TL_F16 && dtype != TL_F32) return fail(TL_ERR_DTYPE, "dtype code %d unknown", dtype);
+    if (batch <= 0 || heads <= 0 || max_seq <= 0 || batch * heads > (1ll << 30)) return fail(TL_ERR_SHAPE, "batch, heads and max_seq must be positive");
+    if (head_dim <= 0 || head_dim % 2) return fail(TL_ERR_SHAPE, "head_dim=%d must be positive and even", head_dim);
+    if (!pos_dev) return fail(TL_ERR_ARG, "position pointer is null");
+    return TL_OK;
+}
+
+int launched()
+{
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(TL_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString(e));
+    return TL_OK;
+}
+
+template <typename T>
+int attn_dispatch(int head_dim, dim3 grid, size_t lds, hipStream_t st, const void* q, const void* k, const void* v,
+                  const long long* pos, void* out, int heads, long long max_seq, float scale)
+{
+    const T* qq = static_cast<const T*>(q);
+    const T* kk = static_cast<const T*>(k);
+    const T* vv = static_cast<const T*>(v);
+    T* oo = static_cast<T*>(out);
+    switch (head_dim) {
+        case 64: hipLaunchKernelGGL((tl_decode_attn<T, 64>), grid, dim3(kAttnThreads), lds, st, qq, kk, vv, pos, oo, heads, max_seq, scale); break;
+        case 128: hipLaunchKernelGGL((tl_decode_attn<T, 128>), grid, dim3(kAttnThreads), lds, st, qq, kk, vv, pos, oo, heads, max_seq, scale); break;
+        case 256: hipLaunchKernelGGL((tl_decode_attn<T, 256>), grid, dim3(kAttnThreads), lds, st, qq, kk, vv, pos, oo, heads, max_seq, scale); break;
+        default: return fail(TL_ERR_UNSUPPORTED, "head_dim=%d (64, 128 or 256 supported)", head_dim);
+    }
+    return TL_OK;
+}
+
+}  // namespace
+
+extern "C" int tl_rope_cache_update(const void* qkv, int dtype, int64_t batch, int heads, int head_dim,
+                                    const void* cos_table, const void* sin_table, const int64_t* pos_dev,
+                                    void* q_out, void* k_cache, void* v_cache, int64_t max_seq, void* stream)
+{
+    if (int rc = check_common(dtype, batch, heads, head_dim, max_seq, pos_dev)) return rc;
+    if (!qkv || !cos_table || !sin_table || !q_out || !k_cache || !v_cache) return fail(TL_ERR_ARG, "device pointer is null");
+    const int64_t total = batch * heads * head_dim;
+    dim3 grid((unsigned)ceil_div(total, 256));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const long long* pos = reinterpret_cast<const long long*>(pos_dev);
+    if (dtype == TL_F16)
+        hipLaunchKernelGGL(tl_rope_cache<__half>, grid, dim3(256), 0, st, static_cast<const __half*>(qkv),
+                           static_cast<const __half*>(cos_table), static_cast<const __half*>(sin_table), pos,
+                           static_cast<__half*>(q_out), static_cast<__half*>(k_cache), static_cast<__half*>(v_cache), (int)batch, heads,
+                           head_dim, (long long)max_seq);
+    else
+        hipLaunchKernelGGL(tl_rope_cache<float>, grid, dim3(256), 0, st, static_cast<const float*>(qkv),
+                           static_cast<const float*>(cos_table), static_cast<const float*>(sin_table), pos,
+                           static_cast<float*>(q_out), static_cast<float*>(k_cache), static_cast<float*>(v_cache), (int)batch, heads,
+                           head_dim, (long long)max_seq);
+    return launched();
+}
+
+extern "C" int tl_decode_attention(const void* q, const void* k_cache, const void* v_cache, int dtype, int64_t batch, int heads,
+                                   int head_dim, int64_t max_seq, const int64_t* pos_dev, void* out, void* stream)
+{
+    if (int rc = check_common(dtype, batch, heads, head_dim, max_seq, pos_dev)) return rc;
+    if (!q || !k_cache || !v_cache || !out) return fail(TL_ERR_ARG, "device pointer is null");
+    const size_t lds = (size_t)max_seq * sizeof(float);
+    if (lds > 120 * 1024) return fail(TL_ERR_UNSUPPORTED, "max_seq=%lld: the scores of one head must fit 120 KB of LDS", (long long)max_seq);
+    const int es = dtype == TL_F16 ? 2 : 4;
+    if (reinterpret_cast<uintptr_t>(k_cache) % 16 || ((int64_t)head_dim * es) % 16) return fail(TL_ERR_ALIGN, "cache rows must be 16-byte aligned");
+    dim3 grid((unsigned)(batch * heads));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const long long* pos = reinterpret_cast<const long long*>(pos_dev);
+    const float scale = 1.0f / sqrtf((float)head_dim);
+    int rc;
+    if (dtype == TL_F16) rc = attn_dispatch<__half>(head_dim, grid, lds, st, q, k_cache, v_cache, pos, out, heads, (long long)max_seq, scale);
+    else rc = attn_dispatch<float>(head_dim, grid, lds, st, q, k_cache, v_cache, pos, out, heads, (long long)max_seq, scale);
+    if (rc) return rc;
+    return launched();
+}

@@ -889,6 +889,7 @@ int launch_block_kernel(KernelArgs a, const tl_layout_header* h, hipStream_t st)
     int tg = std::min(Shape::kTiles, (budget - 1024) / per_tile);
     tg = std::min(tg, (int)(Shape::kStreamCap / (chunk_bytes * a.block_set)));
     tg = std::max(1, std::min(std::min(tg, a.T), 255));
+    tg = std::max(1, std::min(tg, env_int("TL_TILE_GROUP", tg)));
     tg = (int)ceil_div(a.T, ceil_div(a.T, tg));  // same number of groups, evened out
     a.tiles_per_group = tg;
     a.xs_bytes = tg * tile_bytes;

@@ -43,12 +43,12 @@ class RMSNorm(nn.Module):
 
 class DecoderLayer(nn.Module):
     """One block.  q, k and v share their input, so their weights are packed side by side as one
-    [hidden, 3 * hidden] matrix and run as one product; gate and up stay two blobs (the fused
-    gate/up/SiLU kernel takes them as a pair)."""
+    [hidden, 3 * hidden] matrix and run as one product; likewise gate and up as one
+    [hidden, 2 * intermediate] matrix."""
 
     def __init__(self, config, linears, dtype, device):
         super().__init__()
-        self.qkv_proj, self.o_proj, self.gate_proj, self.up_proj, self.down_proj = linears
+        self.qkv_proj, self.o_proj, self.gate_up_proj, self.down_proj = linears
         self.input_layernorm = RMSNorm(config.hidden_size, config.rms_norm_eps, dtype, device)
         self.post_attention_layernorm = RMSNorm(config.hidden_size, config.rms_norm_eps, dtype, device)
 
@@ -58,7 +58,7 @@ class TernaryLlamaDecoder(nn.Module):
     every linear layer, the output head included.  Each linear carries a per-output-channel scale
     1 / sqrt(non-zeros per column) so that activations keep their magnitude through the stack."""
 
-    LINEARS = ("qkv", "o", "gate", "up", "down")
+    LINEARS = ("qkv", "o", "gate_up", "down")
 
     def __init__(self, config, *, seed=0, device="cuda", dtype=torch.float16, max_seq_len=None, pack_threads=8):
         super().__init__()
@@ -73,7 +73,7 @@ class TernaryLlamaDecoder(nn.Module):
         gen.manual_seed(seed)
         draw_dev = dev if dev.type == "cuda" else "cpu"
 
-        shapes = {"qkv": (H, 3 * H), "o": (H, H), "gate": (H, I), "up": (H, I), "down": (I, H)}
+        shapes = {"qkv": (H, 3 * H), "o": (H, H), "gate_up": (H, 2 * I), "down": (I, H)}
 
         def make(shape):
             K, N = shape
@@ -118,6 +118,8 @@ class TernaryLlamaDecoder(nn.Module):
         self.register_buffer("rope_sin", ang.sin().to(dev, dtype), False)
         self._cache = None
         self._graph = None
+        # single-token steps use the library's rotary / cache / attention kernels; False keeps them on torch operators
+        self.native_decode = config.head_dim in (64, 128, 256) and self.max_seq_len * 4 <= 120 * 1024
 
     # -- pieces ------------------------------------------------------------------------------
     @staticmethod
@@ -127,9 +129,9 @@ class TernaryLlamaDecoder(nn.Module):
         return x * cos + rot * sin
 
     def _mlp(self, layer, x2):
-        h = ops.mlp_gate_up(layer.gate_proj.device_weight(), layer.up_proj.device_weight(), x2, layer.gate_proj.w_scale,
-                            layer.up_proj.w_scale)
-        return layer.down_proj(h)
+        gu = layer.gate_up_proj(x2)
+        inter = self.config.intermediate_size
+        return layer.down_proj(torch.nn.functional.silu(gu[:, :inter]) * gu[:, inter:])
 
     def allocate_cache(self, batch):
         c = self.config
@@ -183,6 +185,8 @@ class TernaryLlamaDecoder(nn.Module):
     def _decode_step(self, token, pos, mask):
         """token: LongTensor [B]; pos: LongTensor [1] (cache slot to write); mask: bool [1, 1, 1, max_seq]
         true on slots <= pos.  Static shapes throughout.  Returns logits [B, vocab]."""
+        if self.native_decode:
+            return self._decode_step_native(token, pos)
         x = self.embed_tokens[token][:, None]
         cos, sin = self.rope_cos.index_select(0, pos), self.rope_sin.index_select(0, pos)
 
@@ -192,6 +196,23 @@ class TernaryLlamaDecoder(nn.Module):
         for li, layer in enumerate(self.layers):
             x = self._block(layer, li, x, cos, sin, pos, attend)
         return self.lm_head(self.norm(x[:, 0]))
+
+    def _decode_step_native(self, token, pos):
+        """The decode step with rotary embedding + cache update and the attention over the cache as one
+        library kernel each (activations stay [B, hidden] throughout)."""
+        c = self.config
+        x = self.embed_tokens[token]
+        B = x.shape[0]
+        q = torch.empty((B, c.num_attention_heads, c.head_dim), dtype=x.dtype, device=x.device)
+        for li, layer in enumerate(self.layers):
+            h = layer.input_layernorm(x)
+            qkv = layer.qkv_proj(h)
+            ops.rope_cache_update(qkv, self.rope_cos, self.rope_sin, pos, q, self._cache[li, 0], self._cache[li, 1])
+            a = ops.decode_attention(q, self._cache[li, 0], self._cache[li, 1], pos)
+            x = x + layer.o_proj(a)
+            h = layer.post_attention_layernorm(x)
+            x = x + self._mlp(layer, h)
+        return self.lm_head(self.norm(x))
 
     @torch.no_grad()
     def generate(self, tokens, new_tokens, use_graph=True):

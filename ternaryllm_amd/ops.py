@@ -179,3 +179,45 @@ def spmm_time(weight, x, iters, scale=None, out_dtype=None, x_layout=_lib.TL_X_R
                                      ctypes.byref(ms))
     _lib.check(rc)
     return ms.value, y
+
+
+def rope_cache_update(qkv, cos_table, sin_table, pos, q_out, k_cache, v_cache):
+    """Rotates q and k of one token per batch row and writes k, v into row `pos` of the caches.
+    qkv: [B, 3 * heads * head_dim] (q | k | v); cos/sin tables: [max_seq, head_dim]; pos: int64 device
+    tensor with one element; q_out: [B, heads, head_dim]; caches: [B, heads, max_seq, head_dim]."""
+    B, heads, max_seq, hd = k_cache.shape
+    for t in (qkv, cos_table, sin_table, q_out, k_cache, v_cache):
+        if not t.is_contiguous() or t.dtype != qkv.dtype or t.device != qkv.device:
+            raise ValueError("tensors must be contiguous, of one dtype, on one device")
+    if qkv.numel() != B * 3 * heads * hd or q_out.numel() != B * heads * hd or v_cache.shape != k_cache.shape:
+        raise ValueError("shapes of qkv, q_out and the caches do not agree")
+    if cos_table.shape != (max_seq, hd) or sin_table.shape != (max_seq, hd):
+        raise ValueError("rotary tables must be [max_seq, head_dim]")
+    if pos.dtype != torch.int64 or pos.numel() != 1 or pos.device != qkv.device:
+        raise ValueError("pos must be a one-element int64 tensor on the same device")
+    with torch.cuda.device(qkv.device):
+        rc = _lib.lib().tl_rope_cache_update(qkv.data_ptr(), _code(qkv.dtype, "qkv"), B, heads, hd, cos_table.data_ptr(),
+                                             sin_table.data_ptr(), pos.data_ptr(), q_out.data_ptr(), k_cache.data_ptr(),
+                                             v_cache.data_ptr(), max_seq, _stream_ptr(qkv.device))
+    _lib.check(rc)
+    return q_out
+
+
+def decode_attention(q, k_cache, v_cache, pos, out=None):
+    """Attention of one query per (batch row, head) over cache rows [0, pos].  q: [B, heads, head_dim];
+    caches: [B, heads, max_seq, head_dim]; pos: one-element int64 device tensor.  Returns [B, heads * head_dim]."""
+    B, heads, max_seq, hd = k_cache.shape
+    if out is None:
+        out = torch.empty((B, heads * hd), dtype=q.dtype, device=q.device)
+    for t in (q, k_cache, v_cache, out):
+        if not t.is_contiguous() or t.dtype != q.dtype or t.device != q.device:
+            raise ValueError("tensors must be contiguous, of one dtype, on one device")
+    if q.numel() != B * heads * hd or out.numel() != B * heads * hd or v_cache.shape != k_cache.shape:
+        raise ValueError("shapes of q, out and the caches do not agree")
+    if pos.dtype != torch.int64 or pos.numel() != 1 or pos.device != q.device:
+        raise ValueError("pos must be a one-element int64 tensor on the same device")
+    with torch.cuda.device(q.device):
+        rc = _lib.lib().tl_decode_attention(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), _code(q.dtype, "q"), B, heads, hd,
+                                            max_seq, pos.data_ptr(), out.data_ptr(), _stream_ptr(q.device))
+    _lib.check(rc)
+    return out

@@ -38,7 +38,9 @@ def _reference_logits(model, tokens):
         a = (att @ v).transpose(1, 2).reshape(B, S, H)
         x = x + lin(layer.o_proj, a)
         h = norm(layer.post_attention_layernorm, x)
-        x = x + lin(layer.down_proj, torch.nn.functional.silu(lin(layer.gate_proj, h)) * lin(layer.up_proj, h))
+        gu = lin(layer.gate_up_proj, h)
+        inter = c.intermediate_size
+        x = x + lin(layer.down_proj, torch.nn.functional.silu(gu[..., :inter]) * gu[..., inter:])
     return lin(model.lm_head, norm(model.norm, x))
 
 
@@ -66,6 +68,64 @@ def test_prefill_and_decode_match_fp32_reference(tiny, cuda):
         st["mask"].copy_((torch.arange(tiny.max_seq_len, device=cuda) <= S + j)[None, None, None])
         logits = tiny._decode_step(st["token"], st["pos"], st["mask"]).float()
         assert (logits - ref[:, S + j]).abs().max().item() <= 2e-2 * scale
+
+
+def test_native_decode_step_matches_torch_operators(tiny, cuda):
+    """The library's rotary / cache / attention kernels against the same step on torch operators."""
+    g = torch.Generator().manual_seed(6)
+    B, S = 3, 33
+    tokens = torch.randint(0, tiny.config.vocab_size, (B, S + 2), generator=g).to(cuda)
+    assert tiny.native_decode
+    outs = {}
+    for native in (False, True):
+        tiny.native_decode = native
+        tiny.prefill(tokens[:, :S])
+        st = tiny._decode_state(B)
+        logits = []
+        for j in range(2):
+            st["token"].copy_(tokens[:, S + j])
+            st["pos"].fill_(S + j)
+            st["mask"].copy_((torch.arange(tiny.max_seq_len, device=cuda) <= S + j)[None, None, None])
+            logits.append(tiny._decode_step(st["token"], st["pos"], st["mask"]).float())
+        outs[native] = (torch.stack(logits), tiny._cache[:, :, :, :, : S + 2].float().clone())
+    tiny.native_decode = True
+    scale = outs[False][0].abs().max().item()
+    assert (outs[True][0] - outs[False][0]).abs().max().item() <= 1e-2 * scale
+    assert (outs[True][1] - outs[False][1]).abs().max().item() <= 2e-3 * outs[False][1].abs().max().item()
+
+
+def test_decode_kernels_against_fp32(cuda):
+    """tl_rope_cache_update and tl_decode_attention alone, fp16 and fp32, against a float64 restatement."""
+    from ternaryllm_amd import ops
+    g = torch.Generator().manual_seed(9)
+    for dtype, tol in ((torch.float32, 2e-5), (torch.float16, 3e-3)):
+        for hd in (64, 128):
+            B, H, S = 2, 3, 77
+            pos = 41
+            qkv = torch.randn((B, 3 * H * hd), generator=g).to(dtype).to(cuda)
+            inv = 1.0 / (10000.0 ** (torch.arange(0, hd, 2, dtype=torch.float64) / hd))
+            ang = torch.arange(S, dtype=torch.float64)[:, None] * inv[None, :]
+            ang = torch.cat([ang, ang], -1)
+            cos, sin = ang.cos().to(dtype).to(cuda), ang.sin().to(dtype).to(cuda)
+            kc = torch.randn((B, H, S, hd), generator=g).to(dtype).to(cuda)
+            vc = torch.randn((B, H, S, hd), generator=g).to(dtype).to(cuda)
+            kc0, vc0 = kc.clone(), vc.clone()
+            q = torch.empty((B, H, hd), dtype=dtype, device=cuda)
+            p = torch.tensor([pos], dtype=torch.long, device=cuda)
+            ops.rope_cache_update(qkv, cos, sin, p, q, kc, vc)
+            x = qkv.double().view(B, 3, H, hd)
+            c64, s64 = cos[pos].double(), sin[pos].double()
+            rot = lambda t: t * c64 + torch.cat([-t[..., hd // 2:], t[..., : hd // 2]], -1) * s64
+            assert (q.double() - rot(x[:, 0])).abs().max().item() <= tol * 4
+            assert (kc[:, :, pos].double() - rot(x[:, 1])).abs().max().item() <= tol * 4
+            assert torch.equal(vc[:, :, pos], qkv.view(B, 3, H, hd)[:, 2])
+            keep = torch.ones(S, dtype=torch.bool, device=cuda)
+            keep[pos] = False
+            assert torch.equal(kc[:, :, keep], kc0[:, :, keep]) and torch.equal(vc[:, :, keep], vc0[:, :, keep])
+            out = ops.decode_attention(q, kc, vc, p)
+            sc = (q.double()[:, :, None, :] * kc.double()[:, :, : pos + 1]).sum(-1) / hd ** 0.5
+            ref = (sc.softmax(-1)[..., None] * vc.double()[:, :, : pos + 1]).sum(2).reshape(B, H * hd)
+            assert (out.double() - ref).abs().max().item() <= tol * 4
 
 
 def test_graph_replay_equals_eager_decode(tiny, cuda):
