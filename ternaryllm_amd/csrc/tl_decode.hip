@@ -54,10 +54,10 @@ __global__ __launch_bounds__(256) void tl_rope_cache(const T* __restrict__ qkv, 
 
 // One workgroup per (batch row, head): scores of the query against cache rows [0, pos], softmax in
 // fp32, weighted sum of the value rows.  out is [batch][heads * head_dim], the layout the output
-// projection multiplies.  Threads first own cache rows (a score is one thread's dot product over the
-// row's contiguous head_dim values), then own output dimensions (reads of a value row are contiguous
-// across threads); the two halves of the workgroup split the rows of the second pass.
-constexpr int kAttnThreads = 256;
+// projection multiplies.  A cache row is read as 16-byte pieces by CPR neighbouring lanes, and the
+// workgroup's 1024 threads work on 1024 / CPR rows side by side, so that with a few hundred rows
+// every thread has only a handful of independent loads to wait for.
+constexpr int kAttnThreads = 1024;
 
 template <typename T, int HD>
 __global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restrict__ q, const T* __restrict__ k_cache,
@@ -65,10 +65,13 @@ __global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restri
                                                                T* __restrict__ out, int heads, long long max_seq, float scale)
 {
     extern __shared__ __align__(16) unsigned char smem[];
-    float* score = reinterpret_cast<float*>(smem);            // [n]
-    __shared__ float qs[HD];
+    constexpr int VE = 16 / (int)sizeof(T);   // values per 16-byte piece
+    constexpr int CPR = HD / VE;              // lanes per cache row
+    constexpr int RG = kAttnThreads / CPR;    // rows in flight
+    static_assert(CPR <= 64 && (CPR & (CPR - 1)) == 0, "a row's lanes must sit in one wave");
+    float* score = reinterpret_cast<float*>(smem);  // [n]
     __shared__ float red[kAttnThreads / 64];
-    __shared__ float partial[kAttnThreads / HD > 0 ? kAttnThreads / HD : 1][HD];
+    __shared__ float partial[RG][HD + 1];
     const int tid = threadIdx.x;
     const long long bh = blockIdx.x;
     long long n = *pos_p + 1;  // valid rows
@@ -76,33 +79,40 @@ __global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restri
     if (n < 1) n = 1;
     const T* kc = k_cache + (size_t)bh * max_seq * HD;
     const T* vc = v_cache + (size_t)bh * max_seq * HD;
-    for (int d = tid; d < HD; d += kAttnThreads) qs[d] = to_f(q[(size_t)bh * HD + d]) * scale;
-    __syncthreads();
+    const int c = tid % CPR, rg = tid / CPR;
 
-    float local_max = -INFINITY;
-    for (long long j = tid; j < n; j += kAttnThreads) {
-        const T* row = kc + (size_t)j * HD;
-        float acc = 0.f;
+    auto unpack = [](const uint4& v, float (&f)[VE]) {
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
         if constexpr (sizeof(T) == 2) {
-#pragma unroll 4
-            for (int d = 0; d < HD; d += 8) {
-                const uint4 v = *reinterpret_cast<const uint4*>(row + d);
-                const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    acc = fmaf(__half2float(__ushort_as_half((unsigned short)(w[e] & 0xffffu))), qs[d + 2 * e], acc);
-                    acc = fmaf(__half2float(__ushort_as_half((unsigned short)(w[e] >> 16))), qs[d + 2 * e + 1], acc);
-                }
+            for (int e = 0; e < 4; ++e) {
+                f[2 * e] = __half2float(__ushort_as_half((unsigned short)(w[e] & 0xffffu)));
+                f[2 * e + 1] = __half2float(__ushort_as_half((unsigned short)(w[e] >> 16)));
             }
         } else {
-#pragma unroll 4
-            for (int d = 0; d < HD; d += 4) {
-                const float4 v = *reinterpret_cast<const float4*>(row + d);
-                acc = fmaf(v.x, qs[d], acc); acc = fmaf(v.y, qs[d + 1], acc);
-                acc = fmaf(v.z, qs[d + 2], acc); acc = fmaf(v.w, qs[d + 3], acc);
-            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) f[e] = __uint_as_float(w[e]);
         }
-        score[j] = acc;
+    };
+
+    float qv[VE];
+    {
+        float f[VE];
+        unpack(*reinterpret_cast<const uint4*>(q + (size_t)bh * HD + c * VE), f);
+#pragma unroll
+        for (int e = 0; e < VE; ++e) qv[e] = f[e] * scale;
+    }
+    float local_max = -INFINITY;
+#pragma unroll 4
+    for (long long j = rg; j < n; j += RG) {
+        float f[VE];
+        unpack(*reinterpret_cast<const uint4*>(kc + (size_t)j * HD + c * VE), f);
+        float acc = 0.f;
+#pragma unroll
+        for (int e = 0; e < VE; ++e) acc = fmaf(f[e], qv[e], acc);
+#pragma unroll
+        for (int off = CPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+        if (c == 0) score[j] = acc;
         local_max = fmaxf(local_max, acc);
     }
     // block maximum
@@ -128,22 +138,27 @@ __global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restri
 #pragma unroll
     for (int w = 0; w < kAttnThreads / 64; ++w) total += red[w];
 
-    // weighted sum of value rows: thread -> (slice of the rows, output dimension)
-    constexpr int SLICES = kAttnThreads / HD > 0 ? kAttnThreads / HD : 1;
-    const int d = tid % HD, slice = tid / HD;
-    if (slice < SLICES) {
-        float acc = 0.f;
-        for (long long j = slice; j < n; j += SLICES) acc = fmaf(score[j], to_f(vc[(size_t)j * HD + d]), acc);
-        partial[slice][d] = acc;
+    // weighted sum of value rows: every row group folds its rows, then the groups are added up
+    float acc[VE];
+#pragma unroll
+    for (int e = 0; e < VE; ++e) acc[e] = 0.f;
+#pragma unroll 4
+    for (long long j = rg; j < n; j += RG) {
+        float f[VE];
+        unpack(*reinterpret_cast<const uint4*>(vc + (size_t)j * HD + c * VE), f);
+        const float p = score[j];
+#pragma unroll
+        for (int e = 0; e < VE; ++e) acc[e] = fmaf(p, f[e], acc[e]);
     }
+#pragma unroll
+    for (int e = 0; e < VE; ++e) partial[rg][c * VE + e] = acc[e];
     __syncthreads();
     if (tid < HD) {
-        float acc = 0.f;
-#pragma unroll
-        for (int s = 0; s < SLICES; ++s) acc += partial[s][tid];
+        float sum = 0.f;
+        for (int g = 0; g < RG; ++g) sum += partial[g][tid];
         const long long b = bh / heads;
         const int h = (int)(bh % heads);
-        out[((size_t)b * heads + h) * HD + tid] = from_f<T>(acc / total);
+        out[((size_t)b * heads + h) * HD + tid] = from_f<T>(sum / total);
     }
 }
 
@@ -163,21 +178,32 @@ int launched()
     return TL_OK;
 }
 
+template <typename T, int HD>
+int attn_launch(dim3 grid, size_t lds, hipStream_t st, const void* q, const void* k, const void* v, const long long* pos, void* out,
+                int heads, long long max_seq, float scale)
+{
+    auto kernel = tl_decode_attn<T, HD>;
+    static bool raised = false;  // per instantiation; a repeated or racing call is harmless
+    if (!raised) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 120 * 1024);
+        if (e != hipSuccess) return fail(TL_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+        raised = true;
+    }
+    hipLaunchKernelGGL(kernel, grid, dim3(kAttnThreads), lds, st, static_cast<const T*>(q), static_cast<const T*>(k),
+                       static_cast<const T*>(v), pos, static_cast<T*>(out), heads, max_seq, scale);
+    return TL_OK;
+}
+
 template <typename T>
 int attn_dispatch(int head_dim, dim3 grid, size_t lds, hipStream_t st, const void* q, const void* k, const void* v,
                   const long long* pos, void* out, int heads, long long max_seq, float scale)
 {
-    const T* qq = static_cast<const T*>(q);
-    const T* kk = static_cast<const T*>(k);
-    const T* vv = static_cast<const T*>(v);
-    T* oo = static_cast<T*>(out);
     switch (head_dim) {
-        case 64: hipLaunchKernelGGL((tl_decode_attn<T, 64>), grid, dim3(kAttnThreads), lds, st, qq, kk, vv, pos, oo, heads, max_seq, scale); break;
-        case 128: hipLaunchKernelGGL((tl_decode_attn<T, 128>), grid, dim3(kAttnThreads), lds, st, qq, kk, vv, pos, oo, heads, max_seq, scale); break;
-        case 256: hipLaunchKernelGGL((tl_decode_attn<T, 256>), grid, dim3(kAttnThreads), lds, st, qq, kk, vv, pos, oo, heads, max_seq, scale); break;
+        case 64: return attn_launch<T, 64>(grid, lds, st, q, k, v, pos, out, heads, max_seq, scale);
+        case 128: return attn_launch<T, 128>(grid, lds, st, q, k, v, pos, out, heads, max_seq, scale);
+        case 256: return attn_launch<T, 256>(grid, lds, st, q, k, v, pos, out, heads, max_seq, scale);
         default: return fail(TL_ERR_UNSUPPORTED, "head_dim=%d (64, 128 or 256 supported)", head_dim);
     }
-    return TL_OK;
 }
 
 }  // namespace
@@ -212,8 +238,8 @@ extern "C" int tl_decode_attention(const void* q, const void* k_cache, const voi
     if (!q || !k_cache || !v_cache || !out) return fail(TL_ERR_ARG, "device pointer is null");
     const size_t lds = (size_t)max_seq * sizeof(float);
     if (lds > 120 * 1024) return fail(TL_ERR_UNSUPPORTED, "max_seq=%lld: the scores of one head must fit 120 KB of LDS", (long long)max_seq);
-    const int es = dtype == TL_F16 ? 2 : 4;
-    if (reinterpret_cast<uintptr_t>(k_cache) % 16 || ((int64_t)head_dim * es) % 16) return fail(TL_ERR_ALIGN, "cache rows must be 16-byte aligned");
+    if (reinterpret_cast<uintptr_t>(k_cache) % 16 || reinterpret_cast<uintptr_t>(v_cache) % 16 || reinterpret_cast<uintptr_t>(q) % 16)
+        return fail(TL_ERR_ALIGN, "q and the caches must be 16-byte aligned");
     dim3 grid((unsigned)(batch * heads));
     hipStream_t st = static_cast<hipStream_t>(stream);
     const long long* pos = reinterpret_cast<const long long*>(pos_dev);
