@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the ternary SpMM hot path on one MI355X.
 
-Workload (BASELINE.json, "Llama-2-7B ternary MLP block", the shape the metric is quoted on):
+Workload (the Llama-2-7B ternary MLP block, the shape the headline metric is quoted on):
 one step = one ternary SpMM of the gate projection: 8 x 128 = 1024 token rows, fp16 activations
 ~N(0,1), W ternary [4096 -> 11008] at 80 % sparsity (10 % +1, 10 % -1, i.i.d., seeded), per-output
 fp16 scale ~U(0.5, 1.5), fp32 accumulation, fp16 output.  Inputs are resident in HBM before the
