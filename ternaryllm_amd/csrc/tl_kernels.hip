@@ -59,6 +59,8 @@ struct KernelArgs {
     int x_mode;           // small-M kernel: how activations are staged (kStageElements / kStageSlotVectors / kStageRowVectors)
     unsigned tile_magic;  // ceil(2^32 / tile_rows): k / tile_rows == (k * tile_magic) >> 32 for every k < 2^24
     long long x_sm, x_sk; // small-M kernel: element strides of the activations along M and along K
+    long long split_steps;  // row kernel: 0, or the number of (output tile, K tile) steps shared out among the workgroups
+    float* partial;         // row kernel: partial sums of output tiles whose K tiles were shared out
     float one;  // 1.0f, passed in so that the fp16 -> fp32 accumulate stays a single mixed-precision fma
 };
 
@@ -491,24 +493,25 @@ struct RunFetcher {
 #pragma unroll
         for (int ch = 0; ch < NPRE; ++ch) r.pre[ch] = stream[r.base + ch * 64 + lane];
     }
-    __device__ __forceinline__ void prime(const WeightPtrs& w, int T, int n0, int lane_)
+    // Makes tile t0 the next one advance() hands out.
+    __device__ __forceinline__ void prime(const WeightPtrs& w, int T, int n0, int lane_, int t0)
     {
         chunkstart = as_const(w.chunkstart) + (size_t)(n0 / TL_BLOCK_COLUMNS) * T;
         stream_c = as_const(w.stream);
         stream = w.stream;
         sub = n0 % TL_BLOCK_COLUMNS;
         lane = lane_;
-        const uint32_t chunk0 = chunkstart[0];
+        const uint32_t chunk0 = chunkstart[t0];
         descriptors(nxt.d, chunk0);
         indices(nxt, chunk0);
         chunk1 = chunk2 = 0;
 #pragma unroll
         for (int c = 0; c < C; ++c) d1[c] = 0;
-        if (T > 1) {
-            chunk1 = chunkstart[1];
+        if (t0 + 1 < T) {
+            chunk1 = chunkstart[t0 + 1];
             descriptors(d1, chunk1);
         }
-        if (T > 2) chunk2 = chunkstart[2];
+        if (t0 + 2 < T) chunk2 = chunkstart[t0 + 2];
     }
     // Call at the start of tile t: afterwards `cur` holds tile t's runs.
     __device__ __forceinline__ void advance(int t, int T)
@@ -700,6 +703,44 @@ __device__ __forceinline__ void regs_to_lds(const u32x4 (&pf)[PER], unsigned cha
     }
 }
 
+// Scale, optional SiLU gate, and store of one workgroup's output tile.  Row of accumulator j of a lane:
+// fp16: rows {2l, 2l + 1} and {128 + 2l, 129 + 2l} of the row tile; fp32: rows l and 64 + l.
+template <typename XT, int R, int C, bool GATED>
+__device__ __forceinline__ void rows_store(const KernelArgs& a, int m0, int n0, int lane, const float (&acc)[C][R],
+                                           const float (&acc2)[GATED ? C : 1][R])
+{
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+        const int n = n0 + c;
+        if (n >= a.N) continue;
+        const float s = load_scale(a.w0.scale, a.scale_f16, n);
+        const float s2 = GATED ? load_scale(a.w1.scale, a.scale_f16, n) : 1.0f;
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+            const int m = m0 + (sizeof(XT) == 2 ? (j >> 1) * 128 + 2 * lane + (j & 1) : j * 64 + lane);
+            if (m >= a.M) continue;
+            float v = acc[c][j] * s;
+            if constexpr (GATED) v = silu(v) * (acc2[GATED ? c : 0][j] * s2);
+            store_out(a.Y, a.y_f16, (long long)m * a.ldy + n, v);
+        }
+    }
+}
+
+// Where the partial sums of a workgroup that owns only some tiles of an output tile go: slot
+// (workgroup, which) of the partial area, one float per (wave, column, accumulator, lane), the gate's
+// set first and the up projection's after it.
+template <int R, int C, int WAVES, bool GATED>
+__device__ __forceinline__ float* partial_slot(float* base, int lin, int which)
+{
+    constexpr size_t kSet = (size_t)WAVES * C * R * 64;
+    return base + ((size_t)lin * 2 + which) * kSet * (GATED ? 2 : 1);
+}
+
+// The step list is (output tile, K tile) in output-tile-major order; workgroup `lin` of G owns steps
+// [lin * S / G, (lin + 1) * S / G).
+__device__ __host__ inline long long split_begin(long long lin, long long S, long long G) { return lin * S / G; }
+__device__ __host__ inline long long split_owner(long long step, long long S, long long G) { return ((step + 1) * G - 1) / S; }
+
 template <typename XT, int R, int C, int WAVES, bool GATED>
 __global__ __launch_bounds__(WAVES * 64) void tl_spmm_rows(KernelArgs a)
 {
@@ -718,14 +759,97 @@ __global__ __launch_bounds__(WAVES * 64) void tl_spmm_rows(KernelArgs a)
     // the same few row tiles of the activations instead of all of them.
     const int n_col_tiles = (a.N + WAVES * C - 1) / (WAVES * C);
     const int total = (int)gridDim.x;
-    int id = (int)blockIdx.x;
+    int lin = (int)blockIdx.x;
     const int per_xcd = total / 8;
-    if (id < per_xcd * 8) id = (id & 7) * per_xcd + (id >> 3);
-    const int m0 = (id / n_col_tiles) * MTILE;
-    const int n0 = (id % n_col_tiles) * (WAVES * C) + wave * C;
-    const bool wave_live = n0 < a.N;                                       // uniform; then n0 lies inside a stored column block
+    if (lin < per_xcd * 8) lin = (lin & 7) * per_xcd + (lin >> 3);
+    // One workgroup per output tile, or (a.split_steps != 0) an equal share of all (output tile, K tile)
+    // steps per workgroup: then a workgroup may own only the last tiles of its first output tile and only
+    // the first tiles of its last one, and leaves partial sums for tl_rows_fixup to add up.
+    long long step = a.split_steps ? split_begin(lin, a.split_steps, total) : (long long)lin * a.T;
+    const long long step_end = a.split_steps ? split_begin(lin + 1, a.split_steps, total) : step + a.T;
     const unsigned char* __restrict__ XTr = static_cast<const unsigned char*>(a.X);  // [K][ldx] of XT, m contiguous
+    const int last_rows = a.K - (a.T - 1) * a.tile_rows;
+    const size_t tile_stride = (size_t)a.tile_rows * a.ldx * sizeof(XT);  // bytes between the first rows of two tiles
 
+    // Slot 255 is what padding bytes address: zero it once, staging never writes it.
+    for (int e = threadIdx.x; e < MTILE; e += NT) tile[kSentinel * MTILE + e] = XT(0.0f);
+
+    while (step < step_end) {
+        const int unit = (int)(step / a.T);
+        const int t0 = (int)(step - (long long)unit * a.T);
+        const int t1 = (int)min((long long)a.T, t0 + (step_end - step));
+        const int m0 = (unit / n_col_tiles) * MTILE;
+        const int n0 = (unit % n_col_tiles) * (WAVES * C) + wave * C;
+        const bool wave_live = n0 < a.N;                                   // uniform; then n0 lies inside a stored column block
+
+        float acc[C][R];
+        float acc2[GATED ? C : 1][R];
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+#pragma unroll
+            for (int j = 0; j < R; ++j) {
+                acc[c][j] = 0.f;
+                if (GATED) acc2[GATED ? c : 0][j] = 0.f;
+            }
+
+        // The next activation tile travels global -> registers while the current one is consumed.
+        u32x4 pf[PER];
+        RunFetcher<C> f0, f1;
+        if (wave_live) {
+            f0.prime(a.w0, a.T, n0, lane, t0);
+            if constexpr (GATED) f1.prime(a.w1, a.T, n0, lane, t0);
+        }
+        uint32_t voff[PER];
+        const unsigned char* __restrict__ col0 = XTr + (size_t)m0 * sizeof(XT);
+        stage_offsets<XT, CHUNKS, NT, PER>(voff, a, t0 + 1 < a.T ? a.tile_rows : last_rows);
+        tile_to_regs<PER>(pf, col0 + (size_t)t0 * tile_stride, voff);
+        for (int t = t0; t < t1; ++t) {
+            __syncthreads();  // every wave is done with the previous tile
+            regs_to_lds<CHUNKS, NT, PER>(pf, smem, a, t);
+            __syncthreads();
+            if (t + 1 < t1) {
+                if (t + 2 == a.T && last_rows != a.tile_rows) stage_offsets<XT, CHUNKS, NT, PER>(voff, a, last_rows);
+                tile_to_regs<PER>(pf, col0 + (size_t)(t + 1) * tile_stride, voff);
+            }
+            if (wave_live) {
+                f0.advance(t, a.T);
+                if constexpr (GATED) f1.advance(t, a.T);
+                rows_consume<XT, R, C>(acc, f0.cur, a.w0.stream, lane, a.one);
+                if constexpr (GATED) rows_consume<XT, R, C>(acc2, f1.cur, a.w1.stream, lane, a.one);
+            }
+        }
+
+        if (t0 == 0 && t1 == a.T) {
+            rows_store<XT, R, C, GATED>(a, m0, n0, lane, acc, acc2);
+        } else {
+            float* part = partial_slot<R, C, WAVES, GATED>(a.partial, lin, t0 > 0 ? 0 : 1);
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+#pragma unroll
+                for (int j = 0; j < R; ++j) {
+                    part[((size_t)(wave * C + c) * R + j) * 64 + lane] = acc[c][j];
+                    if constexpr (GATED) part[((size_t)(WAVES * C + wave * C + c) * R + j) * 64 + lane] = acc2[GATED ? c : 0][j];
+                }
+        }
+        step += t1 - t0;
+    }
+}
+
+// One workgroup per output tile: when its K tiles were shared out among several workgroups of
+// tl_spmm_rows, adds up their partial sums and finishes the tile; otherwise there is nothing to do.
+template <typename XT, int R, int C, int WAVES, bool GATED>
+__global__ __launch_bounds__(WAVES * 64) void tl_rows_fixup(KernelArgs a, int G)
+{
+    constexpr int MTILE = 64 * R;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int n_col_tiles = (a.N + WAVES * C - 1) / (WAVES * C);
+    const int unit = (int)blockIdx.x;
+    const long long first = (long long)unit * a.T, last = first + a.T - 1;
+    const int lin_a = (int)split_owner(first, a.split_steps, G), lin_b = (int)split_owner(last, a.split_steps, G);
+    if (lin_a == lin_b) return;  // one workgroup had all of it and has stored it
+    const int m0 = (unit / n_col_tiles) * MTILE;
+    const int n0 = (unit % n_col_tiles) * (WAVES * C) + wave * C;
     float acc[C][R];
     float acc2[GATED ? C : 1][R];
 #pragma unroll
@@ -735,55 +859,20 @@ __global__ __launch_bounds__(WAVES * 64) void tl_spmm_rows(KernelArgs a)
             acc[c][j] = 0.f;
             if (GATED) acc2[GATED ? c : 0][j] = 0.f;
         }
-
-    // Slot 255 is what padding bytes address: zero it once, staging never writes it.
-    for (int e = threadIdx.x; e < MTILE; e += NT) tile[kSentinel * MTILE + e] = XT(0.0f);
-
-    // The next activation tile travels global -> registers while the current one is consumed.
-    u32x4 pf[PER];
-    RunFetcher<C> f0, f1;
-    if (wave_live) {
-        f0.prime(a.w0, a.T, n0, lane);
-        if constexpr (GATED) f1.prime(a.w1, a.T, n0, lane);
-    }
-    uint32_t voff[PER];
-    const int last_rows = a.K - (a.T - 1) * a.tile_rows;
-    const size_t tile_stride = (size_t)a.tile_rows * a.ldx * sizeof(XT);  // bytes between the first rows of two tiles
-    const unsigned char* __restrict__ col0 = XTr + (size_t)m0 * sizeof(XT);
-    stage_offsets<XT, CHUNKS, NT, PER>(voff, a, a.T > 1 ? a.tile_rows : last_rows);
-    tile_to_regs<PER>(pf, col0, voff);
-    for (int t = 0; t < a.T; ++t) {
-        __syncthreads();  // every wave is done with the previous tile
-        regs_to_lds<CHUNKS, NT, PER>(pf, smem, a, t);
-        __syncthreads();
-        if (t + 1 < a.T) {
-            if (t + 2 == a.T && last_rows != a.tile_rows) stage_offsets<XT, CHUNKS, NT, PER>(voff, a, last_rows);
-            tile_to_regs<PER>(pf, col0 + (size_t)(t + 1) * tile_stride, voff);
-        }
-        if (wave_live) {
-            f0.advance(t, a.T);
-            if constexpr (GATED) f1.advance(t, a.T);
-            rows_consume<XT, R, C>(acc, f0.cur, a.w0.stream, lane, a.one);
-            if constexpr (GATED) rows_consume<XT, R, C>(acc2, f1.cur, a.w1.stream, lane, a.one);
-        }
-    }
-
+    for (int lin = lin_a; lin <= lin_b; ++lin) {
+        const long long begin = split_begin(lin, a.split_steps, G);
+        if (split_begin(lin + 1, a.split_steps, G) == begin) continue;  // fewer steps than workgroups: this one had none
+        // a workgroup whose share starts inside this tile left its sums in slot 0, one that started earlier in slot 1
+        const float* part = partial_slot<R, C, WAVES, GATED>(a.partial, lin, begin > first ? 0 : 1);
 #pragma unroll
-    for (int c = 0; c < C; ++c) {
-        const int n = n0 + c;
-        if (n >= a.N) continue;
-        const float s = load_scale(a.w0.scale, a.scale_f16, n);
-        const float s2 = GATED ? load_scale(a.w1.scale, a.scale_f16, n) : 1.0f;
+        for (int c = 0; c < C; ++c)
 #pragma unroll
-        for (int j = 0; j < R; ++j) {
-            // rows of a lane: see rows_add4
-            const int m = m0 + (sizeof(XT) == 2 ? (j >> 1) * 128 + 2 * lane + (j & 1) : j * 64 + lane);
-            if (m >= a.M) continue;
-            float v = acc[c][j] * s;
-            if constexpr (GATED) v = silu(v) * (acc2[GATED ? c : 0][j] * s2);
-            store_out(a.Y, a.y_f16, (long long)m * a.ldy + n, v);
-        }
+            for (int j = 0; j < R; ++j) {
+                acc[c][j] += part[((size_t)(wave * C + c) * R + j) * 64 + lane];
+                if constexpr (GATED) acc2[GATED ? c : 0][j] += part[((size_t)(WAVES * C + wave * C + c) * R + j) * 64 + lane];
+            }
     }
+    if (n0 < a.N) rows_store<XT, R, C, GATED>(a, m0, n0, lane, acc, acc2);
 }
 
 // ---------------------------------------------------------------------------
@@ -988,8 +1077,12 @@ int launch_small(KernelArgs a, const tl_layout_header* h, int x_dtype, void* wor
     }
 }
 
+// Bytes of partial sums the row kernel may leave when K tiles are shared out (both weight sets of the
+// fused gate/up kernel): two slots per workgroup of a one-workgroup-per-compute-unit launch.
+constexpr int64_t kRowsPartialBytes = (int64_t)kComputeUnits * 2 * 2 * kRowsWaves * kRowsCols * 4 * 64 * sizeof(float);
+
 template <typename XT, int R, bool GATED>
-int launch_rows_t(const KernelArgs& a, hipStream_t st)
+int launch_rows_t(KernelArgs a, void* partial, int64_t partial_bytes, hipStream_t st)
 {
     constexpr int MTILE = 64 * R;
     const size_t lds = (size_t)kTileSlots * MTILE * sizeof(XT);
@@ -1003,8 +1096,24 @@ int launch_rows_t(const KernelArgs& a, hipStream_t st)
         if (int rc = raise_lds_limit(kernel, lds)) return rc;
         raised = true;
     }
-    dim3 grid((unsigned)(ceil_div(a.N, kRowsWaves * kRowsCols) * ceil_div(a.M, MTILE)));  // 1-D: the kernel maps ids to tiles
-    hipLaunchKernelGGL(kernel, grid, dim3(kRowsWaves * 64), lds, st, a);
+    const int64_t units = ceil_div(a.N, kRowsWaves * kRowsCols) * ceil_div(a.M, MTILE);
+    // One workgroup per output tile leaves compute units idle in the last round (or all along, with
+    // fewer tiles than units).  When that costs more than a few percent, one workgroup per compute
+    // unit takes an equal share of all (output tile, K tile) steps instead, and a second small launch
+    // adds up the partial sums of the tiles that were shared out.
+    const int64_t rounds = ceil_div(units, kComputeUnits);
+    const bool uneven = (double)rounds * kComputeUnits > 1.06 * (double)units;
+    const bool want = env_int("TL_ROWS_SPLIT", uneven && units * a.T >= 4 * kComputeUnits ? 1 : 0) != 0;
+    if (want && partial && partial_bytes >= kRowsPartialBytes && reinterpret_cast<uintptr_t>(partial) % 16 == 0 && a.T >= 2) {
+        a.split_steps = units * a.T;
+        a.partial = static_cast<float*>(partial);
+        hipLaunchKernelGGL(kernel, dim3(kComputeUnits), dim3(kRowsWaves * 64), lds, st, a);
+        hipLaunchKernelGGL((tl_rows_fixup<XT, R, kRowsCols, kRowsWaves, GATED>), dim3((unsigned)units), dim3(kRowsWaves * 64), 0, st, a,
+                           kComputeUnits);
+        return TL_OK;
+    }
+    a.split_steps = 0;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)units), dim3(kRowsWaves * 64), lds, st, a);  // 1-D: the kernel maps ids to tiles
     return TL_OK;
 }
 
@@ -1016,9 +1125,16 @@ inline bool rows_needs_relayout(const void* X, int x_dtype, int x_layout, int64_
     return x_layout != TL_X_K_MAJOR || ldx % mtile != 0 || ldx < round_up(M, mtile) || reinterpret_cast<uintptr_t>(X) % 16 != 0;
 }
 
-// Runs the re-layout pre-pass into `workspace` when needed, then the row-parallel kernel.
+inline int64_t rows_relayout_bytes(int64_t K, int64_t M, int x_dtype)
+{
+    return round_up(K * round_up(M, rows_mtile(x_dtype)) * (x_dtype == TL_F16 ? 2 : 4), 256);
+}
+
+// Runs the re-layout pre-pass into `workspace` when needed, then the row-parallel kernel.  The
+// workspace holds the K-major image of the activations first, the partial sums behind it.
 int launch_rows(KernelArgs a, int x_dtype, void* workspace, int64_t workspace_bytes, bool gated, hipStream_t st)
 {
+    const int64_t image = rows_relayout_bytes(a.K, a.M, x_dtype);
     if (rows_needs_relayout(a.X, x_dtype, a.x_kmajor ? TL_X_K_MAJOR : TL_X_ROW_MAJOR, a.ldx, a.M)) {
         const int mtile = rows_mtile(x_dtype);
         const int64_t ldm = round_up(a.M, mtile);
@@ -1040,8 +1156,17 @@ int launch_rows(KernelArgs a, int x_dtype, void* workspace, int64_t workspace_by
     // the kernel keeps a thread's byte offsets inside one activation tile in 32 bits
     if ((int64_t)kTileSlots * a.ldx * (x_dtype == TL_F16 ? 2 : 4) >= (int64_t)1 << 32)
         return fail(TL_ERR_ARG, "activation leading dimension %lld is too large for one call; split the rows", (long long)a.ldx);
-    if (x_dtype == TL_F16) return gated ? launch_rows_t<__half, 4, true>(a, st) : launch_rows_t<__half, 4, false>(a, st);
-    return gated ? launch_rows_t<float, 2, true>(a, st) : launch_rows_t<float, 2, false>(a, st);
+    // room for partial sums, if the caller's workspace reaches that far (without it every output tile
+    // simply gets a workgroup of its own)
+    void* partial = nullptr;
+    int64_t partial_bytes = 0;
+    if (workspace && workspace_bytes >= image + kRowsPartialBytes) {
+        partial = static_cast<unsigned char*>(workspace) + image;
+        partial_bytes = workspace_bytes - image;
+    }
+    if (x_dtype == TL_F16)
+        return gated ? launch_rows_t<__half, 4, true>(a, partial, partial_bytes, st) : launch_rows_t<__half, 4, false>(a, partial, partial_bytes, st);
+    return gated ? launch_rows_t<float, 2, true>(a, partial, partial_bytes, st) : launch_rows_t<float, 2, false>(a, partial, partial_bytes, st);
 }
 
 int finish_launch()
@@ -1081,7 +1206,8 @@ extern "C" int tl_spmm_workspace(const tl_layout_header* header, int64_t M, int 
         *workspace_bytes = small_kmajor_bytes(header, M, x_dtype);
         return TL_OK;
     }
-    *workspace_bytes = (int64_t)header->inners * round_up(M, rows_mtile(x_dtype)) * (x_dtype == TL_F16 ? 2 : 4);
+    // the K-major image of the activations, then room for the partial sums of shared-out output tiles
+    *workspace_bytes = rows_relayout_bytes(header->inners, M, x_dtype) + kRowsPartialBytes;
     return TL_OK;
 }
 

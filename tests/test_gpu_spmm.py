@@ -141,3 +141,33 @@ def test_small_m_activation_layouts(cuda, oracle, M, dtype):
             print(f"case M={M} K={K} dtype={dtype} {name}", flush=True)
             y = ops.spmm(dw, xin, x_layout=layout).float().cpu().numpy()
             assert np.array_equal(y.astype(np.float64), ref), (M, K, name)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_rows_kernel_with_and_without_shared_out_tiles(cuda, oracle, dtype, monkeypatch):
+    """The row-parallel kernel in both launch modes (one workgroup per output tile; K tiles shared out
+    among one workgroup per compute unit, partial sums added by the fix-up launch), plain and fused."""
+    from ternaryllm_amd import ops
+    from ternaryllm_amd.packing import PackedWeight
+    for M, K, N in ((70, 1300, 200), (520, 2100, 130), (1100, 777, 330)):
+        wg = ternary_weight(K, N, 0.75, 51 + M)
+        wu = ternary_weight(K, N, 0.75, 52 + M)
+        dg, du = ops.DeviceWeight(PackedWeight.from_dense(wg), cuda), ops.DeviceWeight(PackedWeight.from_dense(wu), cuda)
+        x = activations(M, K, 53 + M, dtype, integer=True)
+        ref = oracle.fast_product(x.double().numpy(), wg)
+        xf = activations(M, K, 54 + M, dtype)
+        sg = (0.5 + torch.rand(N, generator=torch.Generator().manual_seed(55))).to(dtype)
+        g = (xf.double() @ torch.from_numpy(wg).double()) * sg.double()
+        u = (xf.double() @ torch.from_numpy(wu).double()) * sg.double()
+        ref_fused = (torch.nn.functional.silu(g) * u).numpy()
+        fused = {}
+        for mode in ("0", "1"):
+            monkeypatch.setenv("TL_ROWS_SPLIT", mode)
+            print(f"case M={M} K={K} N={N} dtype={dtype} split={mode}", flush=True)
+            y = ops.spmm(dg, x.to(cuda), out_dtype=torch.float32).cpu().numpy()
+            assert np.array_equal(y.astype(np.float64), ref), (M, K, N, mode)
+            h = ops.mlp_gate_up(dg, du, xf.to(cuda), sg.to(cuda), sg.to(cuda), out_dtype=torch.float32).cpu().numpy()
+            scale = np.abs(ref_fused).max()
+            assert np.abs(h - ref_fused).max() <= (FP16_TOL if dtype == torch.float16 else 1e-4) * scale, (M, K, N, mode)
+            fused[mode] = h
+        monkeypatch.delenv("TL_ROWS_SPLIT")
