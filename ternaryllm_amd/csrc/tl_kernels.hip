@@ -158,7 +158,7 @@ struct BlockShape {
                                        : (NT * 256 > kSmallStreamBytes ? kSmallStreamBytes : NT * 256)) / 16 * 16;
     static constexpr int kVectors = (kStreamCap / 16 + NT - 1) / NT;
     static constexpr int kSlotRegs = MT >= 8 ? MT * ES / 4 : MT;
-    static constexpr int kSlots = 72 / kSlotRegs > 16 ? 16 : 72 / kSlotRegs;  // per thread
+    static constexpr int kSlots = MT <= 4 ? 16 : (kSlotRegs >= 16 ? 4 : 36 / kSlotRegs);  // per thread
     static constexpr int kTiles = kSlots * NT / kTileSlots;                   // tiles per group at most
 };
 
@@ -174,8 +174,11 @@ struct BlockShape {
 // one dword (four row indices) per lane and pass; an index is one LDS read and MT accumulating
 // ops.  The LPC partial sums of a column are folded with cross-lane shuffles.  No workgroup depends
 // on another.
+// Four waves per SIMD (two workgroups per compute unit) is what the LDS budget plans for: the register
+// allocation is held to that, except for 16 fp32 rows per slot, whose gathers alone need 64 registers.
 template <int MT, bool XF16>
-__global__ __launch_bounds__(kBlockThreads) void tl_spmm_block(KernelArgs a)
+__global__ __launch_bounds__(kBlockThreads) __attribute__((amdgpu_waves_per_eu(MT * (XF16 ? 2 : 4) >= 64 ? 2 : 4, MT * (XF16 ? 2 : 4) >= 64 ? 2 : 4)))
+void tl_spmm_block(KernelArgs a)
 {
     extern __shared__ __align__(16) unsigned char lds[];
     using XT = typename std::conditional<XF16, __half, float>::type;
