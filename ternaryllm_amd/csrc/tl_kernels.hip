@@ -371,7 +371,7 @@ void tl_spmm_block(KernelArgs a)
 #pragma unroll
     for (int m = 0; m < MT; ++m) acc[m] = 0.f;
 
-    constexpr int TU = MT <= 2 ? 4 : (MT <= 8 ? 2 : 1);  // tiles of one lane whose LDS reads are issued together
+    constexpr int TU = MT <= 8 ? 2 : 1;  // tiles of one lane whose LDS reads are issued together
     prefetch(0, min(TG, a.T));
     for (int t = 0; t < a.T; t += TG) {
         const int nt = min(TG, a.T - t);
