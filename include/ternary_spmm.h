@@ -245,6 +245,17 @@ int tl_decode_attention(const void* q, const void* k_cache, const void* v_cache,
                         int64_t batch, int heads, int head_dim, int64_t max_seq,
                         const int64_t* pos_dev, void* out, void* stream);
 
+/* x_out = x + y, h_out = RMSNorm(x_out) * weight, row by row ([rows][width], one dtype): the residual
+ * add of a decoder layer fused with the normalisation that follows (the reference leaves both to the
+ * Hugging Face Llama it patches, TernaryLLM/TernaryLlama.py:69-75).  y may be NULL: plain RMSNorm of x,
+ * x_out then optional. */
+int tl_add_rmsnorm(const void* x, const void* y, const void* weight, int dtype, int64_t rows, int width,
+                   float eps, void* x_out, void* h_out, void* stream);
+
+/* out[rows][width] = silu(gate_up[:, :width]) * gate_up[:, width:] for gate_up [rows][2 * width]: the
+ * gate of LlamaTernaryMLP (TernaryLLM/TernaryMLP.py:33-35) on a side-by-side gate | up product. */
+int tl_silu_mul(const void* gate_up, int dtype, int64_t rows, int width, void* out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

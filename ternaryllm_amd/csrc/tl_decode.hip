@@ -162,6 +162,107 @@ __global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restri
     }
 }
 
+// x_out = x + y (rounded to T), h_out = x_out / rms(x_out) * weight: the residual add and the RMSNorm that
+// follows it in a decoder layer, one workgroup per row.  y may be null (plain RMSNorm of x).
+template <typename T>
+__global__ __launch_bounds__(256) void tl_add_rmsnorm_k(const T* __restrict__ x, const T* __restrict__ y, const T* __restrict__ weight,
+                                                        T* __restrict__ x_out, T* __restrict__ h_out, int width, float eps)
+{
+    __shared__ float red[4];
+    const size_t row = (size_t)blockIdx.x * width;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < width; i += 256) {
+        float v = to_f(x[row + i]);
+        if (y) v = to_f(from_f<T>(v + to_f(y[row + i])));
+        if (x_out) x_out[row + i] = from_f<T>(v);
+        ss = fmaf(v, v, ss);
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    const float inv = rsqrtf((red[0] + red[1] + red[2] + red[3]) / (float)width + eps);
+    for (int i = threadIdx.x; i < width; i += 256) {
+        float v = to_f(x[row + i]);
+        if (y) v = to_f(from_f<T>(v + to_f(y[row + i])));
+        h_out[row + i] = from_f<T>(v * inv * to_f(weight[i]));
+    }
+}
+
+// The same for rows that are whole 16-byte vectors and at most 4 vectors per thread of a 512-thread
+// workgroup: every value is read once, all loads of a thread are in flight together.
+template <typename T>
+__global__ __launch_bounds__(512) void tl_add_rmsnorm_vec(const T* __restrict__ x, const T* __restrict__ y, const T* __restrict__ weight,
+                                                          T* __restrict__ x_out, T* __restrict__ h_out, int width, float eps)
+{
+    constexpr int VE = 16 / (int)sizeof(T);
+    constexpr int NV = 4;
+    __shared__ float red[8];
+    const size_t row = (size_t)blockIdx.x * width;
+    const int nvec = width / VE;
+    uint4 xv[NV], yv[NV], wv[NV];
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        const int v = min((int)threadIdx.x + k * 512, nvec - 1);
+        xv[k] = *reinterpret_cast<const uint4*>(x + row + (size_t)v * VE);
+        if (y) yv[k] = *reinterpret_cast<const uint4*>(y + row + (size_t)v * VE);
+        wv[k] = *reinterpret_cast<const uint4*>(weight + (size_t)v * VE);
+    }
+    float val[NV][VE];
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        const T* xe = reinterpret_cast<const T*>(&xv[k]);
+        const T* ye = reinterpret_cast<const T*>(&yv[k]);
+        const bool live = (int)threadIdx.x + k * 512 < nvec;
+#pragma unroll
+        for (int e = 0; e < VE; ++e) {
+            float v = to_f(xe[e]);
+            if (y) v = to_f(from_f<T>(v + to_f(ye[e])));
+            val[k][e] = v;
+            if (live) ss = fmaf(v, v, ss);
+        }
+        if (live && x_out) {
+            uint4 o;
+            T* oe = reinterpret_cast<T*>(&o);
+#pragma unroll
+            for (int e = 0; e < VE; ++e) oe[e] = from_f<T>(val[k][e]);
+            *reinterpret_cast<uint4*>(x_out + row + ((size_t)threadIdx.x + k * 512) * VE) = o;
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    float total = 0.f;
+#pragma unroll
+    for (int w = 0; w < 8; ++w) total += red[w];
+    const float inv = rsqrtf(total / (float)width + eps);
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        if ((int)threadIdx.x + k * 512 < nvec) {
+            const T* we = reinterpret_cast<const T*>(&wv[k]);
+            uint4 o;
+            T* oe = reinterpret_cast<T*>(&o);
+#pragma unroll
+            for (int e = 0; e < VE; ++e) oe[e] = from_f<T>(val[k][e] * inv * to_f(we[e]));
+            *reinterpret_cast<uint4*>(h_out + row + ((size_t)threadIdx.x + k * 512) * VE) = o;
+        }
+    }
+}
+
+// out[r][i] = silu(gu[r][i]) * gu[r][width + i]: the gate of the MLP on the side-by-side gate | up product.
+template <typename T>
+__global__ __launch_bounds__(256) void tl_silu_mul_k(const T* __restrict__ gu, T* __restrict__ out, long long rows, int width)
+{
+    const long long i = blockIdx.x * 256ll + threadIdx.x;
+    if (i >= rows * width) return;
+    const long long r = i / width;
+    const int c = (int)(i - r * width);
+    const float g = to_f(gu[(size_t)r * 2 * width + c]), u = to_f(gu[(size_t)r * 2 * width + width + c]);
+    out[i] = from_f<T>(to_f(from_f<T>(g / (1.0f + __expf(-g)))) * u);  // the SiLU is rounded to T before the product, as two separate operators would
+}
+
 int check_common(int dtype, int64_t batch, int heads, int head_dim, int64_t max_seq, const void* pos_dev)
 {
     if (dtype != TL_F16 && dtype != TL_F32) return fail(TL_ERR_DTYPE, "dtype code %d unknown", dtype);
@@ -248,5 +349,53 @@ extern "C" int tl_decode_attention(const void* q, const void* k_cache, const voi
     if (dtype == TL_F16) rc = attn_dispatch<__half>(head_dim, grid, lds, st, q, k_cache, v_cache, pos, out, heads, (long long)max_seq, scale);
     else rc = attn_dispatch<float>(head_dim, grid, lds, st, q, k_cache, v_cache, pos, out, heads, (long long)max_seq, scale);
     if (rc) return rc;
+    return launched();
+}
+
+extern "C" int tl_add_rmsnorm(const void* x, const void* y, const void* weight, int dtype, int64_t rows, int width, float eps,
+                              void* x_out, void* h_out, void* stream)
+{
+    if (dtype != TL_F16 && dtype != TL_F32) return fail(TL_ERR_DTYPE, "dtype code %d unknown", dtype);
+    if (!x || !weight || !h_out) return fail(TL_ERR_ARG, "device pointer is null");
+    if (rows <= 0 || width <= 0 || rows > (1ll << 30)) return fail(TL_ERR_SHAPE, "rows and width must be positive");
+    if (y && !x_out) return fail(TL_ERR_ARG, "x_out is needed when y is given");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int ve = dtype == TL_F16 ? 8 : 4;
+    auto aligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+    if (width % ve == 0 && width / ve <= 4 * 512 && aligned(x) && aligned(y) && aligned(weight) && aligned(x_out) && aligned(h_out)) {
+        if (dtype == TL_F16)
+            hipLaunchKernelGGL(tl_add_rmsnorm_vec<__half>, dim3((unsigned)rows), dim3(512), 0, st, static_cast<const __half*>(x),
+                               static_cast<const __half*>(y), static_cast<const __half*>(weight), static_cast<__half*>(x_out),
+                               static_cast<__half*>(h_out), width, eps);
+        else
+            hipLaunchKernelGGL(tl_add_rmsnorm_vec<float>, dim3((unsigned)rows), dim3(512), 0, st, static_cast<const float*>(x),
+                               static_cast<const float*>(y), static_cast<const float*>(weight), static_cast<float*>(x_out),
+                               static_cast<float*>(h_out), width, eps);
+        return launched();
+    }
+    if (dtype == TL_F16)
+        hipLaunchKernelGGL(tl_add_rmsnorm_k<__half>, dim3((unsigned)rows), dim3(256), 0, st, static_cast<const __half*>(x),
+                           static_cast<const __half*>(y), static_cast<const __half*>(weight), static_cast<__half*>(x_out),
+                           static_cast<__half*>(h_out), width, eps);
+    else
+        hipLaunchKernelGGL(tl_add_rmsnorm_k<float>, dim3((unsigned)rows), dim3(256), 0, st, static_cast<const float*>(x),
+                           static_cast<const float*>(y), static_cast<const float*>(weight), static_cast<float*>(x_out),
+                           static_cast<float*>(h_out), width, eps);
+    return launched();
+}
+
+extern "C" int tl_silu_mul(const void* gate_up, int dtype, int64_t rows, int width, void* out, void* stream)
+{
+    if (dtype != TL_F16 && dtype != TL_F32) return fail(TL_ERR_DTYPE, "dtype code %d unknown", dtype);
+    if (!gate_up || !out) return fail(TL_ERR_ARG, "device pointer is null");
+    if (rows <= 0 || width <= 0 || rows * width > (1ll << 40)) return fail(TL_ERR_SHAPE, "rows and width must be positive");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const unsigned blocks = (unsigned)ceil_div(rows * width, 256);
+    if (dtype == TL_F16)
+        hipLaunchKernelGGL(tl_silu_mul_k<__half>, dim3(blocks), dim3(256), 0, st, static_cast<const __half*>(gate_up), static_cast<__half*>(out),
+                           (long long)rows, width);
+    else
+        hipLaunchKernelGGL(tl_silu_mul_k<float>, dim3(blocks), dim3(256), 0, st, static_cast<const float*>(gate_up), static_cast<float*>(out),
+                           (long long)rows, width);
     return launched();
 }

@@ -204,15 +204,17 @@ class TernaryLlamaDecoder(nn.Module):
         x = self.embed_tokens[token]
         B = x.shape[0]
         q = torch.empty((B, c.num_attention_heads, c.head_dim), dtype=x.dtype, device=x.device)
+        eps = c.rms_norm_eps
+        _, h = ops.add_rmsnorm(x, None, self.layers[0].input_layernorm.weight, eps)
         for li, layer in enumerate(self.layers):
-            h = layer.input_layernorm(x)
             qkv = layer.qkv_proj(h)
             ops.rope_cache_update(qkv, self.rope_cos, self.rope_sin, pos, q, self._cache[li, 0], self._cache[li, 1])
             a = ops.decode_attention(q, self._cache[li, 0], self._cache[li, 1], pos)
-            x = x + layer.o_proj(a)
-            h = layer.post_attention_layernorm(x)
-            x = x + self._mlp(layer, h)
-        return self.lm_head(self.norm(x))
+            x, h = ops.add_rmsnorm(x, layer.o_proj(a), layer.post_attention_layernorm.weight, eps)
+            y = layer.down_proj(ops.silu_mul(layer.gate_up_proj(h)))
+            nxt = self.layers[li + 1].input_layernorm.weight if li + 1 < len(self.layers) else self.norm.weight
+            x, h = ops.add_rmsnorm(x, y, nxt, eps)  # the residual add, and the norm the next layer (or the head) starts with
+        return self.lm_head(h)
 
     @torch.no_grad()
     def generate(self, tokens, new_tokens, use_graph=True):

@@ -221,3 +221,34 @@ def decode_attention(q, k_cache, v_cache, pos, out=None):
                                             max_seq, pos.data_ptr(), out.data_ptr(), _stream_ptr(q.device))
     _lib.check(rc)
     return out
+
+
+def add_rmsnorm(x, y, weight, eps):
+    """(x + y, rmsnorm(x + y) * weight) for [rows, width] tensors of one dtype; y may be None (then the
+    first result is x itself)."""
+    if x.dim() != 2 or not x.is_contiguous() or weight.numel() != x.shape[1] or not weight.is_contiguous():
+        raise ValueError("x must be a contiguous [rows, width] tensor and weight [width]")
+    if y is not None and (y.shape != x.shape or y.dtype != x.dtype or not y.is_contiguous()):
+        raise ValueError("y must match x")
+    if weight.dtype != x.dtype:
+        raise ValueError("weight must have x's dtype")
+    h = torch.empty_like(x)
+    x_out = torch.empty_like(x) if y is not None else x
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().tl_add_rmsnorm(x.data_ptr(), y.data_ptr() if y is not None else None, weight.data_ptr(), _code(x.dtype, "x"),
+                                       x.shape[0], x.shape[1], float(eps), x_out.data_ptr() if y is not None else None, h.data_ptr(),
+                                       _stream_ptr(x.device))
+    _lib.check(rc)
+    return x_out, h
+
+
+def silu_mul(gate_up):
+    """silu(gate_up[:, :w]) * gate_up[:, w:] for a contiguous [rows, 2 * w] tensor."""
+    if gate_up.dim() != 2 or not gate_up.is_contiguous() or gate_up.shape[1] % 2:
+        raise ValueError("gate_up must be a contiguous [rows, 2 * width] tensor")
+    rows, w = gate_up.shape[0], gate_up.shape[1] // 2
+    out = torch.empty((rows, w), dtype=gate_up.dtype, device=gate_up.device)
+    with torch.cuda.device(gate_up.device):
+        rc = _lib.lib().tl_silu_mul(gate_up.data_ptr(), _code(gate_up.dtype, "gate_up"), rows, w, out.data_ptr(), _stream_ptr(gate_up.device))
+    _lib.check(rc)
+    return out

@@ -128,6 +128,28 @@ def test_decode_kernels_against_fp32(cuda):
             assert (out.double() - ref).abs().max().item() <= tol * 4
 
 
+def test_add_rmsnorm_and_silu_mul(cuda):
+    from ternaryllm_amd import ops
+    g = torch.Generator().manual_seed(10)
+    for dtype, tol in ((torch.float32, 1e-5), (torch.float16, 2e-3)):
+        for rows, width in ((1, 4096), (5, 300), (16, 11008)):
+            x = torch.randn((rows, width), generator=g).to(dtype).to(cuda)
+            y = torch.randn((rows, width), generator=g).to(dtype).to(cuda)
+            w = (1 + 0.1 * torch.randn(width, generator=g)).to(dtype).to(cuda)
+            xs, h = ops.add_rmsnorm(x, y, w, 1e-5)
+            assert torch.equal(xs, x + y)
+            ref = xs.double() * torch.rsqrt(xs.double().pow(2).mean(-1, keepdim=True) + 1e-5) * w.double()
+            assert (h.double() - ref).abs().max().item() <= tol * ref.abs().max().item()
+            x0, h0 = ops.add_rmsnorm(x, None, w, 1e-5)
+            assert x0 is x
+            ref0 = x.double() * torch.rsqrt(x.double().pow(2).mean(-1, keepdim=True) + 1e-5) * w.double()
+            assert (h0.double() - ref0).abs().max().item() <= tol * ref0.abs().max().item()
+            gu = torch.randn((rows, 2 * width), generator=g).to(dtype).to(cuda)
+            out = ops.silu_mul(gu)
+            refs = torch.nn.functional.silu(gu[:, :width].double()) * gu[:, width:].double()
+            assert (out.double() - refs).abs().max().item() <= tol * refs.abs().max().item()
+
+
 def test_graph_replay_equals_eager_decode(tiny, cuda):
     g = torch.Generator().manual_seed(4)
     tokens = torch.randint(0, tiny.config.vocab_size, (3, 40), generator=g).to(cuda)
