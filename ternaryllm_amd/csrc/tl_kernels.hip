@@ -4,17 +4,20 @@
 // Two kernels replace the reference's pair
 // (ternaryLLM_GPU/csrc/ter_spmm_kernel.cuh:24-78 SpMV, :106-308 SpMM):
 //
-//   tl_spmm_block  M <= 48 (decode and small batches).  A workgroup owns a block of 16
-//                  columns over all of K and streams its chunks and the matching
-//                  activation rows through LDS; LPC lanes share a column and split
-//                  each run, four dwords = sixteen 8-bit row indices per lane; every
-//                  index is one LDS gather and one fp32 add per activation row; the
-//                  LPC partial sums are folded with cross-lane shuffles.
+//   tl_spmm_block  M <= 48 (decode and small batches).  A workgroup owns 1, 2 or 4 blocks of 16
+//                  columns over all of K and streams their chunks and the matching
+//                  activation rows through LDS (activations in their own type, [slot][row]);
+//                  the lanes that share a column split each run, one dword = four 8-bit row
+//                  indices per lane and pass; every index is one LDS read of the slot's rows
+//                  and one accumulating op per row; the partial sums of a column are folded
+//                  with cross-lane shuffles.
 //   tl_spmm_rows   larger M (prefill).  Lanes own activation rows, a wave owns C
 //                  output columns, so an index is wave-uniform: it is read through
 //                  the scalar path once and serves 64*R rows; the activation tile
 //                  is staged in LDS as [slot][row] so the gather of a wave is one
-//                  contiguous, conflict-free LDS read.
+//                  contiguous, conflict-free LDS read.  Output tiles go one per workgroup,
+//                  or their K tiles are shared out evenly among one workgroup per compute
+//                  unit, with tl_rows_fixup adding up the partial sums.
 //
 // Only additions and subtractions touch the data; fp32 accumulation throughout.
 #include <hip/hip_fp16.h>
