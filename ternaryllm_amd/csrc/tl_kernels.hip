@@ -711,24 +711,72 @@ __device__ __forceinline__ void regs_to_lds(const u32x4 (&pf)[PER], unsigned cha
 
 // Scale, optional SiLU gate, and store of one workgroup's output tile.  Row of accumulator j of a lane:
 // fp16: rows {2l, 2l + 1} and {128 + 2l, 129 + 2l} of the row tile; fp32: rows l and 64 + l.
-template <typename XT, int R, int C, bool GATED>
-__device__ __forceinline__ void rows_store(const KernelArgs& a, int m0, int n0, int lane, const float (&acc)[C][R],
-                                           const float (&acc2)[GATED ? C : 1][R])
+// A lane holds C neighbouring columns of R scattered rows, so storing from the accumulators would write
+// 2- or 4-byte pieces a row apart.  The tile therefore goes through LDS (the activation tile's space,
+// free by now): lanes write their C columns of a row side by side, then the workgroup stores whole
+// rows of WAVES * C columns, 8 or 16 bytes per lane.  Output tiles that the matrix edge cuts, or whose
+// rows are not aligned for that, are stored value by value.
+template <typename XT, int R, int C, int WAVES, bool GATED>
+__device__ __forceinline__ void rows_store(const KernelArgs& a, int m0, int n_wg, int wave, int lane, const float (&acc)[C][R],
+                                           const float (&acc2)[GATED ? C : 1][R], unsigned char* smem)
 {
+    constexpr int MTILE = 64 * R;
+    constexpr int COLS = WAVES * C;
+    static_assert(C == 4, "the staged store moves four columns per lane");
+    const int n0 = n_wg + wave * C;
+    float v[C][R];
 #pragma unroll
     for (int c = 0; c < C; ++c) {
-        const int n = n0 + c;
-        if (n >= a.N) continue;
+        const int n = min(n0 + c, a.N - 1);
         const float s = load_scale(a.w0.scale, a.scale_f16, n);
         const float s2 = GATED ? load_scale(a.w1.scale, a.scale_f16, n) : 1.0f;
 #pragma unroll
         for (int j = 0; j < R; ++j) {
-            const int m = m0 + (sizeof(XT) == 2 ? (j >> 1) * 128 + 2 * lane + (j & 1) : j * 64 + lane);
-            if (m >= a.M) continue;
-            float v = acc[c][j] * s;
-            if constexpr (GATED) v = silu(v) * (acc2[GATED ? c : 0][j] * s2);
-            store_out(a.Y, a.y_f16, (long long)m * a.ldy + n, v);
+            v[c][j] = acc[c][j] * s;
+            if constexpr (GATED) v[c][j] = silu(v[c][j]) * (acc2[GATED ? c : 0][j] * s2);
         }
+    }
+    const int es = a.y_f16 ? 2 : 4;
+    const bool whole = n_wg + COLS <= a.N && (a.ldy * es) % (4 * es) == 0 &&
+                       (reinterpret_cast<uintptr_t>(a.Y) + (size_t)n_wg * es) % (4 * es) == 0;  // uniform over the workgroup
+    if (!whole) {
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const int n = n0 + c;
+            if (n >= a.N) continue;
+#pragma unroll
+            for (int j = 0; j < R; ++j) {
+                const int m = m0 + (sizeof(XT) == 2 ? (j >> 1) * 128 + 2 * lane + (j & 1) : j * 64 + lane);
+                if (m < a.M) store_out(a.Y, a.y_f16, (long long)m * a.ldy + n, v[c][j]);
+            }
+        }
+        return;
+    }
+    const int stride = COLS * es + 4 * es;  // bytes per staged row: the pad keeps the lanes' writes off one bank
+    __syncthreads();                        // every wave is done reading the activation tile
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+        const int r = sizeof(XT) == 2 ? (j >> 1) * 128 + 2 * lane + (j & 1) : j * 64 + lane;
+        unsigned char* dst = smem + (size_t)r * stride + (size_t)wave * C * es;
+        if (a.y_f16) {
+            const __half2 lo = __floats2half2_rn(v[0][j], v[1][j]), hi = __floats2half2_rn(v[2][j], v[3][j]);
+            *reinterpret_cast<uint2*>(dst) = make_uint2(*reinterpret_cast<const uint32_t*>(&lo), *reinterpret_cast<const uint32_t*>(&hi));
+        } else {
+            *reinterpret_cast<float4*>(dst) = make_float4(v[0][j], v[1][j], v[2][j], v[3][j]);
+        }
+    }
+    __syncthreads();
+    constexpr int LANES_PER_ROW = COLS / 4;             // each lane moves four columns
+    constexpr int ROWS_PER_PASS = WAVES * 64 / LANES_PER_ROW;
+    const int q = (int)threadIdx.x % LANES_PER_ROW, r0 = (int)threadIdx.x / LANES_PER_ROW;
+#pragma unroll
+    for (int r = r0; r < MTILE; r += ROWS_PER_PASS) {
+        const int m = m0 + r;
+        if (m >= a.M) continue;
+        const unsigned char* src = smem + (size_t)r * stride + (size_t)q * 4 * es;
+        unsigned char* out = static_cast<unsigned char*>(a.Y) + ((size_t)m * a.ldy + n_wg + q * 4) * es;
+        if (a.y_f16) *reinterpret_cast<uint2*>(out) = *reinterpret_cast<const uint2*>(src);
+        else *reinterpret_cast<float4*>(out) = *reinterpret_cast<const float4*>(src);
     }
 }
 
@@ -826,7 +874,7 @@ __global__ __launch_bounds__(WAVES * 64) void tl_spmm_rows(KernelArgs a)
         }
 
         if (t0 == 0 && t1 == a.T) {
-            rows_store<XT, R, C, GATED>(a, m0, n0, lane, acc, acc2);
+            rows_store<XT, R, C, WAVES, GATED>(a, m0, (unit % n_col_tiles) * (WAVES * C), wave, lane, acc, acc2, smem);
         } else {
             float* part = partial_slot<R, C, WAVES, GATED>(a.partial, lin, t0 > 0 ? 0 : 1);
 #pragma unroll
@@ -855,7 +903,6 @@ __global__ __launch_bounds__(WAVES * 64) void tl_rows_fixup(KernelArgs a, int G)
     const int lin_a = (int)split_owner(first, a.split_steps, G), lin_b = (int)split_owner(last, a.split_steps, G);
     if (lin_a == lin_b) return;  // one workgroup had all of it and has stored it
     const int m0 = (unit / n_col_tiles) * MTILE;
-    const int n0 = (unit % n_col_tiles) * (WAVES * C) + wave * C;
     float acc[C][R];
     float acc2[GATED ? C : 1][R];
 #pragma unroll
@@ -878,7 +925,8 @@ __global__ __launch_bounds__(WAVES * 64) void tl_rows_fixup(KernelArgs a, int G)
                 if constexpr (GATED) acc2[GATED ? c : 0][j] += part[((size_t)(WAVES * C + wave * C + c) * R + j) * 64 + lane];
             }
     }
-    if (n0 < a.N) rows_store<XT, R, C, GATED>(a, m0, n0, lane, acc, acc2);
+    extern __shared__ __align__(16) unsigned char smem[];
+    rows_store<XT, R, C, WAVES, GATED>(a, m0, (unit % n_col_tiles) * (WAVES * C), wave, lane, acc, acc2, smem);
 }
 
 // ---------------------------------------------------------------------------
@@ -1114,8 +1162,15 @@ int launch_rows_t(KernelArgs a, void* partial, int64_t partial_bytes, hipStream_
         a.split_steps = units * a.T;
         a.partial = static_cast<float*>(partial);
         hipLaunchKernelGGL(kernel, dim3(kComputeUnits), dim3(kRowsWaves * 64), lds, st, a);
-        hipLaunchKernelGGL((tl_rows_fixup<XT, R, kRowsCols, kRowsWaves, GATED>), dim3((unsigned)units), dim3(kRowsWaves * 64), 0, st, a,
-                           kComputeUnits);
+        // LDS of the fix-up: the staged output tile (fp32 at most, padded rows)
+        const size_t fix_lds = (size_t)MTILE * (kRowsWaves * kRowsCols * 4 + 16);
+        auto fixup = tl_rows_fixup<XT, R, kRowsCols, kRowsWaves, GATED>;
+        static bool fix_raised = false;
+        if (!fix_raised) {
+            if (int rc = raise_lds_limit(fixup, fix_lds)) return rc;
+            fix_raised = true;
+        }
+        hipLaunchKernelGGL(fixup, dim3((unsigned)units), dim3(kRowsWaves * 64), fix_lds, st, a, kComputeUnits);
         return TL_OK;
     }
     a.split_steps = 0;
