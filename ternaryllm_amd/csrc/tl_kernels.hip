@@ -722,7 +722,7 @@ __device__ __forceinline__ void rows_store(const KernelArgs& a, int m0, int n_wg
 {
     constexpr int MTILE = 64 * R;
     constexpr int COLS = WAVES * C;
-    static_assert(C == 4, "the staged store moves four columns per lane");
+    static_assert(C % 4 == 0, "the staged store moves groups of four columns per lane");
     const int n0 = n_wg + wave * C;
     float v[C][R];
 #pragma unroll
@@ -737,8 +737,11 @@ __device__ __forceinline__ void rows_store(const KernelArgs& a, int m0, int n_wg
         }
     }
     const int es = a.y_f16 ? 2 : 4;
+    const int stride = COLS * es + 4 * es;  // bytes per staged row: the pad keeps the lanes' writes off one bank
+    // uniform over the workgroup; the staged tile must stay below the sentinel slot at the end of the activation tile
     const bool whole = n_wg + COLS <= a.N && (a.ldy * es) % (4 * es) == 0 &&
-                       (reinterpret_cast<uintptr_t>(a.Y) + (size_t)n_wg * es) % (4 * es) == 0;  // uniform over the workgroup
+                       (reinterpret_cast<uintptr_t>(a.Y) + (size_t)n_wg * es) % (4 * es) == 0 &&
+                       (size_t)MTILE * stride <= (size_t)kSentinel * MTILE * sizeof(XT);
     if (!whole) {
 #pragma unroll
         for (int c = 0; c < C; ++c) {
@@ -752,17 +755,19 @@ __device__ __forceinline__ void rows_store(const KernelArgs& a, int m0, int n_wg
         }
         return;
     }
-    const int stride = COLS * es + 4 * es;  // bytes per staged row: the pad keeps the lanes' writes off one bank
-    __syncthreads();                        // every wave is done reading the activation tile
+    __syncthreads();  // every wave is done reading the activation tile
 #pragma unroll
     for (int j = 0; j < R; ++j) {
         const int r = sizeof(XT) == 2 ? (j >> 1) * 128 + 2 * lane + (j & 1) : j * 64 + lane;
-        unsigned char* dst = smem + (size_t)r * stride + (size_t)wave * C * es;
-        if (a.y_f16) {
-            const __half2 lo = __floats2half2_rn(v[0][j], v[1][j]), hi = __floats2half2_rn(v[2][j], v[3][j]);
-            *reinterpret_cast<uint2*>(dst) = make_uint2(*reinterpret_cast<const uint32_t*>(&lo), *reinterpret_cast<const uint32_t*>(&hi));
-        } else {
-            *reinterpret_cast<float4*>(dst) = make_float4(v[0][j], v[1][j], v[2][j], v[3][j]);
+#pragma unroll
+        for (int g = 0; g < C; g += 4) {
+            unsigned char* dst = smem + (size_t)r * stride + (size_t)(wave * C + g) * es;
+            if (a.y_f16) {
+                const __half2 lo = __floats2half2_rn(v[g][j], v[g + 1][j]), hi = __floats2half2_rn(v[g + 2][j], v[g + 3][j]);
+                *reinterpret_cast<uint2*>(dst) = make_uint2(*reinterpret_cast<const uint32_t*>(&lo), *reinterpret_cast<const uint32_t*>(&hi));
+            } else {
+                *reinterpret_cast<float4*>(dst) = make_float4(v[g][j], v[g + 1][j], v[g + 2][j], v[g + 3][j]);
+            }
         }
     }
     __syncthreads();
@@ -951,7 +956,8 @@ int check_dtype(int d, const char* what)
 
 constexpr int kSmallMaxM = 48;       // above this the row-parallel kernel takes over
 constexpr int kRowsWaves = 16;
-constexpr int kRowsCols = 4;
+constexpr int kRowsCols = 4;       // columns per wave of the fused gate/up kernel (two accumulator sets)
+constexpr int kRowsColsPlain = 8;  // columns per wave of the plain kernel: an activation tile then serves 128 columns
 
 inline int rows_mtile(int x_dtype) { return x_dtype == TL_F16 ? 256 : 128; }
 
@@ -1134,13 +1140,15 @@ int launch_small(KernelArgs a, const tl_layout_header* h, int x_dtype, void* wor
 // Bytes of partial sums the row kernel may leave when K tiles are shared out (both weight sets of the
 // fused gate/up kernel): two slots per workgroup of a one-workgroup-per-compute-unit launch.
 constexpr int64_t kRowsPartialBytes = (int64_t)kComputeUnits * 2 * 2 * kRowsWaves * kRowsCols * 4 * 64 * sizeof(float);
+static_assert(kRowsColsPlain == 2 * kRowsCols, "one accumulator set of the plain kernel is as large as the fused kernel's two");
 
 template <typename XT, int R, bool GATED>
 int launch_rows_t(KernelArgs a, void* partial, int64_t partial_bytes, hipStream_t st)
 {
     constexpr int MTILE = 64 * R;
     const size_t lds = (size_t)kTileSlots * MTILE * sizeof(XT);
-    auto kernel = tl_spmm_rows<XT, R, kRowsCols, kRowsWaves, GATED>;
+    constexpr int COLS = GATED ? kRowsCols : kRowsColsPlain;
+    auto kernel = tl_spmm_rows<XT, R, COLS, kRowsWaves, GATED>;
     static bool raised = false;  // per instantiation; a repeated call is harmless
     if (!raised) {
         // the kernel addresses its activation tile from LDS offset 0: it must own no static LDS
@@ -1150,7 +1158,7 @@ int launch_rows_t(KernelArgs a, void* partial, int64_t partial_bytes, hipStream_
         if (int rc = raise_lds_limit(kernel, lds)) return rc;
         raised = true;
     }
-    const int64_t units = ceil_div(a.N, kRowsWaves * kRowsCols) * ceil_div(a.M, MTILE);
+    const int64_t units = ceil_div(a.N, kRowsWaves * COLS) * ceil_div(a.M, MTILE);
     // One workgroup per output tile leaves compute units idle in the last round (or all along, with
     // fewer tiles than units).  When that costs more than a few percent, one workgroup per compute
     // unit takes an equal share of all (output tile, K tile) steps instead, and a second small launch
@@ -1163,8 +1171,8 @@ int launch_rows_t(KernelArgs a, void* partial, int64_t partial_bytes, hipStream_
         a.partial = static_cast<float*>(partial);
         hipLaunchKernelGGL(kernel, dim3(kComputeUnits), dim3(kRowsWaves * 64), lds, st, a);
         // LDS of the fix-up: the staged output tile (fp32 at most, padded rows)
-        const size_t fix_lds = (size_t)MTILE * (kRowsWaves * kRowsCols * 4 + 16);
-        auto fixup = tl_rows_fixup<XT, R, kRowsCols, kRowsWaves, GATED>;
+        const size_t fix_lds = (size_t)MTILE * (kRowsWaves * COLS * 4 + 16);
+        auto fixup = tl_rows_fixup<XT, R, COLS, kRowsWaves, GATED>;
         static bool fix_raised = false;
         if (!fix_raised) {
             if (int rc = raise_lds_limit(fixup, fix_lds)) return rc;
