@@ -63,6 +63,8 @@ struct KernelArgs {
     unsigned tile_magic;  // ceil(2^32 / tile_rows): k / tile_rows == (k * tile_magic) >> 32 for every k < 2^24
     long long x_sm, x_sk; // small-M kernel: element strides of the activations along M and along K
     long long split_steps;  // row kernel: 0, or the number of (output tile, K tile) steps shared out among the workgroups
+    int whole_units;        // row kernel: output tiles every workgroup works through on its own first
+    int split_first_unit;   // row kernel: first output tile of those whose steps are shared out
     float* partial;         // row kernel: partial sums of output tiles whose K tiles were shared out
     float one;  // 1.0f, passed in so that the fp16 -> fp32 accumulate stays a single mixed-precision fma
 };
@@ -821,11 +823,13 @@ __global__ __launch_bounds__(WAVES * 64) void tl_spmm_rows(KernelArgs a)
     int lin = (int)blockIdx.x;
     const int per_xcd = total / 8;
     if (lin < per_xcd * 8) lin = (lin & 7) * per_xcd + (lin >> 3);
-    // One workgroup per output tile, or (a.split_steps != 0) an equal share of all (output tile, K tile)
-    // steps per workgroup: then a workgroup may own only the last tiles of its first output tile and only
-    // the first tiles of its last one, and leaves partial sums for tl_rows_fixup to add up.
-    long long step = a.split_steps ? split_begin(lin, a.split_steps, total) : (long long)lin * a.T;
-    const long long step_end = a.split_steps ? split_begin(lin + 1, a.split_steps, total) : step + a.T;
+    // A workgroup first works through a.whole_units output tiles of its own.  With a.split_steps != 0 the
+    // output tiles from a.split_first_unit on are left over, and each workgroup takes an equal share of
+    // their (output tile, K tile) steps: it may then own only the last tiles of one output tile and only
+    // the first tiles of the next, and leaves partial sums for tl_rows_fixup to add up.
+    int own = 0;
+    long long step = a.split_steps ? split_begin(lin, a.split_steps, total) : 0;
+    const long long step_end = a.split_steps ? split_begin(lin + 1, a.split_steps, total) : 0;
     const unsigned char* __restrict__ XTr = static_cast<const unsigned char*>(a.X);  // [K][ldx] of XT, m contiguous
     const int last_rows = a.K - (a.T - 1) * a.tile_rows;
     const size_t tile_stride = (size_t)a.tile_rows * a.ldx * sizeof(XT);  // bytes between the first rows of two tiles
@@ -833,10 +837,20 @@ __global__ __launch_bounds__(WAVES * 64) void tl_spmm_rows(KernelArgs a)
     // Slot 255 is what padding bytes address: zero it once, staging never writes it.
     for (int e = threadIdx.x; e < MTILE; e += NT) tile[kSentinel * MTILE + e] = XT(0.0f);
 
-    while (step < step_end) {
-        const int unit = (int)(step / a.T);
-        const int t0 = (int)(step - (long long)unit * a.T);
-        const int t1 = (int)min((long long)a.T, t0 + (step_end - step));
+    while (own < a.whole_units || step < step_end) {
+        int unit, t0, t1;
+        if (own < a.whole_units) {
+            unit = lin * a.whole_units + own;
+            t0 = 0;
+            t1 = a.T;
+            ++own;
+        } else {
+            const int shared = (int)(step / a.T);
+            unit = a.split_first_unit + shared;
+            t0 = (int)(step - (long long)shared * a.T);
+            t1 = (int)min((long long)a.T, t0 + (step_end - step));
+            step += t1 - t0;
+        }
         const int m0 = (unit / n_col_tiles) * MTILE;
         const int n0 = (unit % n_col_tiles) * (WAVES * C) + wave * C;
         const bool wave_live = n0 < a.N;                                   // uniform; then n0 lies inside a stored column block
@@ -890,12 +904,11 @@ __global__ __launch_bounds__(WAVES * 64) void tl_spmm_rows(KernelArgs a)
                     if constexpr (GATED) part[((size_t)(WAVES * C + wave * C + c) * R + j) * 64 + lane] = acc2[GATED ? c : 0][j];
                 }
         }
-        step += t1 - t0;
     }
 }
 
-// One workgroup per output tile: when its K tiles were shared out among several workgroups of
-// tl_spmm_rows, adds up their partial sums and finishes the tile; otherwise there is nothing to do.
+// One workgroup per shared-out output tile: adds up the partial sums its workgroups left and finishes
+// the tile (nothing to do when the whole tile fell into one workgroup's share).
 template <typename XT, int R, int C, int WAVES, bool GATED>
 __global__ __launch_bounds__(WAVES * 64) void tl_rows_fixup(KernelArgs a, int G)
 {
@@ -903,8 +916,8 @@ __global__ __launch_bounds__(WAVES * 64) void tl_rows_fixup(KernelArgs a, int G)
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int n_col_tiles = (a.N + WAVES * C - 1) / (WAVES * C);
-    const int unit = (int)blockIdx.x;
-    const long long first = (long long)unit * a.T, last = first + a.T - 1;
+    const int unit = a.split_first_unit + (int)blockIdx.x;
+    const long long first = (long long)blockIdx.x * a.T, last = first + a.T - 1;  // in the list of shared-out steps
     const int lin_a = (int)split_owner(first, a.split_steps, G), lin_b = (int)split_owner(last, a.split_steps, G);
     if (lin_a == lin_b) return;  // one workgroup had all of it and has stored it
     const int m0 = (unit / n_col_tiles) * MTILE;
@@ -1161,13 +1174,17 @@ int launch_rows_t(KernelArgs a, void* partial, int64_t partial_bytes, hipStream_
     const int64_t units = ceil_div(a.N, kRowsWaves * COLS) * ceil_div(a.M, MTILE);
     // One workgroup per output tile leaves compute units idle in the last round (or all along, with
     // fewer tiles than units).  When that costs more than a few percent, one workgroup per compute
-    // unit takes an equal share of all (output tile, K tile) steps instead, and a second small launch
-    // adds up the partial sums of the tiles that were shared out.
+    // unit is launched instead: each works through an equal number of whole output tiles, the tiles
+    // left over are shared out by (output tile, K tile) steps, and a second small launch adds up the
+    // partial sums of those.
     const int64_t rounds = ceil_div(units, kComputeUnits);
     const bool uneven = (double)rounds * kComputeUnits > 1.06 * (double)units;
     const bool want = env_int("TL_ROWS_SPLIT", uneven && units * a.T >= 4 * kComputeUnits ? 1 : 0) != 0;
-    if (want && partial && partial_bytes >= kRowsPartialBytes && reinterpret_cast<uintptr_t>(partial) % 16 == 0 && a.T >= 2) {
-        a.split_steps = units * a.T;
+    const int64_t leftover = units % kComputeUnits;  // output tiles beyond an equal number of whole ones per workgroup
+    if (want && leftover && partial && partial_bytes >= kRowsPartialBytes && reinterpret_cast<uintptr_t>(partial) % 16 == 0 && a.T >= 2) {
+        a.whole_units = (int)(units / kComputeUnits);
+        a.split_first_unit = a.whole_units * kComputeUnits;
+        a.split_steps = leftover * a.T;
         a.partial = static_cast<float*>(partial);
         hipLaunchKernelGGL(kernel, dim3(kComputeUnits), dim3(kRowsWaves * 64), lds, st, a);
         // LDS of the fix-up: the staged output tile (fp32 at most, padded rows)
@@ -1178,10 +1195,12 @@ int launch_rows_t(KernelArgs a, void* partial, int64_t partial_bytes, hipStream_
             if (int rc = raise_lds_limit(fixup, fix_lds)) return rc;
             fix_raised = true;
         }
-        hipLaunchKernelGGL(fixup, dim3((unsigned)units), dim3(kRowsWaves * 64), fix_lds, st, a, kComputeUnits);
+        hipLaunchKernelGGL(fixup, dim3((unsigned)leftover), dim3(kRowsWaves * 64), fix_lds, st, a, kComputeUnits);
         return TL_OK;
     }
     a.split_steps = 0;
+    a.whole_units = 1;
+    a.split_first_unit = 0;
     hipLaunchKernelGGL(kernel, dim3((unsigned)units), dim3(kRowsWaves * 64), lds, st, a);  // 1-D: the kernel maps ids to tiles
     return TL_OK;
 }
