@@ -60,6 +60,7 @@ struct KernelArgs {
     int lpc_shift, lw_shift;  // small-M kernel: log2 of lanes per column and of lanes per run
     int xs_bytes, buf_bytes;  // small-M kernel: LDS for the staged activations / for the chunk copies
     int x_mode;           // small-M kernel: how activations are staged (kStageElements / kStageSlotVectors / kStageRowVectors)
+    unsigned vpt_magic;   // small-M kernel, row-copy staging: ceil(2^32 / (tile_rows / values per vector))
     unsigned tile_magic;  // ceil(2^32 / tile_rows): k / tile_rows == (k * tile_magic) >> 32 for every k < 2^24
     long long x_sm, x_sk; // small-M kernel: element strides of the activations along M and along K
     long long split_steps;  // row kernel: 0, or the number of (output tile, K tile) steps shared out among the workgroups
@@ -149,6 +150,7 @@ constexpr int kBlockThreads = 512;            // workgroup of the small-M kernel
 constexpr int kStageElements = 0;     // a thread owns slots and reads their MT values one by one (any layout)
 constexpr int kStageSlotVectors = 1;  // K-major, aligned: a thread owns slots and reads each as 16-byte vectors
 constexpr int kStageRowVectors = 2;   // row-major, aligned, MT <= 4: a thread owns 16-byte pieces of the rows
+constexpr int kStageRowCopy = 3;      // one row, aligned, tile height a whole number of vectors: tiles are copied vector by vector
 constexpr int kMaxBlockSet = 4;               // column blocks one workgroup may own
 constexpr int kSmallStreamBytes = 32 * 1024;  // LDS for the chunks of one group of tiles
 constexpr int kMaxChunkBytes = (TL_BLOCK_COLUMNS + TL_BLOCK_COLUMNS * 128) * 4;  // a chunk of all-non-zero columns
@@ -229,6 +231,22 @@ void tl_spmm_block(KernelArgs a)
                 if (g >= pre[j]) { base = lo[j]; first = pre[j]; }
             cv[i] = *reinterpret_cast<const u32x4*>(a.w0.stream + base + (size_t)(g - first) * 4);
         }
+        if constexpr (MT == 1) {
+            if (a.x_mode == kStageRowCopy) {
+                // vector v of the group: piece v % vpt of tile v / vpt, vpt pieces per tile
+                const int vpt = a.tile_rows / VE;
+#pragma unroll
+                for (int i = 0; i < XPR; ++i) {
+                    const int v = min(tid + i * NT, nt * vpt - 1);
+                    const int tile = (int)(((unsigned long long)(unsigned)v * a.vpt_magic) >> 32);  // v / vpt
+                    const int k = min((t + tile) * a.tile_rows + (v - tile * vpt) * VE, a.K - VE);   // pieces past K re-read the last one
+                    const u32x4 q = *reinterpret_cast<const u32x4*>(Xb + (size_t)k * ES);
+                    xr[i * 4 / RPS][i * 4 % RPS] = q[0]; xr[(i * 4 + 1) / RPS][(i * 4 + 1) % RPS] = q[1];
+                    xr[(i * 4 + 2) / RPS][(i * 4 + 2) % RPS] = q[2]; xr[(i * 4 + 3) / RPS][(i * 4 + 3) % RPS] = q[3];
+                }
+                return;
+            }
+        }
         if constexpr (MT <= 4) {
             if (a.x_mode == kStageRowVectors) {
                 // vectors [v_lo, v_hi) of a row cover the group's k range
@@ -291,6 +309,23 @@ void tl_spmm_block(KernelArgs a)
         if (tid < kMaxBlockSet * (TG + 1)) {
             const int j = tid / (TG + 1), tl = tid % (TG + 1);
             if (j < bs && tl <= nt) cst[tid] = pre[j] * 4 + cs[(size_t)j * a.T + t + tl] - lo[j];
+        }
+        if constexpr (MT == 1) {
+            if (a.x_mode == kStageRowCopy) {
+                // slots past a tile's height (the sentinel slot among them) were zeroed once and are never written
+                const int vpt = a.tile_rows / VE;
+#pragma unroll
+                for (int i = 0; i < XPR; ++i) {
+                    const int v = tid + i * NT;
+                    const int tile = (int)(((unsigned long long)(unsigned)v * a.vpt_magic) >> 32);
+                    const int j = v - tile * vpt;
+                    if (v < nt * vpt && (t + tile) * a.tile_rows + j * VE < a.K)
+                        *reinterpret_cast<u32x4*>(reinterpret_cast<unsigned char*>(xs) + ((size_t)tile * kTileSlots + (size_t)j * VE) * ES) =
+                            u32x4{xr[i * 4 / RPS][i * 4 % RPS], xr[(i * 4 + 1) / RPS][(i * 4 + 1) % RPS],
+                                  xr[(i * 4 + 2) / RPS][(i * 4 + 2) % RPS], xr[(i * 4 + 3) / RPS][(i * 4 + 3) % RPS]};
+                }
+                return;
+            }
         }
         if constexpr (MT <= 4) {
             if (a.x_mode == kStageRowVectors) {
@@ -376,6 +411,10 @@ void tl_spmm_block(KernelArgs a)
 #pragma unroll
     for (int m = 0; m < MT; ++m) acc[m] = 0.f;
 
+    if constexpr (MT == 1) {
+        if (a.x_mode == kStageRowCopy)
+            for (int e = tid; e < a.xs_bytes / 16; e += NT) reinterpret_cast<u32x4*>(xs)[e] = u32x4{0u, 0u, 0u, 0u};
+    }
     constexpr int TU = MT <= 8 ? 2 : 1;  // tiles of one lane whose LDS reads are issued together
     prefetch(0, min(TG, a.T));
     for (int t = 0; t < a.T; t += TG) {
@@ -1141,6 +1180,12 @@ int launch_small(KernelArgs a, const tl_layout_header* h, int x_dtype, void* wor
     // whole vectors of a row are read: K must be whole vectors too, so that none runs past a row's end
     if (!a.x_kmajor && mt <= 4 && aligned && ((int64_t)a.K * es) % 16 == 0) a.x_mode = kStageRowVectors;
     a.tile_magic = (unsigned)(((1ull << 32) + h->tile_rows - 1) / h->tile_rows);
+    // one row whose tiles are whole aligned vectors: straight vector copies
+    const int ve = 16 / es;
+    if (mt == 1 && a.x_sk == 1 && reinterpret_cast<uintptr_t>(a.X) % 16 == 0 && h->tile_rows % ve == 0 && a.K % ve == 0) {
+        a.x_mode = kStageRowCopy;
+        a.vpt_magic = (unsigned)(((1ull << 32) + h->tile_rows / ve - 1) / (h->tile_rows / ve));
+    }
     switch (mt) {
         case 1: return launch_small_mt<1>(a, h, st);
         case 2: return launch_small_mt<2>(a, h, st);

@@ -12,6 +12,7 @@
 //     (block, tile): 16 descriptors followed by the block's runs.  What a workgroup needs
 //     for a range of tiles is then a single contiguous piece of memory.
 #include <cstring>
+#include <algorithm>
 #include <vector>
 
 #include "tl_common.h"
@@ -31,8 +32,10 @@ int pick_geometry(int columns, int inners, int tile_rows, Geometry* g)
     if (tile_rows < 0 || tile_rows > kMaxTileRows)
         return fail(TL_ERR_ARG, "tile_rows=%d must be in [1, %d] (0 = default)", tile_rows, kMaxTileRows);
     if (tile_rows == 0) {
-        const int t = (int)ceil_div(inners, kMaxTileRows);
-        tile_rows = (int)ceil_div(inners, t);
+        // the largest balanced height that is a multiple of 8: a tile's rows then start on a 16-byte
+        // boundary of an fp16 (or fp32) activation row, which the decode kernel copies as whole vectors
+        const int t = (int)ceil_div(inners, 248);
+        tile_rows = std::min<int>(248, (int)round_up(ceil_div(inners, t), 8));
     }
     g->tile_rows = tile_rows;
     g->n_tiles = (int)ceil_div(inners, tile_rows);
