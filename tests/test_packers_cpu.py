@@ -181,3 +181,36 @@ def test_cpu_baselines_match_exact_product():
     p = cpu_baseline.PortProvider()
     xv = x[0]
     assert np.allclose(p.gemv(np.ascontiguousarray(w, np.int8), xv, 64, 1024), xv.astype(np.float64) @ w, atol=1e-3)
+
+
+def test_compute_entry_points_reject_bad_arguments_before_any_launch():
+    """Argument checks of the compute calls run on the host: they must answer without a GPU."""
+    L = _lib.lib()
+    w = ternary_weight(64, 32, 0.5, 2)
+    pw = packing.PackedWeight.from_dense(w)
+    hdr = ctypes.byref(pw.header)
+    need = ctypes.c_int64(-1)
+    assert L.tl_spmm_workspace(hdr, 1, _lib.TL_F16, 0, ctypes.byref(need)) == 0 and need.value == 0
+    assert L.tl_spmm_workspace(hdr, 16, _lib.TL_F16, 0, ctypes.byref(need)) == 0 and need.value == 64 * 16 * 2
+    assert L.tl_spmm_workspace(hdr, 100, _lib.TL_F16, 0, ctypes.byref(need)) == 0 and need.value > 64 * 256 * 2
+    assert L.tl_spmm_workspace(hdr, 0, _lib.TL_F16, 0, ctypes.byref(need)) < 0
+    assert L.tl_spmm_workspace(hdr, 4, 7, 0, ctypes.byref(need)) < 0
+    fake = ctypes.c_void_p(256 * 1024)  # never dereferenced: every call below fails its checks first
+    assert L.tl_spmm(hdr, None, fake, 0, 0, 64, 1, fake, 0, 32, None, 0, None, 0, None) < 0            # null blob
+    assert L.tl_spmm(hdr, fake, fake, 0, 0, 10, 1, fake, 0, 32, None, 0, None, 0, None) < 0            # ldx < K
+    assert L.tl_spmm(hdr, fake, fake, 0, 0, 64, 1, fake, 0, 8, None, 0, None, 0, None) < 0             # ldy < N
+    assert L.tl_spmm(hdr, fake, fake, 0, 2, 64, 1, fake, 0, 32, None, 0, None, 0, None) < 0            # unknown layout
+    assert L.tl_spmm(hdr, ctypes.c_void_p(257), fake, 0, 0, 64, 1, fake, 0, 32, None, 0, None, 0, None) < 0  # unaligned blob
+    pos = ctypes.c_void_p(4096)
+    assert L.tl_rope_cache_update(fake, 5, 1, 2, 64, fake, fake, pos, fake, fake, fake, 16, None) < 0  # dtype
+    assert L.tl_rope_cache_update(fake, 1, 1, 2, 63, fake, fake, pos, fake, fake, fake, 16, None) < 0  # odd head_dim
+    assert L.tl_rope_cache_update(fake, 1, 1, 2, 64, fake, fake, None, fake, fake, fake, 16, None) < 0  # no position
+    assert L.tl_decode_attention(fake, fake, fake, 1, 1, 2, 96, 16, pos, fake, None) < 0                # head_dim not served
+    assert L.tl_decode_attention(fake, fake, fake, 1, 1, 2, 64, 1 << 20, pos, fake, None) < 0           # scores do not fit LDS
+    assert L.tl_decode_attention(fake, fake, ctypes.c_void_p(4104), 1, 1, 2, 64, 16, pos, fake, None) < 0  # unaligned cache
+    assert L.tl_add_rmsnorm(fake, None, fake, 9, 1, 64, 1e-5, None, fake, None) < 0
+    assert L.tl_add_rmsnorm(fake, fake, fake, 1, 1, 64, 1e-5, None, fake, None) < 0                     # y without x_out
+    assert L.tl_add_rmsnorm(fake, None, fake, 1, 0, 64, 1e-5, None, fake, None) < 0
+    assert L.tl_silu_mul(None, 1, 1, 64, fake, None) < 0
+    assert L.tl_silu_mul(fake, 1, 1, 0, fake, None) < 0
+    assert L.tl_last_error()
