@@ -171,3 +171,27 @@ def test_rows_kernel_with_and_without_shared_out_tiles(cuda, oracle, dtype, monk
             assert np.abs(h - ref_fused).max() <= (FP16_TOL if dtype == torch.float16 else 1e-4) * scale, (M, K, N, mode)
             fused[mode] = h
         monkeypatch.delenv("TL_ROWS_SPLIT")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_output_into_a_strided_buffer(cuda, oracle, dtype):
+    """`out=` as a column slice of a wider buffer: leading dimensions that allow the row kernel's whole-row
+    stores and ones that do not, for both kernels; nothing outside the slice may be touched."""
+    from ternaryllm_amd import ops
+    from ternaryllm_amd.packing import PackedWeight
+    K, N = 600, 256
+    w = ternary_weight(K, N, 0.8, 61)
+    dw = ops.DeviceWeight(PackedWeight.from_dense(w), cuda)
+    for M in (3, 20, 300):
+        x = activations(M, K, 62 + M, dtype, integer=True)
+        ref = oracle.fast_product(x.double().numpy(), w)
+        for width, first in ((N + 4, 4), (N + 5, 3), (N + 8, 0), (N + 1, 1)):
+            buf = torch.full((M, width), 7.0, dtype=torch.float32, device=cuda)
+            out = buf[:, first:first + N]
+            print(f"case M={M} dtype={dtype} width={width} first={first}", flush=True)
+            ops.spmm(dw, x.to(cuda), out_dtype=torch.float32, out=out)
+            got = buf.cpu().numpy()
+            assert np.array_equal(got[:, first:first + N].astype(np.float64), ref), (M, width, first)
+            mask = np.ones(width, bool)
+            mask[first:first + N] = False
+            assert (got[:, mask] == 7.0).all(), (M, width, first)
