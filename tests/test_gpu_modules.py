@@ -181,3 +181,27 @@ def test_surgery_on_a_hugging_face_llama(cuda):
         ref = dense(ids).logits.float()
     assert torch.isfinite(ref).all()
     assert (got - ref).abs().max().item() <= 1e-3 * ref.abs().max().item()
+
+
+@pytest.mark.parametrize("name,M,K,N,s,dtype", [
+    ("config 1", 16, 4096, 4096, 0.5, torch.float32),
+    ("config 2", 1, 4096, 4096, 0.66, torch.float16),
+    ("config 3 down", 1024, 11008, 4096, 0.8, torch.float16),
+    ("config 4 projection", 1024, 4096, 4096, 0.9, torch.float16),
+    ("config 5 decode head", 16, 4096, 32000, 0.66, torch.float16),
+])
+def test_baseline_configs_at_full_size(cuda, name, M, K, N, s, dtype):
+    """The other benchmark shapes at their full sizes, on small-integer activations (every partial sum exact):
+    the two checksum identities of the product, and for a few rows the product itself."""
+    from ternaryllm_amd import ops
+    from ternaryllm_amd.packing import PackedWeight
+    w = ternary_weight(K, N, s, 1300 + N % 97)
+    dw = ops.DeviceWeight(PackedWeight.from_dense(w), cuda)
+    x = activations(M, K, 5, dtype, integer=True)
+    print(f"case {name}", flush=True)
+    y = ops.spmm(dw, x.to(cuda), out_dtype=torch.float32)
+    wd = w.astype(np.float64)
+    assert np.array_equal(y.double().sum(1).cpu().numpy(), x.double().numpy() @ wd.sum(1))
+    assert np.array_equal(y.double().sum(0).cpu().numpy(), x.double().numpy().sum(0) @ wd)
+    rows = sorted({0, M // 2, M - 1})
+    assert np.array_equal(y[rows].double().cpu().numpy(), x[rows].double().numpy() @ wd)
