@@ -81,38 +81,28 @@ def one_tile(pos_rows, neg_rows, tk=16):
     return w
 
 
-def test_mcsc_hand_worked_tiles(oracle):
-    # (1) more -1 than +1, odd pair count, leftover 3: the pair region shrinks from 6 to 4 entries and the
-    #     leftover count 3 -> 2 -> 0 (ter_spmm_wrapper.cu:277-291); the stream keeps every index.
-    rows, off, _ = oracle.tiled_mcsc(one_tile([1, 4, 9], [2, 7, 8, 11, 13, 15]), 16)
-    assert rows.tolist() == [1, 2, 4, 7, 9, 8, 11, 13, 15]
-    assert off.tolist() == [0, 4, 4, -1]
-    # (2) neg <= pos, odd pair count (1 pair -> 0 kept), leftover 4 stays 4, sign +1
-    rows, off, _ = oracle.tiled_mcsc(one_tile([0, 3, 5, 6, 10], [2]), 16)
-    assert rows.tolist() == [0, 2, 3, 5, 6, 10]
-    assert off.tolist() == [0, 0, 4, 1]
-    # (3) balanced, even pairs: nothing is dropped
-    rows, off, _ = oracle.tiled_mcsc(one_tile([0, 3, 5, 6], [1, 2, 4, 9]), 16)
-    assert rows.tolist() == [0, 1, 3, 2, 5, 4, 6, 9]
-    assert off.tolist() == [0, 8, 8, 1]
-    # (4) padding_size 4, odd pair count: pairs [p0 n0 p1 n1 p2 n2] padded to 8 with p0, then the leftover
-    #     (-1 rows 11, 13, 15) overwrites the padding from position 6 on; array padded to 8 + 4.
-    rows, off, _ = oracle.tiled_mcsc(one_tile([1, 4, 9], [2, 7, 8, 11, 13, 15]), 16, True, 4)
-    assert rows.tolist() == [1, 2, 4, 7, 9, 8, 11, 13, 15, 0, 0, 0]
-    assert off.tolist() == [0, 8, 8, -1]
+def hand_cases():
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "mcsc_hand_cases.json")) as f:
+        return json.load(f)["cases"]
 
 
-def test_mcsc_two_tiles_overwrite_the_dropped_tail(oracle):
-    # tile 0 keeps 4 of its 9 entries, so tile 1 starts at cursor 4 and overwrites the rest of tile 0
-    w = np.zeros((32, 1), np.int32)
-    w[[1, 4, 9], 0] = 1
-    w[[2, 7, 8, 11, 13, 15], 0] = -1
-    w[[16 + 0, 16 + 3], 0] = 1
-    w[[16 + 1, 16 + 2], 0] = -1
-    rows, off, tiles = oracle.tiled_mcsc(w, 16)
-    assert off.tolist() == [0, 4, 4, -1, 4, 8, 8, 1]
-    assert rows.tolist() == [1, 2, 4, 7, 0, 1, 3, 2, 15, 0, 0, 0, 0]
-    assert tiles.tolist() == [0, 1]  # equal stored lengths: stable order
+def hand_case_weight(case):
+    w = np.zeros((case["inners"], 1), np.int32)
+    w[case["pos_rows"], 0] = 1
+    w[case["neg_rows"], 0] = -1
+    return w
+
+
+@pytest.mark.parametrize("case", hand_cases(), ids=lambda c: c["name"][:40])
+def test_mcsc_hand_worked_tiles(oracle, case):
+    """tests/golden/mcsc_hand_cases.json: tiles worked out by hand from ter_spmm_wrapper.cu:156-315 (the
+    4-alignment truncation :277-291, padding with overwrite :253-275, the truncated cursor :293-300)."""
+    rows, off, tiles = oracle.tiled_mcsc(hand_case_weight(case), case["tile_k"], case["padding"], case["padding_size"])
+    assert rows.tolist() == case["merged_row_idx"]
+    assert off.tolist() == case["merged_off"]
+    assert tiles.tolist() == case["col_tile_idx"]
 
 
 def test_mcsc_reduces_to_interleave_when_balanced(oracle):

@@ -214,3 +214,17 @@ def test_compute_entry_points_reject_bad_arguments_before_any_launch():
     assert L.tl_silu_mul(None, 1, 1, 64, fake, None) < 0
     assert L.tl_silu_mul(fake, 1, 1, 0, fake, None) < 0
     assert L.tl_last_error()
+
+
+def test_library_packer_on_the_hand_worked_tiles():
+    """The library's merged packer against tests/golden/mcsc_hand_cases.json (outputs derived by hand from
+    the reference's source)."""
+    from tests.test_oracle_pins import hand_case_weight, hand_cases
+    for case in hand_cases():
+        w = hand_case_weight(case)
+        cp, cn = packing.count_nnz(w)
+        rows, off, tiles = packing.convert_to_ter_tiled_mcsc(w, 1, case["inners"], cp, cn, case["tile_k"], case["padding"],
+                                                             case["padding_size"])
+        assert rows.tolist() == case["merged_row_idx"], case["name"]
+        assert off.tolist() == case["merged_off"], case["name"]
+        assert tiles.tolist() == case["col_tile_idx"], case["name"]
