@@ -101,15 +101,12 @@ __device__ __forceinline__ void gather_add(float (&acc)[MT], const XT* __restric
         const uint32_t r = (word >> (8 * b)) & 0xffu;
         const XT* row = xt + r * MT;
         if constexpr (sizeof(XT) == 4) {
-            if constexpr (MT % 4 == 0) {
-#pragma unroll
-                for (int m = 0; m < MT; m += 4) {
-                    const float4 v = *reinterpret_cast<const float4*>(row + m);
-                    acc[m + 0] = fmaf(v.x, sign, acc[m + 0]);
-                    acc[m + 1] = fmaf(v.y, sign, acc[m + 1]);
-                    acc[m + 2] = fmaf(v.z, sign, acc[m + 2]);
-                    acc[m + 3] = fmaf(v.w, sign, acc[m + 3]);
-                }
+            if constexpr (MT == 4) {
+                const float4 v = *reinterpret_cast<const float4*>(row);
+                acc[0] = fmaf(v.x, sign, acc[0]);
+                acc[1] = fmaf(v.y, sign, acc[1]);
+                acc[2] = fmaf(v.z, sign, acc[2]);
+                acc[3] = fmaf(v.w, sign, acc[3]);
             } else if constexpr (MT == 2) {
                 const float2 v = *reinterpret_cast<const float2*>(row);
                 acc[0] = fmaf(v.x, sign, acc[0]);
@@ -118,17 +115,7 @@ __device__ __forceinline__ void gather_add(float (&acc)[MT], const XT* __restric
                 acc[0] = fmaf(row[0], sign, acc[0]);
             }
         } else {
-            if constexpr (MT >= 8) {
-#pragma unroll
-                for (int m = 0; m < MT; m += 8) {
-                    const u32x4 v = *reinterpret_cast<const u32x4*>(row + m);
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        acc[m + 2 * j] = fmaf(__half2float(__ushort_as_half((unsigned short)(v[j] & 0xffffu))), sign, acc[m + 2 * j]);
-                        acc[m + 2 * j + 1] = fmaf(__half2float(__ushort_as_half((unsigned short)(v[j] >> 16))), sign, acc[m + 2 * j + 1]);
-                    }
-                }
-            } else if constexpr (MT == 4) {
+            if constexpr (MT == 4) {
                 const uint2 v = *reinterpret_cast<const uint2*>(row);
                 acc[0] = fmaf(__half2float(__ushort_as_half((unsigned short)(v.x & 0xffffu))), sign, acc[0]);
                 acc[1] = fmaf(__half2float(__ushort_as_half((unsigned short)(v.x >> 16))), sign, acc[1]);
@@ -145,6 +132,31 @@ __device__ __forceinline__ void gather_add(float (&acc)[MT], const XT* __restric
     }
 }
 
+// The same for a lane that owns four neighbouring rows of the slot (`xq` already points at them):
+// one 8- or 16-byte LDS read and four accumulating ops per index.
+template <int MT, typename XT>
+__device__ __forceinline__ void gather_add_quad(float (&acc)[4], const XT* __restrict__ xq, uint32_t word, float sign)
+{
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+        const uint32_t r = (word >> (8 * b)) & 0xffu;
+        const XT* row = xq + r * MT;
+        if constexpr (sizeof(XT) == 4) {
+            const float4 v = *reinterpret_cast<const float4*>(row);
+            acc[0] = fmaf(v.x, sign, acc[0]);
+            acc[1] = fmaf(v.y, sign, acc[1]);
+            acc[2] = fmaf(v.z, sign, acc[2]);
+            acc[3] = fmaf(v.w, sign, acc[3]);
+        } else {
+            const uint2 v = *reinterpret_cast<const uint2*>(row);
+            acc[0] = fmaf(__half2float(__ushort_as_half((unsigned short)(v.x & 0xffffu))), sign, acc[0]);
+            acc[1] = fmaf(__half2float(__ushort_as_half((unsigned short)(v.x >> 16))), sign, acc[1]);
+            acc[2] = fmaf(__half2float(__ushort_as_half((unsigned short)(v.y & 0xffffu))), sign, acc[2]);
+            acc[3] = fmaf(__half2float(__ushort_as_half((unsigned short)(v.y >> 16))), sign, acc[3]);
+        }
+    }
+}
+
 constexpr int kBlockThreads = 512;            // workgroup of the small-M kernel
 // Staging of the activations by the small-M kernel:
 constexpr int kStageElements = 0;     // a thread owns slots and reads their MT values one by one (any layout)
@@ -157,15 +169,14 @@ constexpr int kMaxChunkBytes = (TL_BLOCK_COLUMNS + TL_BLOCK_COLUMNS * 128) * 4; 
 
 // What one thread keeps in registers while a group of tiles is in flight: kVectors 16-byte pieces of
 // the stream and, for kSlots slots of the staged tiles, kSlotRegs dwords of activations each.
-// Slots of 8 rows and more are only ever staged as whole vectors (MT * ES / 4 dwords), narrower ones
-// also element by element (one dword per value).
+// (One dword per value: slots are staged element by element or as vectors, as the layout allows.)
 template <int MT, int ES, int NT>
 struct BlockShape {
     static constexpr int kStreamCap = (NT * 256 < kMaxChunkBytes ? kMaxChunkBytes + 240
                                        : (NT * 256 > kSmallStreamBytes ? kSmallStreamBytes : NT * 256)) / 16 * 16;
     static constexpr int kVectors = (kStreamCap / 16 + NT - 1) / NT;
-    static constexpr int kSlotRegs = MT >= 8 ? MT * ES / 4 : MT;
-    static constexpr int kSlots = MT <= 4 ? 16 : (kSlotRegs >= 16 ? 4 : 36 / kSlotRegs);  // per thread
+    static constexpr int kSlotRegs = MT;
+    static constexpr int kSlots = 16;  // per thread
     static constexpr int kTiles = kSlots * NT / kTileSlots;                   // tiles per group at most
 };
 
@@ -182,9 +193,9 @@ struct BlockShape {
 // ops.  The LPC partial sums of a column are folded with cross-lane shuffles.  No workgroup depends
 // on another.
 // Four waves per SIMD (two workgroups per compute unit) is what the LDS budget plans for: the register
-// allocation is held to that, except for 16 fp32 rows per slot, whose gathers alone need 64 registers.
+// allocation is held to that.  MT is 1, 2 or 4; taller slots go to tl_spmm_quad.
 template <int MT, bool XF16>
-__global__ __launch_bounds__(kBlockThreads) __attribute__((amdgpu_waves_per_eu(MT * (XF16 ? 2 : 4) >= 64 ? 2 : 4, MT * (XF16 ? 2 : 4) >= 64 ? 2 : 4)))
+__global__ __launch_bounds__(kBlockThreads) __attribute__((amdgpu_waves_per_eu(4, 4)))
 void tl_spmm_block(KernelArgs a)
 {
     extern __shared__ __align__(16) unsigned char lds[];
@@ -199,7 +210,8 @@ void tl_spmm_block(KernelArgs a)
     constexpr int VE = 16 / ES;          // activation values per 16-byte vector
     // row-vector staging: vectors per thread and row that cover a group of Shape::kTiles tiles (+2 for the ragged ends)
     constexpr int XPR = ((Shape::kTiles * kMaxTileRows + VE - 1) / VE + 2 + NT - 1) / NT;
-    static_assert(MT > 4 || MT * XPR * 4 <= SPT * RPS, "row vectors must fit the staging registers");
+    static_assert(MT <= 4, "slots of 8 and 16 rows are tl_spmm_quad's");
+    static_assert(MT * XPR * 4 <= SPT * RPS, "row vectors must fit the staging registers");
     const int tid = threadIdx.x;
     const int BS = a.block_set, TG = a.tiles_per_group;
     const int nb0 = blockIdx.x * BS, m0 = blockIdx.y * MT;
@@ -273,7 +285,7 @@ void tl_spmm_block(KernelArgs a)
             const int tile = e >> 8, r = e & 255;
             // slots that hold no row re-read a valid element; they are stored as zeros
             const int k = min((t + min(tile, nt - 1)) * a.tile_rows + min(r, a.tile_rows - 1), a.K - 1);
-            if (MT >= 8 || a.x_mode == kStageSlotVectors) {
+            if (a.x_mode == kStageSlotVectors) {
                 if constexpr (VPS > 0) {
                     const unsigned char* src = Xb + ((size_t)k * a.ldx + m0) * ES;
 #pragma unroll
@@ -371,10 +383,7 @@ void tl_spmm_block(KernelArgs a)
             if (tile < nt) {
                 const bool real = r < min(a.tile_rows, a.K - (t + tile) * a.tile_rows);
                 uint32_t packed[MT * ES / 4 > 0 ? MT * ES / 4 : 1];
-                if constexpr (MT >= 8) {
-#pragma unroll
-                    for (int d = 0; d < MT * ES / 4; ++d) packed[d] = real ? xr[s][d] : 0u;
-                } else if (a.x_mode == kStageSlotVectors && VPS > 0) {
+                if (a.x_mode == kStageSlotVectors && VPS > 0) {
 #pragma unroll
                     for (int d = 0; d < MT * ES / 4; ++d) packed[d] = real ? xr[s][d] : 0u;
                 } else if constexpr (XF16) {
@@ -415,7 +424,7 @@ void tl_spmm_block(KernelArgs a)
         if (a.x_mode == kStageRowCopy)
             for (int e = tid; e < a.xs_bytes / 16; e += NT) reinterpret_cast<u32x4*>(xs)[e] = u32x4{0u, 0u, 0u, 0u};
     }
-    constexpr int TU = MT <= 8 ? 2 : 1;  // tiles of one lane whose LDS reads are issued together
+    constexpr int TU = 2;  // tiles of one lane whose LDS reads are issued together
     prefetch(0, min(TG, a.T));
     for (int t = 0; t < a.T; t += TG) {
         const int nt = min(TG, a.T - t);
@@ -467,6 +476,130 @@ void tl_spmm_block(KernelArgs a)
 #pragma unroll
         for (int m = 0; m < MT; ++m)
             if (m0 + m < a.M) store_out(a.Y, a.y_f16, (long long)(m0 + m) * a.ldy + n, acc[m] * s);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Small-M kernel for slots of 8 and 16 rows, staged by direct global -> LDS loads.
+// ---------------------------------------------------------------------------
+// One workgroup owns one block of 16 columns and MT activation rows over all of K, walked in groups
+// of TG tiles.  A group's chunks and its activation rows (from the aligned K-major image, whose row k
+// holds the MT values of slot k side by side) are copied into LDS by `global_load_lds_dwordx4`: a lane
+// names 16 bytes in memory, they land at M0 + 16 * lane, and no register holds them on the way.  Two
+// LDS buffers alternate: the loads of group g + 1 are issued before group g is consumed, and one
+// barrier per group orders both the reuse of a buffer and the arrival of the next one.  Slots past a
+// tile's height (the sentinel among them) are written as zeros by ordinary stores.
+// With no staging registers a workgroup needs few registers, so several share a compute unit and
+// hide each other's waits; the launcher sizes TG for that.
+// Gather: a lane owns four rows of one column, the MT / 4 lanes of a column sit side by side and the 16
+// columns next to each other, so one gather instruction reads 16 slots (one per column) as whole
+// contiguous pieces.  The P lane groups of a column share its runs: TP tiles side by side, LW groups
+// per run, up to four dwords (16 independent gathers) per turn.  The P partial sums are folded through LDS.
+template <int MT, bool XF16>
+__global__ __launch_bounds__(kBlockThreads) void tl_spmm_quad(KernelArgs a)
+{
+    extern __shared__ __align__(16) unsigned char lds[];
+    using XT = typename std::conditional<XF16, __half, float>::type;
+    constexpr int NT = kBlockThreads;
+    constexpr int ES = (int)sizeof(XT);
+    constexpr int SLOT = MT * ES;      // bytes of a slot
+    constexpr int VPS = SLOT / 16;     // 16-byte pieces per slot
+    constexpr int Q = MT / 4;
+    static_assert(MT == 8 || MT == 16, "row quads of 8- and 16-row slots");
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int TG = a.tiles_per_group;
+    const int nb = blockIdx.x, m0 = blockIdx.y * MT;
+    const int stage_bytes = a.xs_bytes + a.buf_bytes;
+    uint32_t* cst = reinterpret_cast<uint32_t*>(lds + 2 * stage_bytes);  // [2][TG + 1] chunk starts inside a buffer's chunk copies
+    const_u32_ptr cs = as_const(a.w0.chunkstart) + (size_t)nb * a.T;
+    const unsigned char* Xb = static_cast<const unsigned char*>(a.X) + (size_t)m0 * ES;
+    const size_t row_bytes = (size_t)a.ldx * ES;
+    using global_ptr = const __attribute__((address_space(1))) void*;
+    using lds_ptr = __attribute__((address_space(3))) void*;
+
+    // global -> LDS buffer `which` for the tiles [t, t + nt)
+    auto issue = [&](int t, int nt, int which) {
+        unsigned char* xs = lds + which * stage_bytes;
+        unsigned char* buf = xs + a.xs_bytes;
+        const int pieces = nt * kTileSlots * VPS;  // a multiple of 64: whole waves
+        for (int first = wave * 64; first < pieces; first += NT) {
+            const int p = first + lane, slot = p / VPS, v = p % VPS;
+            const int r = slot & (kTileSlots - 1), k = (t + (slot >> 8)) * a.tile_rows + r;
+            if (r < a.tile_rows && k < a.K)
+                __builtin_amdgcn_global_load_lds((global_ptr)(Xb + (size_t)k * row_bytes + v * 16), (lds_ptr)(xs + (size_t)first * 16), 16, 0, 0);
+            else
+                *reinterpret_cast<u32x4*>(xs + (size_t)p * 16) = u32x4{0u, 0u, 0u, 0u};
+        }
+        const uint32_t lo = cs[t];
+        const int vectors = (int)((cs[t + nt] - lo) / 4);
+        for (int first = wave * 64; first < vectors; first += NT)
+            if (first + lane < vectors)
+                __builtin_amdgcn_global_load_lds((global_ptr)(a.w0.stream + lo + (size_t)(first + lane) * 4), (lds_ptr)(buf + (size_t)first * 16), 16, 0, 0);
+        if (tid <= nt) cst[which * (TG + 1) + tid] = cs[t + tid] - lo;
+    };
+
+    const int lw_shift = a.lw_shift;
+    const int LPC = 1 << a.lpc_shift, LW = 1 << lw_shift, TP = LPC >> lw_shift;
+    const int q = tid % Q, c16 = (tid / Q) & 15, lig = tid / (Q * TL_BLOCK_COLUMNS);
+    const int tp = lig >> lw_shift, lw = lig & (LW - 1);
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+
+    issue(0, min(TG, a.T), 0);
+    int which = 0;
+    for (int t = 0; t < a.T; t += TG, which ^= 1) {
+        const int nt = min(TG, a.T - t);
+        // this wave's loads have landed; after the barrier everybody's have, and the other buffer is free
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (t + TG < a.T) issue(t + TG, min(TG, a.T - t - TG), which ^ 1);
+        const unsigned char* xs = lds + which * stage_bytes;
+        const uint32_t* buf = reinterpret_cast<const uint32_t*>(xs + a.xs_bytes);
+        const uint32_t* my_cst = cst + which * (TG + 1);
+        for (int tl = tp; tl < nt; tl += TP) {
+            const uint32_t* chunk = buf + my_cst[tl];
+            const uint32_t d = chunk[c16];
+            const uint32_t* run = chunk + (d >> 16);
+            const int pd = run_pos_dwords(d), tot = pd + run_neg_dwords(d);
+            const XT* xq = reinterpret_cast<const XT*>(xs) + (size_t)tl * kTileSlots * MT + q * 4;
+            int i = lw;
+            for (; i + 3 * LW < tot; i += 4 * LW) {
+                const uint32_t w0 = run[i], w1 = run[i + LW], w2 = run[i + 2 * LW], w3 = run[i + 3 * LW];
+                gather_add_quad<MT, XT>(acc, xq, w0, i < pd ? 1.0f : -1.0f);
+                gather_add_quad<MT, XT>(acc, xq, w1, i + LW < pd ? 1.0f : -1.0f);
+                gather_add_quad<MT, XT>(acc, xq, w2, i + 2 * LW < pd ? 1.0f : -1.0f);
+                gather_add_quad<MT, XT>(acc, xq, w3, i + 3 * LW < pd ? 1.0f : -1.0f);
+            }
+            if (i + LW < tot) {
+                const uint32_t w0 = run[i], w1 = run[i + LW];
+                gather_add_quad<MT, XT>(acc, xq, w0, i < pd ? 1.0f : -1.0f);
+                gather_add_quad<MT, XT>(acc, xq, w1, i + LW < pd ? 1.0f : -1.0f);
+                i += 2 * LW;
+            }
+            if (i < tot) gather_add_quad<MT, XT>(acc, xq, run[i], i < pd ? 1.0f : -1.0f);
+        }
+    }
+    // fold the LPC partial sums of each (column, row quad) through LDS
+    __syncthreads();
+    float4* red = reinterpret_cast<float4*>(lds);
+    red[tid] = make_float4(acc[0], acc[1], acc[2], acc[3]);
+    __syncthreads();
+    constexpr int per_group = TL_BLOCK_COLUMNS * Q;  // threads of one lane group
+    if (tid < per_group) {
+        float4 sum = red[tid];
+#pragma unroll 4
+        for (int l = 1; l < LPC; ++l) {
+            const float4 o = red[l * per_group + tid];
+            sum.x += o.x; sum.y += o.y; sum.z += o.z; sum.w += o.w;
+        }
+        const int n = nb * TL_BLOCK_COLUMNS + c16;
+        if (n < a.N) {
+            const float sc = load_scale(a.w0.scale, a.scale_f16, n);
+            const float out[4] = {sum.x, sum.y, sum.z, sum.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (m0 + q * 4 + j < a.M) store_out(a.Y, a.y_f16, (long long)(m0 + q * 4 + j) * a.ldy + n, out[j] * sc);
+        }
     }
 }
 
@@ -1107,12 +1240,6 @@ int launch_block_kernel(KernelArgs a, const tl_layout_header* h, hipStream_t st)
     return TL_OK;
 }
 
-template <int MT>
-int launch_small_mt(const KernelArgs& a, const tl_layout_header* h, hipStream_t st)
-{
-    return a.x_f16 ? launch_block_kernel<MT, true>(a, h, st) : launch_block_kernel<MT, false>(a, h, st);
-}
-
 inline int log2_exact(int v)
 {
     int s = 0;
@@ -1120,15 +1247,67 @@ inline int log2_exact(int v)
     return s;
 }
 
+// The direct-load kernel for 8- and 16-row slots.  Its LDS holds two buffers of TG tiles (activation image +
+// chunk copies); TG is sized so that `share` workgroups fit a compute unit, as many as the launch can
+// give each compute unit, up to four.
+template <int MT, bool XF16>
+int launch_quad_kernel(KernelArgs a, const tl_layout_header* h, hipStream_t st)
+{
+    constexpr int es = XF16 ? 2 : 4;
+    constexpr int groups = kBlockThreads / (TL_BLOCK_COLUMNS * (MT / 4));  // lane groups per column
+    const int tile_bytes = kTileSlots * MT * es;
+    const int chunk_bytes = (int)h->max_chunk_dwords * 4;
+    const unsigned gx = (unsigned)a.NB, gy = (unsigned)ceil_div(a.M, MT);
+    const int share = std::max(1, std::min(env_int("TL_QUAD_SHARE", 4), (int)ceil_div((int64_t)gx * gy, kComputeUnits)));
+    const int budget = 160 * 1024 / share - 1024;
+    int tg = std::max(1, std::min(a.T, (budget - 256) / (2 * (tile_bytes + chunk_bytes))));
+    tg = std::max(1, std::min(tg, env_int("TL_TILE_GROUP", tg)));
+    tg = (int)ceil_div(a.T, ceil_div(a.T, tg));  // same number of groups, evened out
+    a.tiles_per_group = tg;
+    a.xs_bytes = tg * tile_bytes;
+    a.buf_bytes = (int)round_up((int64_t)tg * chunk_bytes, 16);
+    const size_t lds = std::max<size_t>(2 * ((size_t)a.xs_bytes + a.buf_bytes) + 2 * (size_t)(tg + 1) * 4, (size_t)kBlockThreads * 16);
+    if (lds > 160 * 1024) return fail(TL_ERR_UNSUPPORTED, "two tiles of %d rows need %zu bytes of LDS", MT, lds);
+    // lane groups per run: a run's dwords go round the LW groups, four per group and turn; no more
+    // tiles side by side than a group of tiles has
+    const double mean_run = h->mean_run_dwords_x16 / 16.0;
+    int lw = 2;
+    while (lw < groups && lw * 8 < mean_run) lw *= 2;
+    while (groups / lw > tg) lw *= 2;
+    lw = std::min(env_int("TL_LW", lw), groups);
+    if (lw < 1 || (lw & (lw - 1))) return fail(TL_ERR_ARG, "TL_LW=%d (a power of two expected)", lw);
+    a.lpc_shift = log2_exact(groups);
+    a.lw_shift = log2_exact(lw);
+    auto kernel = tl_spmm_quad<MT, XF16>;
+    static bool raised = false;  // per instantiation; a repeated or racing call is harmless
+    if (!raised) {
+        if (int rc = raise_lds_limit(kernel, 160 * 1024)) return rc;
+        raised = true;
+    }
+    hipLaunchKernelGGL(kernel, dim3(gx, gy), dim3(kBlockThreads), lds, st, a);
+    return TL_OK;
+}
+
+template <int MT>
+int launch_small_mt(const KernelArgs& a, const tl_layout_header* h, hipStream_t st)
+{
+    return a.x_f16 ? launch_block_kernel<MT, true>(a, h, st) : launch_block_kernel<MT, false>(a, h, st);
+}
+
 int launch_small(KernelArgs a, const tl_layout_header* h, int x_dtype, void* workspace, int64_t workspace_bytes, hipStream_t st)
 {
     int mt = 1;
     while (mt < a.M && mt < 16) mt *= 2;
+    // 16-row slots with no more workgroups than compute units: 8-row slots give twice the workgroups,
+    // each with half the LDS image, so that two share a compute unit and hide each other's waits.
+    if (mt == 16 && (int64_t)a.NB * ceil_div(a.M, 16) <= kComputeUnits) mt = 8;
+    mt = env_int("TL_SMALL_MT", mt);
+    if (mt != 1 && mt != 2 && mt != 4 && mt != 8 && mt != 16) return fail(TL_ERR_ARG, "TL_SMALL_MT=%d (1, 2, 4, 8 or 16 expected)", mt);
     const int es = x_dtype == TL_F16 ? 2 : 4;
     a.x_sm = a.x_kmajor ? 1 : a.ldx;
     a.x_sk = a.x_kmajor ? a.ldx : 1;
     bool aligned = (a.ldx * es) % 16 == 0 && reinterpret_cast<uintptr_t>(a.X) % 16 == 0;
-    // Slots of 8 rows and more are staged as whole vectors from an aligned K-major image; activations
+    // Slots of 8 and 16 rows are copied into LDS as 16-byte pieces of an aligned K-major image; activations
     // that are not one already are brought into that form in the workspace first.
     if (mt >= 8 && !(a.x_kmajor && aligned && a.ldx >= round_up(a.M, mt))) {
         const int64_t need = small_kmajor_bytes(h, a.M, x_dtype);
@@ -1150,16 +1329,19 @@ int launch_small(KernelArgs a, const tl_layout_header* h, int x_dtype, void* wor
         a.x_sk = ldo;
         aligned = true;
     }
+    if (mt >= 8) {
+        if (mt == 8) return a.x_f16 ? launch_quad_kernel<8, true>(a, h, st) : launch_quad_kernel<8, false>(a, h, st);
+        return a.x_f16 ? launch_quad_kernel<16, true>(a, h, st) : launch_quad_kernel<16, false>(a, h, st);
+    }
     // Column blocks per workgroup.  A compute unit works through ceil(workgroups / 256) workgroups of
-    // `set` blocks each; among the sets that keep that product smallest, wider ones re-read the
-    // activations less often, which pays once a slot holds many rows.
+    // `set` blocks each: the narrowest set that keeps that product smallest.
     int set = 1;
     {
         int64_t best = -1;
         for (int cand = 1; cand <= kMaxBlockSet; cand *= 2) {
             if ((int64_t)h->max_chunk_dwords * 4 * cand > BlockShape<1, 2, kBlockThreads>::kStreamCap) break;
             const int64_t cost = ceil_div(ceil_div(a.NB, cand), kComputeUnits) * cand;
-            if (best < 0 || cost < best || (cost == best && mt >= 8)) { best = cost; set = cand; }
+            if (best < 0 || cost < best) { best = cost; set = cand; }
         }
     }
     set = env_int("TL_BLOCK_SET", set);
@@ -1189,9 +1371,7 @@ int launch_small(KernelArgs a, const tl_layout_header* h, int x_dtype, void* wor
     switch (mt) {
         case 1: return launch_small_mt<1>(a, h, st);
         case 2: return launch_small_mt<2>(a, h, st);
-        case 4: return launch_small_mt<4>(a, h, st);
-        case 8: return launch_small_mt<8>(a, h, st);
-        default: return launch_small_mt<16>(a, h, st);
+        default: return launch_small_mt<4>(a, h, st);
     }
 }
 
