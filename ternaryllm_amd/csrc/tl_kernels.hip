@@ -604,6 +604,106 @@ __global__ __launch_bounds__(kBlockThreads) void tl_spmm_quad(KernelArgs a)
 }
 
 // ---------------------------------------------------------------------------
+// One activation row (decode), staged by direct global -> LDS loads.
+// ---------------------------------------------------------------------------
+// As tl_spmm_quad, for M = 1 and a contiguous, 16-byte aligned activation row whose tiles are whole
+// 16-byte pieces: a tile's LDS image [256 slots] is a straight copy of its piece of the row, followed by
+// zeros.  One workgroup owns one block of 16 columns; 32 lanes share a column as in tl_spmm_block
+// (TP tiles side by side, LW lanes per run, one dword per lane and pass, two tiles' reads issued
+// together), and fold their sums with cross-lane shuffles.  When all of K fits the LDS there is a
+// single group: every load of the workgroup is in flight at once and nothing is staged twice.
+template <bool XF16>
+__global__ __launch_bounds__(kBlockThreads) void tl_spmv_direct(KernelArgs a)
+{
+    extern __shared__ __align__(16) unsigned char lds[];
+    using XT = typename std::conditional<XF16, __half, float>::type;
+    constexpr int NT = kBlockThreads;
+    constexpr int ES = (int)sizeof(XT);
+    constexpr int VE = 16 / ES;                  // values per 16-byte piece
+    constexpr int PPT = kTileSlots / VE;         // pieces per tile image
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int TG = a.tiles_per_group;
+    const int nb = blockIdx.x;
+    const int stage_bytes = a.xs_bytes + a.buf_bytes;
+    const int buffers = TG < a.T ? 2 : 1;
+    uint32_t* cst = reinterpret_cast<uint32_t*>(lds + buffers * stage_bytes);  // [buffers][TG + 1] chunk starts inside a buffer's chunk copies
+    const_u32_ptr cs = as_const(a.w0.chunkstart) + (size_t)nb * a.T;
+    const unsigned char* Xb = static_cast<const unsigned char*>(a.X);
+    using global_ptr = const __attribute__((address_space(1))) void*;
+    using lds_ptr = __attribute__((address_space(3))) void*;
+
+    auto issue = [&](int t, int nt, int which) {
+        unsigned char* xs = lds + which * stage_bytes;
+        unsigned char* buf = xs + a.xs_bytes;
+        const uint32_t lo = cs[t];
+        const int vectors = (int)((cs[t + nt] - lo) / 4);
+        for (int first = wave * 64; first < vectors; first += NT)
+            if (first + lane < vectors)
+                __builtin_amdgcn_global_load_lds((global_ptr)(a.w0.stream + lo + (size_t)(first + lane) * 4), (lds_ptr)(buf + (size_t)first * 16), 16, 0, 0);
+        const int pieces = nt * PPT;  // PPT is 32 or 64: a wave's 64 pieces never straddle the image's end by less than a tile
+        for (int first = wave * 64; first < pieces; first += NT) {
+            const int p = first + lane, tile = p / PPT, k = (t + tile) * a.tile_rows + (p % PPT) * VE;
+            if (p < pieces) {
+                if ((p % PPT) * VE < a.tile_rows && k < a.K)
+                    __builtin_amdgcn_global_load_lds((global_ptr)(Xb + (size_t)k * ES), (lds_ptr)(xs + (size_t)first * 16), 16, 0, 0);
+                else
+                    *reinterpret_cast<u32x4*>(xs + (size_t)p * 16) = u32x4{0u, 0u, 0u, 0u};
+            }
+        }
+        if (tid <= nt) cst[which * (TG + 1) + tid] = cs[t + tid] - lo;
+    };
+
+    const int lpc_shift = a.lpc_shift, lw_shift = a.lw_shift;
+    const int LPC = 1 << lpc_shift, LW = 1 << lw_shift, TP = LPC >> lw_shift;
+    const int c16 = tid >> lpc_shift, lig = tid & (LPC - 1);
+    const int tp = lig >> lw_shift, lw = lig & (LW - 1);
+    float acc[1] = {0.f};
+    constexpr int TU = 2;  // tiles of one lane whose LDS reads are issued together
+
+    issue(0, min(TG, a.T), 0);
+    int which = 0;
+    for (int t = 0; t < a.T; t += TG, which ^= 1) {
+        const int nt = min(TG, a.T - t);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (t + TG < a.T) issue(t + TG, min(TG, a.T - t - TG), which ^ 1);
+        const XT* xs = reinterpret_cast<const XT*>(lds + which * stage_bytes);
+        const uint32_t* buf = reinterpret_cast<const uint32_t*>(lds + which * stage_bytes + a.xs_bytes);
+        const uint32_t* my_cst = cst + which * (TG + 1);
+        for (int tl0 = tp; tl0 < nt; tl0 += TP * TU) {
+            uint32_t d[TU];
+            const uint32_t* run[TU];
+#pragma unroll
+            for (int u = 0; u < TU; ++u) {
+                const int tl = tl0 + u * TP;
+                const uint32_t* chunk = buf + my_cst[min(tl, nt - 1)];
+                d[u] = tl < nt ? chunk[c16] : 0u;  // tiles past the group: empty run
+                run[u] = chunk + (d[u] >> 16);
+            }
+            uint32_t w[TU];
+#pragma unroll
+            for (int u = 0; u < TU; ++u)  // lanes past the run's end take an all-sentinel word: four gathers of zero
+                w[u] = lw < run_pos_dwords(d[u]) + run_neg_dwords(d[u]) ? run[u][lw] : 0xffffffffu;
+#pragma unroll
+            for (int u = 0; u < TU; ++u) {
+                const int pd = run_pos_dwords(d[u]), tot = pd + run_neg_dwords(d[u]);
+                if (u > 0 && __builtin_amdgcn_ballot_w64(tot > 0) == 0) continue;  // no lane of the wave has this tile
+                const XT* xt = xs + (size_t)min(tl0 + u * TP, nt - 1) * kTileSlots;
+                gather_add<1, XT>(acc, xt, w[u], lw < pd ? 1.0f : -1.0f);
+                for (int i = lw + LW; i < tot; i += LW)  // runs longer than the lane group
+                    gather_add<1, XT>(acc, xt, run[u][i], i < pd ? 1.0f : -1.0f);
+            }
+        }
+    }
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1)
+        if (off < LPC) acc[0] += __shfl_xor(acc[0], off, 64);
+    const int n = nb * TL_BLOCK_COLUMNS + c16;
+    if (lig == 0 && n < a.N) store_out(a.Y, a.y_f16, n, acc[0] * load_scale(a.w0.scale, a.scale_f16, n));
+}
+
+// ---------------------------------------------------------------------------
 // Activation re-layout for the row-parallel kernel: XT[k][m] (m contiguous, padded
 // with zeros to ldm columns) from row-major X[m][k] or K-major X[k][m].
 // ---------------------------------------------------------------------------
@@ -1288,6 +1388,44 @@ int launch_quad_kernel(KernelArgs a, const tl_layout_header* h, hipStream_t st)
     return TL_OK;
 }
 
+// The direct-load kernel for one activation row.  All of K in one group when `share` workgroups of that
+// size fit a compute unit, else two alternating buffers of TG tiles.
+template <bool XF16>
+int launch_spmv_direct(KernelArgs a, const tl_layout_header* h, hipStream_t st)
+{
+    constexpr int es = XF16 ? 2 : 4;
+    const int tile_bytes = kTileSlots * es;
+    const int chunk_bytes = (int)h->max_chunk_dwords * 4;
+    const int share = std::max(1, std::min(env_int("TL_SPMV_SHARE", 4), (int)ceil_div(a.NB, kComputeUnits)));
+    const int budget = 160 * 1024 / share - 1024;
+    int tg = a.T;
+    if ((int64_t)a.T * (tile_bytes + chunk_bytes) + 256 > budget) tg = std::max(1, (budget - 256) / (2 * (tile_bytes + chunk_bytes)));
+    tg = std::max(1, std::min(tg, env_int("TL_TILE_GROUP", tg)));
+    tg = (int)ceil_div(a.T, ceil_div(a.T, tg));  // same number of groups, evened out
+    a.tiles_per_group = tg;
+    a.xs_bytes = tg * tile_bytes;
+    a.buf_bytes = (int)round_up((int64_t)tg * chunk_bytes, 16);
+    const int buffers = tg < a.T ? 2 : 1;
+    const size_t lds = (size_t)buffers * ((size_t)a.xs_bytes + a.buf_bytes) + (size_t)buffers * (tg + 1) * 4;
+    if (lds > 160 * 1024) return fail(TL_ERR_UNSUPPORTED, "one tile needs %zu bytes of LDS", lds);
+    const int lpc = kBlockThreads / TL_BLOCK_COLUMNS;
+    const double mean_run = h->mean_run_dwords_x16 / 16.0;
+    int lw = 4;
+    while (lw < lpc && lw * 3 < mean_run) lw *= 2;
+    lw = std::min(env_int("TL_LW", lw), lpc);
+    if (lw < 1 || (lw & (lw - 1))) return fail(TL_ERR_ARG, "TL_LW=%d (a power of two expected)", lw);
+    a.lpc_shift = log2_exact(lpc);
+    a.lw_shift = log2_exact(lw);
+    auto kernel = tl_spmv_direct<XF16>;
+    static bool raised = false;  // per instantiation; a repeated or racing call is harmless
+    if (!raised) {
+        if (int rc = raise_lds_limit(kernel, 160 * 1024)) return rc;
+        raised = true;
+    }
+    hipLaunchKernelGGL(kernel, dim3((unsigned)a.NB), dim3(kBlockThreads), lds, st, a);
+    return TL_OK;
+}
+
 template <int MT>
 int launch_small_mt(const KernelArgs& a, const tl_layout_header* h, hipStream_t st)
 {
@@ -1333,6 +1471,10 @@ int launch_small(KernelArgs a, const tl_layout_header* h, int x_dtype, void* wor
         if (mt == 8) return a.x_f16 ? launch_quad_kernel<8, true>(a, h, st) : launch_quad_kernel<8, false>(a, h, st);
         return a.x_f16 ? launch_quad_kernel<16, true>(a, h, st) : launch_quad_kernel<16, false>(a, h, st);
     }
+    // one contiguous aligned row whose tiles are whole 16-byte pieces: straight copies into LDS
+    if (mt == 1 && a.x_sk == 1 && reinterpret_cast<uintptr_t>(a.X) % 16 == 0 && h->tile_rows % (16 / es) == 0 && a.K % (16 / es) == 0 &&
+        env_int("TL_SPMV_DIRECT", 1))
+        return a.x_f16 ? launch_spmv_direct<true>(a, h, st) : launch_spmv_direct<false>(a, h, st);
     // Column blocks per workgroup.  A compute unit works through ceil(workgroups / 256) workgroups of
     // `set` blocks each: the narrowest set that keeps that product smallest.
     int set = 1;
