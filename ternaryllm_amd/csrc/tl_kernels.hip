@@ -1,16 +1,19 @@
 // gfx950 kernels and launchers of libternary_spmm: Y = (X * W) * scale for a ternary W
 // held in the wave-tiled CSC blob (see tl_layout.cpp for the format).
 //
-// Two kernels replace the reference's pair
+// Four kernels replace the reference's pair
 // (ternaryLLM_GPU/csrc/ter_spmm_kernel.cuh:24-78 SpMV, :106-308 SpMM):
 //
-//   tl_spmm_block  M <= 48 (decode and small batches).  A workgroup owns 1, 2 or 4 blocks of 16
-//                  columns over all of K and streams their chunks and the matching
-//                  activation rows through LDS (activations in their own type, [slot][row]);
-//                  the lanes that share a column split each run, one dword = four 8-bit row
-//                  indices per lane and pass; every index is one LDS read of the slot's rows
-//                  and one accumulating op per row; the partial sums of a column are folded
-//                  with cross-lane shuffles.
+//   tl_spmv_direct M = 1 (decode), a contiguous aligned activation row.  A workgroup owns a block of
+//                  16 columns over all of K; its chunks and the row's tiles are copied straight into
+//                  LDS by direct global -> LDS loads, all in flight at once when K fits; the 32
+//                  lanes of a column split its runs, one dword = four 8-bit row indices per lane
+//                  and pass; every index is one LDS read and one accumulating op.
+//   tl_spmm_quad   M = 5 ... 48, slots of 8 or 16 rows from an aligned K-major image, staged the same
+//                  way; a lane owns four rows of a column, so a gather reads 16 slots as whole pieces.
+//   tl_spmm_block  M = 2 ... 4, and single rows that are strided or unaligned.  Owns 1, 2 or 4 blocks;
+//                  chunks and activations travel through registers into LDS (activations in
+//                  their own type, [slot][row]); partial sums folded with cross-lane shuffles.
 //   tl_spmm_rows   larger M (prefill).  Lanes own activation rows, a wave owns C
 //                  output columns, so an index is wave-uniform: it is read through
 //                  the scalar path once and serves 64*R rows; the activation tile
