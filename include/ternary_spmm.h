@@ -240,21 +240,25 @@ int tl_rope_cache_update(const void* qkv, int dtype, int64_t batch, int heads, i
  * (TernaryLLM/TernaryAttn.py:100-113), scores and softmax in fp32.
  *   q          device [batch][heads][head_dim]
  *   out        device [batch][heads * head_dim]
- * head_dim 64, 128 or 256; max_seq * 4 bytes of scores must fit 120 KB of LDS. */
+ * head_dim 64, 128 or 256; max_seq * 4 bytes of scores must fit 120 KB of LDS.
+ * out_kmajor_ld: 0, or the leading dimension (>= batch) of a K-major output [heads * head_dim][ld] --
+ * the layout tl_spmm multiplies 5 to 48 rows from without a re-layout pass (here and in the two
+ * functions below). */
 int tl_decode_attention(const void* q, const void* k_cache, const void* v_cache, int dtype,
                         int64_t batch, int heads, int head_dim, int64_t max_seq,
-                        const int64_t* pos_dev, void* out, void* stream);
+                        const int64_t* pos_dev, void* out, int64_t out_kmajor_ld, void* stream);
 
 /* x_out = x + y, h_out = RMSNorm(x_out) * weight, row by row ([rows][width], one dtype): the residual
  * add of a decoder layer fused with the normalisation that follows (the reference leaves both to the
  * Hugging Face Llama it patches, TernaryLLM/TernaryLlama.py:69-75).  y may be NULL: plain RMSNorm of x,
- * x_out then optional. */
+ * x_out then optional.  h_kmajor_ld: 0, or the leading dimension (>= rows) of a K-major h_out [width][ld]. */
 int tl_add_rmsnorm(const void* x, const void* y, const void* weight, int dtype, int64_t rows, int width,
-                   float eps, void* x_out, void* h_out, void* stream);
+                   float eps, void* x_out, void* h_out, int64_t h_kmajor_ld, void* stream);
 
 /* out[rows][width] = silu(gate_up[:, :width]) * gate_up[:, width:] for gate_up [rows][2 * width]: the
- * gate of LlamaTernaryMLP (TernaryLLM/TernaryMLP.py:33-35) on a side-by-side gate | up product. */
-int tl_silu_mul(const void* gate_up, int dtype, int64_t rows, int width, void* out, void* stream);
+ * gate of LlamaTernaryMLP (TernaryLLM/TernaryMLP.py:33-35) on a side-by-side gate | up product.
+ * out_kmajor_ld: 0, or the leading dimension (>= rows) of a K-major out [width][ld]. */
+int tl_silu_mul(const void* gate_up, int dtype, int64_t rows, int width, void* out, int64_t out_kmajor_ld, void* stream);
 
 #ifdef __cplusplus
 }

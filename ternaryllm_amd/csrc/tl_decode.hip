@@ -62,7 +62,8 @@ constexpr int kAttnThreads = 1024;
 template <typename T, int HD>
 __global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restrict__ q, const T* __restrict__ k_cache,
                                                                const T* __restrict__ v_cache, const long long* __restrict__ pos_p,
-                                                               T* __restrict__ out, int heads, long long max_seq, float scale)
+                                                               T* __restrict__ out, long long out_kld, int heads, long long max_seq,
+                                                               float scale)
 {
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int VE = 16 / (int)sizeof(T);   // values per 16-byte piece
@@ -158,7 +159,8 @@ __global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restri
         for (int g = 0; g < RG; ++g) sum += partial[g][tid];
         const long long b = bh / heads;
         const int h = (int)(bh % heads);
-        out[((size_t)b * heads + h) * HD + tid] = from_f<T>(sum / total);
+        const size_t col = (size_t)h * HD + tid;  // of the [batch][heads * head_dim] output
+        out[out_kld ? col * out_kld + b : (size_t)b * heads * HD + col] = from_f<T>(sum / total);
     }
 }
 
@@ -166,7 +168,7 @@ __global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restri
 // follows it in a decoder layer, one workgroup per row.  y may be null (plain RMSNorm of x).
 template <typename T>
 __global__ __launch_bounds__(256) void tl_add_rmsnorm_k(const T* __restrict__ x, const T* __restrict__ y, const T* __restrict__ weight,
-                                                        T* __restrict__ x_out, T* __restrict__ h_out, int width, float eps)
+                                                        T* __restrict__ x_out, T* __restrict__ h_out, long long h_kld, int width, float eps)
 {
     __shared__ float red[4];
     const size_t row = (size_t)blockIdx.x * width;
@@ -185,7 +187,7 @@ __global__ __launch_bounds__(256) void tl_add_rmsnorm_k(const T* __restrict__ x,
     for (int i = threadIdx.x; i < width; i += 256) {
         float v = to_f(x[row + i]);
         if (y) v = to_f(from_f<T>(v + to_f(y[row + i])));
-        h_out[row + i] = from_f<T>(v * inv * to_f(weight[i]));
+        h_out[h_kld ? (size_t)i * h_kld + blockIdx.x : row + i] = from_f<T>(v * inv * to_f(weight[i]));
     }
 }
 
@@ -193,7 +195,7 @@ __global__ __launch_bounds__(256) void tl_add_rmsnorm_k(const T* __restrict__ x,
 // workgroup: every value is read once, all loads of a thread are in flight together.
 template <typename T>
 __global__ __launch_bounds__(512) void tl_add_rmsnorm_vec(const T* __restrict__ x, const T* __restrict__ y, const T* __restrict__ weight,
-                                                          T* __restrict__ x_out, T* __restrict__ h_out, int width, float eps)
+                                                          T* __restrict__ x_out, T* __restrict__ h_out, long long h_kld, int width, float eps)
 {
     constexpr int VE = 16 / (int)sizeof(T);
     constexpr int NV = 4;
@@ -246,19 +248,39 @@ __global__ __launch_bounds__(512) void tl_add_rmsnorm_vec(const T* __restrict__ 
             T* oe = reinterpret_cast<T*>(&o);
 #pragma unroll
             for (int e = 0; e < VE; ++e) oe[e] = from_f<T>(val[k][e] * inv * to_f(we[e]));
-            *reinterpret_cast<uint4*>(h_out + row + ((size_t)threadIdx.x + k * 512) * VE) = o;
+            const size_t col = ((size_t)threadIdx.x + k * 512) * VE;
+            if (h_kld) {
+#pragma unroll
+                for (int e = 0; e < VE; ++e) h_out[(col + e) * h_kld + blockIdx.x] = oe[e];
+            } else {
+                *reinterpret_cast<uint4*>(h_out + row + col) = o;
+            }
         }
     }
 }
 
 // out[r][i] = silu(gu[r][i]) * gu[r][width + i]: the gate of the MLP on the side-by-side gate | up product.
+// With out_kld the result goes to a K-major image [width][out_kld]; threads then walk the image in its
+// own order (rows of one column side by side, stores contiguous), and the columns past `rows` are zeroed.
 template <typename T>
-__global__ __launch_bounds__(256) void tl_silu_mul_k(const T* __restrict__ gu, T* __restrict__ out, long long rows, int width)
+__global__ __launch_bounds__(256) void tl_silu_mul_k(const T* __restrict__ gu, T* __restrict__ out, long long out_kld, long long rows, int width)
 {
     const long long i = blockIdx.x * 256ll + threadIdx.x;
-    if (i >= rows * width) return;
-    const long long r = i / width;
-    const int c = (int)(i - r * width);
+    long long r;
+    int c;
+    if (out_kld) {
+        if (i >= out_kld * width) return;
+        c = (int)(i / out_kld);
+        r = i - c * out_kld;
+        if (r >= rows) {
+            out[i] = from_f<T>(0.0f);
+            return;
+        }
+    } else {
+        if (i >= rows * width) return;
+        r = i / width;
+        c = (int)(i - r * width);
+    }
     const float g = to_f(gu[(size_t)r * 2 * width + c]), u = to_f(gu[(size_t)r * 2 * width + width + c]);
     out[i] = from_f<T>(to_f(from_f<T>(g / (1.0f + __expf(-g)))) * u);  // the SiLU is rounded to T before the product, as two separate operators would
 }
@@ -281,7 +303,7 @@ int launched()
 
 template <typename T, int HD>
 int attn_launch(dim3 grid, size_t lds, hipStream_t st, const void* q, const void* k, const void* v, const long long* pos, void* out,
-                int heads, long long max_seq, float scale)
+                long long out_kld, int heads, long long max_seq, float scale)
 {
     auto kernel = tl_decode_attn<T, HD>;
     static bool raised = false;  // per instantiation; a repeated or racing call is harmless
@@ -291,18 +313,18 @@ int attn_launch(dim3 grid, size_t lds, hipStream_t st, const void* q, const void
         raised = true;
     }
     hipLaunchKernelGGL(kernel, grid, dim3(kAttnThreads), lds, st, static_cast<const T*>(q), static_cast<const T*>(k),
-                       static_cast<const T*>(v), pos, static_cast<T*>(out), heads, max_seq, scale);
+                       static_cast<const T*>(v), pos, static_cast<T*>(out), out_kld, heads, max_seq, scale);
     return TL_OK;
 }
 
 template <typename T>
 int attn_dispatch(int head_dim, dim3 grid, size_t lds, hipStream_t st, const void* q, const void* k, const void* v,
-                  const long long* pos, void* out, int heads, long long max_seq, float scale)
+                  const long long* pos, void* out, long long out_kld, int heads, long long max_seq, float scale)
 {
     switch (head_dim) {
-        case 64: return attn_launch<T, 64>(grid, lds, st, q, k, v, pos, out, heads, max_seq, scale);
-        case 128: return attn_launch<T, 128>(grid, lds, st, q, k, v, pos, out, heads, max_seq, scale);
-        case 256: return attn_launch<T, 256>(grid, lds, st, q, k, v, pos, out, heads, max_seq, scale);
+        case 64: return attn_launch<T, 64>(grid, lds, st, q, k, v, pos, out, out_kld, heads, max_seq, scale);
+        case 128: return attn_launch<T, 128>(grid, lds, st, q, k, v, pos, out, out_kld, heads, max_seq, scale);
+        case 256: return attn_launch<T, 256>(grid, lds, st, q, k, v, pos, out, out_kld, heads, max_seq, scale);
         default: return fail(TL_ERR_UNSUPPORTED, "head_dim=%d (64, 128 or 256 supported)", head_dim);
     }
 }
@@ -333,10 +355,11 @@ extern "C" int tl_rope_cache_update(const void* qkv, int dtype, int64_t batch, i
 }
 
 extern "C" int tl_decode_attention(const void* q, const void* k_cache, const void* v_cache, int dtype, int64_t batch, int heads,
-                                   int head_dim, int64_t max_seq, const int64_t* pos_dev, void* out, void* stream)
+                                   int head_dim, int64_t max_seq, const int64_t* pos_dev, void* out, int64_t out_kmajor_ld, void* stream)
 {
     if (int rc = check_common(dtype, batch, heads, head_dim, max_seq, pos_dev)) return rc;
     if (!q || !k_cache || !v_cache || !out) return fail(TL_ERR_ARG, "device pointer is null");
+    if (out_kmajor_ld && out_kmajor_ld < batch) return fail(TL_ERR_SHAPE, "out_kmajor_ld=%lld is less than the batch", (long long)out_kmajor_ld);
     const size_t lds = (size_t)max_seq * sizeof(float);
     if (lds > 120 * 1024) return fail(TL_ERR_UNSUPPORTED, "max_seq=%lld: the scores of one head must fit 120 KB of LDS", (long long)max_seq);
     if (reinterpret_cast<uintptr_t>(k_cache) % 16 || reinterpret_cast<uintptr_t>(v_cache) % 16 || reinterpret_cast<uintptr_t>(q) % 16)
@@ -346,19 +369,22 @@ extern "C" int tl_decode_attention(const void* q, const void* k_cache, const voi
     const long long* pos = reinterpret_cast<const long long*>(pos_dev);
     const float scale = 1.0f / sqrtf((float)head_dim);
     int rc;
-    if (dtype == TL_F16) rc = attn_dispatch<__half>(head_dim, grid, lds, st, q, k_cache, v_cache, pos, out, heads, (long long)max_seq, scale);
-    else rc = attn_dispatch<float>(head_dim, grid, lds, st, q, k_cache, v_cache, pos, out, heads, (long long)max_seq, scale);
+    if (dtype == TL_F16) rc = attn_dispatch<__half>(head_dim, grid, lds, st, q, k_cache, v_cache, pos, out, (long long)out_kmajor_ld, heads,
+                                                    (long long)max_seq, scale);
+    else rc = attn_dispatch<float>(head_dim, grid, lds, st, q, k_cache, v_cache, pos, out, (long long)out_kmajor_ld, heads, (long long)max_seq, scale);
     if (rc) return rc;
     return launched();
 }
 
 extern "C" int tl_add_rmsnorm(const void* x, const void* y, const void* weight, int dtype, int64_t rows, int width, float eps,
-                              void* x_out, void* h_out, void* stream)
+                              void* x_out, void* h_out, int64_t h_kmajor_ld, void* stream)
 {
     if (dtype != TL_F16 && dtype != TL_F32) return fail(TL_ERR_DTYPE, "dtype code %d unknown", dtype);
     if (!x || !weight || !h_out) return fail(TL_ERR_ARG, "device pointer is null");
     if (rows <= 0 || width <= 0 || rows > (1ll << 30)) return fail(TL_ERR_SHAPE, "rows and width must be positive");
     if (y && !x_out) return fail(TL_ERR_ARG, "x_out is needed when y is given");
+    if (h_kmajor_ld && h_kmajor_ld < rows) return fail(TL_ERR_SHAPE, "h_kmajor_ld=%lld is less than the rows", (long long)h_kmajor_ld);
+    const long long kld = (long long)h_kmajor_ld;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int ve = dtype == TL_F16 ? 8 : 4;
     auto aligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
@@ -366,36 +392,37 @@ extern "C" int tl_add_rmsnorm(const void* x, const void* y, const void* weight, 
         if (dtype == TL_F16)
             hipLaunchKernelGGL(tl_add_rmsnorm_vec<__half>, dim3((unsigned)rows), dim3(512), 0, st, static_cast<const __half*>(x),
                                static_cast<const __half*>(y), static_cast<const __half*>(weight), static_cast<__half*>(x_out),
-                               static_cast<__half*>(h_out), width, eps);
+                               static_cast<__half*>(h_out), kld, width, eps);
         else
             hipLaunchKernelGGL(tl_add_rmsnorm_vec<float>, dim3((unsigned)rows), dim3(512), 0, st, static_cast<const float*>(x),
                                static_cast<const float*>(y), static_cast<const float*>(weight), static_cast<float*>(x_out),
-                               static_cast<float*>(h_out), width, eps);
+                               static_cast<float*>(h_out), kld, width, eps);
         return launched();
     }
     if (dtype == TL_F16)
         hipLaunchKernelGGL(tl_add_rmsnorm_k<__half>, dim3((unsigned)rows), dim3(256), 0, st, static_cast<const __half*>(x),
                            static_cast<const __half*>(y), static_cast<const __half*>(weight), static_cast<__half*>(x_out),
-                           static_cast<__half*>(h_out), width, eps);
+                           static_cast<__half*>(h_out), kld, width, eps);
     else
         hipLaunchKernelGGL(tl_add_rmsnorm_k<float>, dim3((unsigned)rows), dim3(256), 0, st, static_cast<const float*>(x),
                            static_cast<const float*>(y), static_cast<const float*>(weight), static_cast<float*>(x_out),
-                           static_cast<float*>(h_out), width, eps);
+                           static_cast<float*>(h_out), kld, width, eps);
     return launched();
 }
 
-extern "C" int tl_silu_mul(const void* gate_up, int dtype, int64_t rows, int width, void* out, void* stream)
+extern "C" int tl_silu_mul(const void* gate_up, int dtype, int64_t rows, int width, void* out, int64_t out_kmajor_ld, void* stream)
 {
     if (dtype != TL_F16 && dtype != TL_F32) return fail(TL_ERR_DTYPE, "dtype code %d unknown", dtype);
     if (!gate_up || !out) return fail(TL_ERR_ARG, "device pointer is null");
     if (rows <= 0 || width <= 0 || rows * width > (1ll << 40)) return fail(TL_ERR_SHAPE, "rows and width must be positive");
+    if (out_kmajor_ld && out_kmajor_ld < rows) return fail(TL_ERR_SHAPE, "out_kmajor_ld=%lld is less than the rows", (long long)out_kmajor_ld);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const unsigned blocks = (unsigned)ceil_div(rows * width, 256);
+    const unsigned blocks = (unsigned)ceil_div((out_kmajor_ld ? out_kmajor_ld : rows) * width, 256);
     if (dtype == TL_F16)
         hipLaunchKernelGGL(tl_silu_mul_k<__half>, dim3(blocks), dim3(256), 0, st, static_cast<const __half*>(gate_up), static_cast<__half*>(out),
-                           (long long)rows, width);
+                           (long long)out_kmajor_ld, (long long)rows, width);
     else
         hipLaunchKernelGGL(tl_silu_mul_k<float>, dim3(blocks), dim3(256), 0, st, static_cast<const float*>(gate_up), static_cast<float*>(out),
-                           (long long)rows, width);
+                           (long long)out_kmajor_ld, (long long)rows, width);
     return launched();
 }

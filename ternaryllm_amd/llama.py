@@ -205,15 +205,18 @@ class TernaryLlamaDecoder(nn.Module):
         B = x.shape[0]
         q = torch.empty((B, c.num_attention_heads, c.head_dim), dtype=x.dtype, device=x.device)
         eps = c.rms_norm_eps
-        _, h = ops.add_rmsnorm(x, None, self.layers[0].input_layernorm.weight, eps)
+        # 5 to 48 rows: the products read a K-major image, so whatever feeds one writes it in that layout
+        # (its transpose as a view) and no re-layout pass runs in front of the products
+        km = 5 <= B <= 48 and c.hidden_size != B and c.intermediate_size != B
+        _, h = ops.add_rmsnorm(x, None, self.layers[0].input_layernorm.weight, eps, kmajor=km)
         for li, layer in enumerate(self.layers):
             qkv = layer.qkv_proj(h)
             ops.rope_cache_update(qkv, self.rope_cos, self.rope_sin, pos, q, self._cache[li, 0], self._cache[li, 1])
-            a = ops.decode_attention(q, self._cache[li, 0], self._cache[li, 1], pos)
-            x, h = ops.add_rmsnorm(x, layer.o_proj(a), layer.post_attention_layernorm.weight, eps)
-            y = layer.down_proj(ops.silu_mul(layer.gate_up_proj(h)))
+            a = ops.decode_attention(q, self._cache[li, 0], self._cache[li, 1], pos, kmajor=km)
+            x, h = ops.add_rmsnorm(x, layer.o_proj(a), layer.post_attention_layernorm.weight, eps, kmajor=km)
+            y = layer.down_proj(ops.silu_mul(layer.gate_up_proj(h), kmajor=km))
             nxt = self.layers[li + 1].input_layernorm.weight if li + 1 < len(self.layers) else self.norm.weight
-            x, h = ops.add_rmsnorm(x, y, nxt, eps)  # the residual add, and the norm the next layer (or the head) starts with
+            x, h = ops.add_rmsnorm(x, y, nxt, eps, kmajor=km)  # the residual add, and the norm the next layer (or the head) starts with
         return self.lm_head(h)
 
     @torch.no_grad()

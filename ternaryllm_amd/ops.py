@@ -203,52 +203,68 @@ def rope_cache_update(qkv, cos_table, sin_table, pos, q_out, k_cache, v_cache):
     return q_out
 
 
-def decode_attention(q, k_cache, v_cache, pos, out=None):
+def _kmajor_image(rows, width, like):
+    """An uninitialised K-major image [width][ld] for `rows` activation rows, ld = rows rounded up to 16: the
+    layout spmm multiplies 5 to 48 rows from without a re-layout pass.  Returns (buffer, ld)."""
+    ld = (rows + 15) // 16 * 16
+    return torch.empty((width, ld), dtype=like.dtype, device=like.device), ld
+
+
+def decode_attention(q, k_cache, v_cache, pos, out=None, kmajor=False):
     """Attention of one query per (batch row, head) over cache rows [0, pos].  q: [B, heads, head_dim];
-    caches: [B, heads, max_seq, head_dim]; pos: one-element int64 device tensor.  Returns [B, heads * head_dim]."""
+    caches: [B, heads, max_seq, head_dim]; pos: one-element int64 device tensor.  Returns [B, heads * head_dim],
+    or with kmajor its transpose [heads * head_dim, B] as a view of a K-major image (for spmm's x_layout=1)."""
     B, heads, max_seq, hd = k_cache.shape
-    if out is None:
+    ld = 0
+    if kmajor:
+        if out is not None:
+            raise ValueError("out= and kmajor exclude each other")
+        image, ld = _kmajor_image(B, heads * hd, q)
+        out = image
+    elif out is None:
         out = torch.empty((B, heads * hd), dtype=q.dtype, device=q.device)
     for t in (q, k_cache, v_cache, out):
         if not t.is_contiguous() or t.dtype != q.dtype or t.device != q.device:
             raise ValueError("tensors must be contiguous, of one dtype, on one device")
-    if q.numel() != B * heads * hd or out.numel() != B * heads * hd or v_cache.shape != k_cache.shape:
+    if q.numel() != B * heads * hd or out.numel() != max(B, ld) * heads * hd or v_cache.shape != k_cache.shape:
         raise ValueError("shapes of q, out and the caches do not agree")
     if pos.dtype != torch.int64 or pos.numel() != 1 or pos.device != q.device:
         raise ValueError("pos must be a one-element int64 tensor on the same device")
     with torch.cuda.device(q.device):
         rc = _lib.lib().tl_decode_attention(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), _code(q.dtype, "q"), B, heads, hd,
-                                            max_seq, pos.data_ptr(), out.data_ptr(), _stream_ptr(q.device))
+                                            max_seq, pos.data_ptr(), out.data_ptr(), ld, _stream_ptr(q.device))
     _lib.check(rc)
-    return out
+    return out[:, :B] if kmajor else out
 
 
-def add_rmsnorm(x, y, weight, eps):
+def add_rmsnorm(x, y, weight, eps, kmajor=False):
     """(x + y, rmsnorm(x + y) * weight) for [rows, width] tensors of one dtype; y may be None (then the
-    first result is x itself)."""
+    first result is x itself).  With kmajor the second result is its transpose [width, rows], a view of a
+    K-major image (for spmm's x_layout=1)."""
     if x.dim() != 2 or not x.is_contiguous() or weight.numel() != x.shape[1] or not weight.is_contiguous():
         raise ValueError("x must be a contiguous [rows, width] tensor and weight [width]")
     if y is not None and (y.shape != x.shape or y.dtype != x.dtype or not y.is_contiguous()):
         raise ValueError("y must match x")
     if weight.dtype != x.dtype:
         raise ValueError("weight must have x's dtype")
-    h = torch.empty_like(x)
+    h, ld = _kmajor_image(x.shape[0], x.shape[1], x) if kmajor else (torch.empty_like(x), 0)
     x_out = torch.empty_like(x) if y is not None else x
     with torch.cuda.device(x.device):
         rc = _lib.lib().tl_add_rmsnorm(x.data_ptr(), y.data_ptr() if y is not None else None, weight.data_ptr(), _code(x.dtype, "x"),
                                        x.shape[0], x.shape[1], float(eps), x_out.data_ptr() if y is not None else None, h.data_ptr(),
-                                       _stream_ptr(x.device))
+                                       ld, _stream_ptr(x.device))
     _lib.check(rc)
-    return x_out, h
+    return x_out, (h[:, :x.shape[0]] if kmajor else h)
 
 
-def silu_mul(gate_up):
-    """silu(gate_up[:, :w]) * gate_up[:, w:] for a contiguous [rows, 2 * w] tensor."""
+def silu_mul(gate_up, kmajor=False):
+    """silu(gate_up[:, :w]) * gate_up[:, w:] for a contiguous [rows, 2 * w] tensor; with kmajor the transpose
+    [w, rows] of that, a view of a K-major image (for spmm's x_layout=1)."""
     if gate_up.dim() != 2 or not gate_up.is_contiguous() or gate_up.shape[1] % 2:
         raise ValueError("gate_up must be a contiguous [rows, 2 * width] tensor")
     rows, w = gate_up.shape[0], gate_up.shape[1] // 2
-    out = torch.empty((rows, w), dtype=gate_up.dtype, device=gate_up.device)
+    out, ld = _kmajor_image(rows, w, gate_up) if kmajor else (torch.empty((rows, w), dtype=gate_up.dtype, device=gate_up.device), 0)
     with torch.cuda.device(gate_up.device):
-        rc = _lib.lib().tl_silu_mul(gate_up.data_ptr(), _code(gate_up.dtype, "gate_up"), rows, w, out.data_ptr(), _stream_ptr(gate_up.device))
+        rc = _lib.lib().tl_silu_mul(gate_up.data_ptr(), _code(gate_up.dtype, "gate_up"), rows, w, out.data_ptr(), ld, _stream_ptr(gate_up.device))
     _lib.check(rc)
-    return out
+    return out[:, :rows] if kmajor else out

@@ -94,6 +94,28 @@ def test_native_decode_step_matches_torch_operators(tiny, cuda):
     assert (outs[True][1] - outs[False][1]).abs().max().item() <= 2e-3 * outs[False][1].abs().max().item()
 
 
+def test_batched_decode_step_on_k_major_activations(tiny, cuda):
+    """Eight rows: the step keeps its activations as K-major images between the kernels; same check as above."""
+    g = torch.Generator().manual_seed(7)
+    B, S = 8, 20
+    tokens = torch.randint(0, tiny.config.vocab_size, (B, S + 2), generator=g).to(cuda)
+    outs = {}
+    for native in (False, True):
+        tiny.native_decode = native
+        tiny.prefill(tokens[:, :S])
+        st = tiny._decode_state(B)
+        logits = []
+        for j in range(2):
+            st["token"].copy_(tokens[:, S + j])
+            st["pos"].fill_(S + j)
+            st["mask"].copy_((torch.arange(tiny.max_seq_len, device=cuda) <= S + j)[None, None, None])
+            logits.append(tiny._decode_step(st["token"], st["pos"], st["mask"]).float())
+        outs[native] = torch.stack(logits)
+    tiny.native_decode = True
+    tiny._state = None
+    assert (outs[True] - outs[False]).abs().max().item() <= 1e-2 * outs[False].abs().max().item()
+
+
 def test_decode_kernels_against_fp32(cuda):
     """tl_rope_cache_update and tl_decode_attention alone, fp16 and fp32, against a float64 restatement."""
     from ternaryllm_amd import ops
@@ -126,6 +148,8 @@ def test_decode_kernels_against_fp32(cuda):
             sc = (q.double()[:, :, None, :] * kc.double()[:, :, : pos + 1]).sum(-1) / hd ** 0.5
             ref = (sc.softmax(-1)[..., None] * vc.double()[:, :, : pos + 1]).sum(2).reshape(B, H * hd)
             assert (out.double() - ref).abs().max().item() <= tol * 4
+            outk = ops.decode_attention(q, kc, vc, p, kmajor=True)   # the same values as a K-major image
+            assert outk.shape == (H * hd, B) and outk.stride(0) == 16 and torch.equal(outk.t(), out)
 
 
 def test_add_rmsnorm_and_silu_mul(cuda):
@@ -140,6 +164,8 @@ def test_add_rmsnorm_and_silu_mul(cuda):
             assert torch.equal(xs, x + y)
             ref = xs.double() * torch.rsqrt(xs.double().pow(2).mean(-1, keepdim=True) + 1e-5) * w.double()
             assert (h.double() - ref).abs().max().item() <= tol * ref.abs().max().item()
+            xk, hk = ops.add_rmsnorm(x, y, w, 1e-5, kmajor=True)     # the same values as a K-major image
+            assert torch.equal(xk, xs) and hk.shape == (width, rows) and hk.stride(0) % 16 == 0 and torch.equal(hk.t(), h)
             x0, h0 = ops.add_rmsnorm(x, None, w, 1e-5)
             assert x0 is x
             ref0 = x.double() * torch.rsqrt(x.double().pow(2).mean(-1, keepdim=True) + 1e-5) * w.double()
@@ -148,6 +174,7 @@ def test_add_rmsnorm_and_silu_mul(cuda):
             out = ops.silu_mul(gu)
             refs = torch.nn.functional.silu(gu[:, :width].double()) * gu[:, width:].double()
             assert (out.double() - refs).abs().max().item() <= tol * refs.abs().max().item()
+            assert torch.equal(ops.silu_mul(gu, kmajor=True).t(), out)
 
 
 def test_graph_replay_equals_eager_decode(tiny, cuda):
