@@ -283,6 +283,17 @@ def main():
         extra["c3_mlp_block_fused"] = {"ms": round(mlp_ms, 4), "tokens_per_s": round(M / (mlp_ms * 1e-3), 1)}
     if not args.no_extra:
         extra["c2_decode_cold_weights_graph"] = cold_decode_leg(dev)
+        if not args.no_cpu:
+            try:  # the reference's decode kernel (ported) on the host's cores, same W, beside config 2
+                from oracle import cpu_baseline
+                w2, pw2, _ = weight_and_packed(4096, 4096, 0.66, 1244, dev)
+                r2 = cpu_baseline.time_gemv(w2.numpy(), torch.randn(4096, generator=g).numpy(), runs=20)
+                B2 = 4 * int(pw2.nnz) + 4096 * 4 + 4096 * 4  # int32 indices, as the reference's decode format holds them
+                extra["c2_cpu_baseline"] = {"value": round(B2 / r2["seconds"] / 1e9, 3), "unit": "GB/s", "cores": r2["threads"], "kind": r2["kind"],
+                                            "kernel": r2["kernel"], "us": round(r2["seconds"] * 1e6, 1), "tokens_per_s": round(1 / r2["seconds"], 1),
+                                            "max_err_over_max": r2["max_err_over_max"]}
+            except Exception as e:  # noqa: BLE001 - the baseline is optional, the GPU figures are not
+                extra["c2_cpu_baseline"] = {"value": None, "sample": "failed: %s" % e}
         # the decoder's other products, one row and sixteen, over 24 cold copies each
         extra["decode_cold_shapes"] = [cold_decode_leg(dev, K, N, copies=24, calls=240, M=M)
                                        for K, N in ((4096, 4096), (4096, 11008), (11008, 4096)) for M in (1, 16)]

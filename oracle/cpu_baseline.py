@@ -159,3 +159,30 @@ def time_gemm(w, x, runs=10, prefer_reference=True, check=True):
     p.free(h)
     return {"seconds": dt, "kind": p.kind, "kernel": p.kernel_name, "threads": threads(), "max_rel_err": max_err,
             "cpu": cpu_model()}
+
+
+def time_gemv(w, x, runs=20):
+    """Times y = x @ W (one row) on the CPU with this repository's port of the reference's decode kernel
+    GEMV_CPU_FP32_rowMajor_TCSC_Merged_GroupMin_G64_AVX2_OpenMP (ternaryLLM_CPU/src/GEMM_CPU_FP32.cpp:15008-15081;
+    the reference's own file holds it behind aligned loads that fault under GCC, so the port is what runs).
+    w: int [K, N] ternary (N % 64 == 0), x: float [K].  Checked against the float64 product first."""
+    p = PortProvider()
+    K, N = w.shape
+    assert N % 64 == 0 and K < 32768
+    w8 = np.ascontiguousarray(w, dtype=np.int8)
+    xv = np.ascontiguousarray(x, np.float32)
+    y = np.zeros(N, np.float32)
+    h = p.L.port_group_build(w8.ctypes.data, K, N, 64, 0)
+    p.L.port_gemv_g64_avx2(xv.ctypes.data, h, y.ctypes.data, N, K)
+    ref = xv.astype(np.float64) @ w.astype(np.float64)
+    max_err = float(np.max(np.abs(y - ref)) / max(1e-9, np.abs(ref).max()))
+    if max_err > 1e-4:
+        p.L.port_group_free(h)
+        raise RuntimeError(f"CPU GEMV port disagrees with the exact product (max err / max {max_err})")
+    t0 = time.perf_counter()
+    for _ in range(runs):
+        p.L.port_gemv_g64_avx2(xv.ctypes.data, h, y.ctypes.data, N, K)
+    dt = (time.perf_counter() - t0) / runs
+    p.L.port_group_free(h)
+    return {"seconds": dt, "kind": "port", "kernel": "port of GEMV_CPU_FP32_rowMajor_TCSC_Merged_GroupMin_G64_AVX2_OpenMP",
+            "threads": threads(), "max_err_over_max": max_err, "cpu": cpu_model()}
