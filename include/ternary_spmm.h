@@ -240,7 +240,7 @@ int tl_rope_cache_update(const void* qkv, int dtype, int64_t batch, int heads, i
  * (TernaryLLM/TernaryAttn.py:100-113), scores and softmax in fp32.
  *   q          device [batch][heads][head_dim]
  *   out        device [batch][heads * head_dim]
- * head_dim 64, 128 or 256; max_seq * 4 bytes of scores must fit 120 KB of LDS.
+ * head_dim 64, 128 or 256; one pass over the cache (running maximum and sums), any max_seq.
  * out_kmajor_ld: 0, or the leading dimension (>= batch) of a K-major output [heads * head_dim][ld] --
  * the layout tl_spmm multiplies 5 to 48 rows from without a re-layout pass (here and in the two
  * functions below). */

@@ -54,10 +54,14 @@ __global__ __launch_bounds__(256) void tl_rope_cache(const T* __restrict__ qkv, 
 
 // One workgroup per (batch row, head): scores of the query against cache rows [0, pos], softmax in
 // fp32, weighted sum of the value rows.  out is [batch][heads * head_dim], the layout the output
-// projection multiplies.  A cache row is read as 16-byte pieces by CPR neighbouring lanes, and the
-// workgroup's 1024 threads work on 1024 / CPR rows side by side, so that with a few hundred rows
-// every thread has only a handful of independent loads to wait for.
+// projection multiplies (or its K-major image).  A cache row is read as 16-byte pieces by CPR
+// neighbouring lanes, and the workgroup's 1024 threads work on RG = 1024 / CPR rows side by side.
+// One pass over the cache: a row group takes NB of its rows at a time, key and value pieces of all of
+// them requested together, and keeps a running maximum, sum of exponentials and weighted sum (rescaled
+// when the maximum moves), so nothing waits for memory a second time; the RG running results are
+// combined through LDS at the end.
 constexpr int kAttnThreads = 1024;
+constexpr int kAttnBatch = 4;  // rows of a row group whose loads are in flight together
 
 template <typename T, int HD>
 __global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restrict__ q, const T* __restrict__ k_cache,
@@ -65,14 +69,13 @@ __global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restri
                                                                T* __restrict__ out, long long out_kld, int heads, long long max_seq,
                                                                float scale)
 {
-    extern __shared__ __align__(16) unsigned char smem[];
     constexpr int VE = 16 / (int)sizeof(T);   // values per 16-byte piece
     constexpr int CPR = HD / VE;              // lanes per cache row
-    constexpr int RG = kAttnThreads / CPR;    // rows in flight
+    constexpr int RG = kAttnThreads / CPR;    // row groups
+    constexpr int NB = kAttnBatch;
     static_assert(CPR <= 64 && (CPR & (CPR - 1)) == 0, "a row's lanes must sit in one wave");
-    float* score = reinterpret_cast<float*>(smem);  // [n]
-    __shared__ float red[kAttnThreads / 64];
     __shared__ float partial[RG][HD + 1];
+    __shared__ float group_max[RG], group_sum[RG];
     const int tid = threadIdx.x;
     const long long bh = blockIdx.x;
     long long n = *pos_p + 1;  // valid rows
@@ -103,64 +106,68 @@ __global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restri
 #pragma unroll
         for (int e = 0; e < VE; ++e) qv[e] = f[e] * scale;
     }
-    float local_max = -INFINITY;
-#pragma unroll 4
-    for (long long j = rg; j < n; j += RG) {
-        float f[VE];
-        unpack(*reinterpret_cast<const uint4*>(kc + (size_t)j * HD + c * VE), f);
-        float acc = 0.f;
-#pragma unroll
-        for (int e = 0; e < VE; ++e) acc = fmaf(f[e], qv[e], acc);
-#pragma unroll
-        for (int off = CPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
-        if (c == 0) score[j] = acc;
-        local_max = fmaxf(local_max, acc);
-    }
-    // block maximum
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) local_max = fmaxf(local_max, __shfl_xor(local_max, off, 64));
-    if ((tid & 63) == 0) red[tid >> 6] = local_max;
-    __syncthreads();
-    float m = red[0];
-#pragma unroll
-    for (int w = 1; w < kAttnThreads / 64; ++w) m = fmaxf(m, red[w]);
-    __syncthreads();
-    float local_sum = 0.f;
-    for (long long j = tid; j < n; j += kAttnThreads) {
-        const float e = __expf(score[j] - m);
-        score[j] = e;
-        local_sum += e;
-    }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) local_sum += __shfl_xor(local_sum, off, 64);
-    if ((tid & 63) == 0) red[tid >> 6] = local_sum;
-    __syncthreads();
-    float total = 0.f;
-#pragma unroll
-    for (int w = 0; w < kAttnThreads / 64; ++w) total += red[w];
-
-    // weighted sum of value rows: every row group folds its rows, then the groups are added up
+    float m = -INFINITY, l = 0.f;  // the same in all lanes of a row group
     float acc[VE];
 #pragma unroll
     for (int e = 0; e < VE; ++e) acc[e] = 0.f;
-#pragma unroll 4
-    for (long long j = rg; j < n; j += RG) {
-        float f[VE];
-        unpack(*reinterpret_cast<const uint4*>(vc + (size_t)j * HD + c * VE), f);
-        const float p = score[j];
+    for (long long j0 = rg; j0 < n; j0 += (long long)RG * NB) {
+        uint4 kk[NB], vv[NB];
 #pragma unroll
-        for (int e = 0; e < VE; ++e) acc[e] = fmaf(p, f[e], acc[e]);
+        for (int u = 0; u < NB; ++u) {
+            const long long j = min(j0 + (long long)u * RG, n - 1);  // past the end: the last row again, not used
+            kk[u] = *reinterpret_cast<const uint4*>(kc + (size_t)j * HD + c * VE);
+            vv[u] = *reinterpret_cast<const uint4*>(vc + (size_t)j * HD + c * VE);
+        }
+        float sc[NB];
+        float top = m;
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            float f[VE];
+            unpack(kk[u], f);
+            float dot = 0.f;
+#pragma unroll
+            for (int e = 0; e < VE; ++e) dot = fmaf(f[e], qv[e], dot);
+#pragma unroll
+            for (int off = CPR / 2; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
+            sc[u] = j0 + (long long)u * RG < n ? dot : -INFINITY;
+            top = fmaxf(top, sc[u]);
+        }
+        const float keep = __expf(m - top);  // m == -inf on the first turn: exp(-inf) = 0, and l, acc are 0
+        l *= keep;
+#pragma unroll
+        for (int e = 0; e < VE; ++e) acc[e] *= keep;
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            const float p = __expf(sc[u] - top);  // 0 for the rows past the end
+            float f[VE];
+            unpack(vv[u], f);
+            l += p;
+#pragma unroll
+            for (int e = 0; e < VE; ++e) acc[e] = fmaf(p, f[e], acc[e]);
+        }
+        m = top;
     }
 #pragma unroll
     for (int e = 0; e < VE; ++e) partial[rg][c * VE + e] = acc[e];
+    if (c == 0) {
+        group_max[rg] = m;   // -inf for a row group without rows
+        group_sum[rg] = l;
+    }
     __syncthreads();
     if (tid < HD) {
-        float sum = 0.f;
-        for (int g = 0; g < RG; ++g) sum += partial[g][tid];
+        float top = -INFINITY;
+#pragma unroll 8
+        for (int g = 0; g < RG; ++g) top = fmaxf(top, group_max[g]);
+        float norm = 0.f, o = 0.f;
+#pragma unroll 4
+        for (int g = 0; g < RG; ++g) {
+            const float wgt = group_max[g] == -INFINITY ? 0.f : __expf(group_max[g] - top);
+            norm = fmaf(group_sum[g], wgt, norm);
+            o = fmaf(partial[g][tid], wgt, o);
+        }
         const long long b = bh / heads;
-        const int h = (int)(bh % heads);
-        const size_t col = (size_t)h * HD + tid;  // of the [batch][heads * head_dim] output
-        out[out_kld ? col * out_kld + b : (size_t)b * heads * HD + col] = from_f<T>(sum / total);
+        const size_t col = (size_t)(bh % heads) * HD + tid;  // of the [batch][heads * head_dim] output
+        out[out_kld ? col * out_kld + b : (size_t)b * heads * HD + col] = from_f<T>(o / norm);
     }
 }
 
@@ -306,12 +313,6 @@ int attn_launch(dim3 grid, size_t lds, hipStream_t st, const void* q, const void
                 long long out_kld, int heads, long long max_seq, float scale)
 {
     auto kernel = tl_decode_attn<T, HD>;
-    static bool raised = false;  // per instantiation; a repeated or racing call is harmless
-    if (!raised) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 120 * 1024);
-        if (e != hipSuccess) return fail(TL_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-        raised = true;
-    }
     hipLaunchKernelGGL(kernel, grid, dim3(kAttnThreads), lds, st, static_cast<const T*>(q), static_cast<const T*>(k),
                        static_cast<const T*>(v), pos, static_cast<T*>(out), out_kld, heads, max_seq, scale);
     return TL_OK;
@@ -360,8 +361,7 @@ extern "C" int tl_decode_attention(const void* q, const void* k_cache, const voi
     if (int rc = check_common(dtype, batch, heads, head_dim, max_seq, pos_dev)) return rc;
     if (!q || !k_cache || !v_cache || !out) return fail(TL_ERR_ARG, "device pointer is null");
     if (out_kmajor_ld && out_kmajor_ld < batch) return fail(TL_ERR_SHAPE, "out_kmajor_ld=%lld is less than the batch", (long long)out_kmajor_ld);
-    const size_t lds = (size_t)max_seq * sizeof(float);
-    if (lds > 120 * 1024) return fail(TL_ERR_UNSUPPORTED, "max_seq=%lld: the scores of one head must fit 120 KB of LDS", (long long)max_seq);
+    const size_t lds = 0;
     if (reinterpret_cast<uintptr_t>(k_cache) % 16 || reinterpret_cast<uintptr_t>(v_cache) % 16 || reinterpret_cast<uintptr_t>(q) % 16)
         return fail(TL_ERR_ALIGN, "q and the caches must be 16-byte aligned");
     dim3 grid((unsigned)(batch * heads));

@@ -152,6 +152,23 @@ def test_decode_kernels_against_fp32(cuda):
             assert outk.shape == (H * hd, B) and outk.stride(0) == 16 and torch.equal(outk.t(), out)
 
 
+def test_decode_attention_over_a_long_cache(cuda):
+    """One pass with running sums: no bound on the cache length (40 000 rows here), few rows, and a
+    position past the end (all rows valid, nothing out of bounds)."""
+    from ternaryllm_amd import ops
+    g = torch.Generator().manual_seed(12)
+    B, H, hd, S = 1, 2, 64, 40000
+    q = torch.randn((B, H, hd), generator=g).to(torch.float16).to(cuda)
+    kc = torch.randn((B, H, S, hd), generator=g).to(torch.float16).to(cuda)
+    vc = torch.randn((B, H, S, hd), generator=g).to(torch.float16).to(cuda)
+    for pos in (0, 2, 1023, S - 1, S + 5):
+        n = min(pos, S - 1) + 1
+        out = ops.decode_attention(q, kc, vc, torch.tensor([pos], dtype=torch.long, device=cuda))
+        sc = (q.double()[:, :, None, :] * kc.double()[:, :, :n]).sum(-1) / hd ** 0.5
+        ref = (sc.softmax(-1)[..., None] * vc.double()[:, :, :n]).sum(2).reshape(B, H * hd)
+        assert (out.double() - ref).abs().max().item() <= 3e-3 * max(1.0, ref.abs().max().item()), pos
+
+
 def test_add_rmsnorm_and_silu_mul(cuda):
     from ternaryllm_amd import ops
     g = torch.Generator().manual_seed(10)

@@ -206,7 +206,6 @@ def test_compute_entry_points_reject_bad_arguments_before_any_launch():
     assert L.tl_rope_cache_update(fake, 1, 1, 2, 63, fake, fake, pos, fake, fake, fake, 16, None) < 0  # odd head_dim
     assert L.tl_rope_cache_update(fake, 1, 1, 2, 64, fake, fake, None, fake, fake, fake, 16, None) < 0  # no position
     assert L.tl_decode_attention(fake, fake, fake, 1, 1, 2, 96, 16, pos, fake, 0, None) < 0             # head_dim not served
-    assert L.tl_decode_attention(fake, fake, fake, 1, 1, 2, 64, 1 << 20, pos, fake, 0, None) < 0        # scores do not fit LDS
     assert L.tl_decode_attention(fake, fake, ctypes.c_void_p(4104), 1, 1, 2, 64, 16, pos, fake, 0, None) < 0  # unaligned cache
     assert L.tl_decode_attention(fake, fake, fake, 1, 6, 2, 64, 16, pos, fake, 4, None) < 0             # K-major leading dimension below the batch
     assert L.tl_add_rmsnorm(fake, None, fake, 9, 1, 64, 1e-5, None, fake, 0, None) < 0
