@@ -114,9 +114,12 @@ __global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restri
         uint4 kk[NB], vv[NB];
 #pragma unroll
         for (int u = 0; u < NB; ++u) {
-            const long long j = min(j0 + (long long)u * RG, n - 1);  // past the end: the last row again, not used
-            kk[u] = *reinterpret_cast<const uint4*>(kc + (size_t)j * HD + c * VE);
-            vv[u] = *reinterpret_cast<const uint4*>(vc + (size_t)j * HD + c * VE);
+            const long long j = j0 + (long long)u * RG;
+            kk[u] = vv[u] = make_uint4(0u, 0u, 0u, 0u);
+            if (j < n) {  // rows past the end are not fetched
+                kk[u] = *reinterpret_cast<const uint4*>(kc + (size_t)j * HD + c * VE);
+                vv[u] = *reinterpret_cast<const uint4*>(vc + (size_t)j * HD + c * VE);
+            }
         }
         float sc[NB];
         float top = m;
