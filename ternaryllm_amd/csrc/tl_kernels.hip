@@ -615,12 +615,11 @@ __global__ __launch_bounds__(kBlockThreads) void tl_spmm_quad(KernelArgs a)
 // (TP tiles side by side, LW lanes per run, one dword per lane and pass, two tiles' reads issued
 // together), and fold their sums with cross-lane shuffles.  When all of K fits the LDS there is a
 // single group: every load of the workgroup is in flight at once and nothing is staged twice.
-template <bool XF16>
-__global__ __launch_bounds__(kBlockThreads) void tl_spmv_direct(KernelArgs a)
+template <bool XF16, int NT>
+__global__ __launch_bounds__(NT) void tl_spmv_direct(KernelArgs a)
 {
     extern __shared__ __align__(16) unsigned char lds[];
     using XT = typename std::conditional<XF16, __half, float>::type;
-    constexpr int NT = kBlockThreads;
     constexpr int ES = (int)sizeof(XT);
     constexpr int VE = 16 / ES;                  // values per 16-byte piece
     constexpr int PPT = kTileSlots / VE;         // pieces per tile image
@@ -700,7 +699,7 @@ __global__ __launch_bounds__(kBlockThreads) void tl_spmv_direct(KernelArgs a)
         }
     }
 #pragma unroll
-    for (int off = 16; off > 0; off >>= 1)
+    for (int off = 32; off > 0; off >>= 1)
         if (off < LPC) acc[0] += __shfl_xor(acc[0], off, 64);
     const int n = nb * TL_BLOCK_COLUMNS + c16;
     if (lig == 0 && n < a.N) store_out(a.Y, a.y_f16, n, acc[0] * load_scale(a.w0.scale, a.scale_f16, n));
@@ -1393,8 +1392,8 @@ int launch_quad_kernel(KernelArgs a, const tl_layout_header* h, hipStream_t st)
 
 // The direct-load kernel for one activation row.  All of K in one group when `share` workgroups of that
 // size fit a compute unit, else two alternating buffers of TG tiles.
-template <bool XF16>
-int launch_spmv_direct(KernelArgs a, const tl_layout_header* h, hipStream_t st)
+template <bool XF16, int NT>
+int launch_spmv_direct_nt(KernelArgs a, const tl_layout_header* h, hipStream_t st)
 {
     constexpr int es = XF16 ? 2 : 4;
     const int tile_bytes = kTileSlots * es;
@@ -1411,7 +1410,7 @@ int launch_spmv_direct(KernelArgs a, const tl_layout_header* h, hipStream_t st)
     const int buffers = tg < a.T ? 2 : 1;
     const size_t lds = (size_t)buffers * ((size_t)a.xs_bytes + a.buf_bytes) + (size_t)buffers * (tg + 1) * 4;
     if (lds > 160 * 1024) return fail(TL_ERR_UNSUPPORTED, "one tile needs %zu bytes of LDS", lds);
-    const int lpc = kBlockThreads / TL_BLOCK_COLUMNS;
+    const int lpc = NT / TL_BLOCK_COLUMNS;
     const double mean_run = h->mean_run_dwords_x16 / 16.0;
     int lw = 4;
     while (lw < lpc && lw * 3 < mean_run) lw *= 2;
@@ -1419,14 +1418,23 @@ int launch_spmv_direct(KernelArgs a, const tl_layout_header* h, hipStream_t st)
     if (lw < 1 || (lw & (lw - 1))) return fail(TL_ERR_ARG, "TL_LW=%d (a power of two expected)", lw);
     a.lpc_shift = log2_exact(lpc);
     a.lw_shift = log2_exact(lw);
-    auto kernel = tl_spmv_direct<XF16>;
+    auto kernel = tl_spmv_direct<XF16, NT>;
     static bool raised = false;  // per instantiation; a repeated or racing call is harmless
     if (!raised) {
         if (int rc = raise_lds_limit(kernel, 160 * 1024)) return rc;
         raised = true;
     }
-    hipLaunchKernelGGL(kernel, dim3((unsigned)a.NB), dim3(kBlockThreads), lds, st, a);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)a.NB), dim3(NT), lds, st, a);
     return TL_OK;
+}
+
+// With no more blocks than compute units a workgroup has its compute unit to itself: 1024 threads
+// (64 lanes per column) then keep more gathers in flight than 512 do.
+template <bool XF16>
+int launch_spmv_direct(const KernelArgs& a, const tl_layout_header* h, hipStream_t st)
+{
+    const bool wide = env_int("TL_SPMV_WIDE", a.NB <= kComputeUnits ? 1 : 0) != 0;
+    return wide ? launch_spmv_direct_nt<XF16, 1024>(a, h, st) : launch_spmv_direct_nt<XF16, kBlockThreads>(a, h, st);
 }
 
 template <int MT>

@@ -200,8 +200,8 @@ def test_output_into_a_strided_buffer(cuda, oracle, dtype):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 def test_small_m_kernels_in_every_mode(cuda, oracle, dtype, monkeypatch):
     """The direct-load kernels in the modes a default launch of a small shape does not reach: 8- and 16-row
-    slots, one group of tiles or two alternating buffers, several lane groups per run or one; and the
-    register-staged kernel on a single row."""
+    slots, one group of tiles or two alternating buffers, several lane groups per run or one, 512 or 1024
+    threads for a single row; and the register-staged kernel on a single row."""
     from ternaryllm_amd import ops
     from ternaryllm_amd.packing import PackedWeight
     K, N = 2100, 200  # 9 tiles, the last one short; 13 column blocks, the last one narrow
@@ -211,7 +211,7 @@ def test_small_m_kernels_in_every_mode(cuda, oracle, dtype, monkeypatch):
     for M in (1, 6, 16, 37):
         x = activations(M, K, 72 + M, dtype, integer=True)
         ref = oracle.fast_product(x.double().numpy(), w)
-        extra = [{"TL_SPMV_DIRECT": "0"}] if M == 1 else [{"TL_SMALL_MT": "8"}, {"TL_SMALL_MT": "16"}, {"TL_SMALL_MT": "16", "TL_TILE_GROUP": "2"}]
+        extra = [{"TL_SPMV_DIRECT": "0"}, {"TL_SPMV_WIDE": "0"}, {"TL_SPMV_WIDE": "1"}, {"TL_SPMV_WIDE": "1", "TL_TILE_GROUP": "2"}] if M == 1 else [{"TL_SMALL_MT": "8"}, {"TL_SMALL_MT": "16"}, {"TL_SMALL_MT": "16", "TL_TILE_GROUP": "2"}]
         for env in settings + extra:
             for key, value in env.items():
                 monkeypatch.setenv(key, value)
