@@ -251,6 +251,20 @@ def main():
 
     # ---- the other regimes of the path ---------------------------------------
     if not args.no_extra:
+        # what a plain device copy reaches on this box, beside the 8 TB/s the fractions are quoted against
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(10):
+            dst.copy_(src)
+        e1.record()
+        torch.cuda.synchronize()
+        extra["device_copy_1GiB"] = {"GB_per_s_read_plus_write": round(2 * src.numel() * 10 / (e0.elapsed_time(e1) * 1e-3) / 1e9, 1),
+                                     "pct_hbm_peak": round(100 * 2 * src.numel() * 10 / (e0.elapsed_time(e1) * 1e-3) / 1e9 / HBM_PEAK_GBS, 1)}
+        del src, dst
         def one(name, M2, K2, N2, s2, dt, seed):
             w2, pw2, dw2 = weight_and_packed(K2, N2, s2, seed, dev)
             x2 = torch.randn((M2, K2), generator=g).to(dt).to(dev)
