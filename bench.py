@@ -234,6 +234,11 @@ def main():
         "gop_equiv_per_s": round(2.0 * M * K * N / (ev_ms * 1e-3) / 1e9, 1),
         "row_major_input_ms_per_step": round(wall_rm_ms, 5),
     }
+    # the reference's own statistic (benchmark_ternary_mlp.py:51-53,98): 100 single calls timed one by one,
+    # mean of the fastest 10; median and 10th percentile beside it
+    singles = sorted(ops.spmm_time(dw, xk, 1, sd, x_layout=_lib.TL_X_K_MAJOR)[0] for _ in range(100))
+    extra["headline_single_call_ms"] = {"best10_of_100_mean": round(best_k_mean(singles, 10), 5), "median": round(singles[50], 5),
+                                        "p10": round(singles[10], 5)}
 
     # ---- CPU baseline on the same W and X ------------------------------------
     if not args.no_cpu:
