@@ -16,8 +16,10 @@
  *   - host packers write into caller-provided arrays after a sizing call.
  *   - compute entry points enqueue on the hipStream_t passed as `void* stream`
  *     (NULL = the default stream) and return without synchronising.
- *   - all functions are re-entrant; there is no mutable global state besides the
- *     thread-local error text.
+ *   - all functions are re-entrant.  Process-wide state: the thread-local error text;
+ *     the tuning knobs, read from the environment at the first launch (TL_* variables,
+ *     see tl_reload_options); the compute-unit count of each device, asked once; and
+ *     set-once flags that record that a kernel's LDS limit has been raised.
  */
 #ifndef TERNARY_SPMM_H
 #define TERNARY_SPMM_H
@@ -54,6 +56,12 @@ extern "C" {
 
 const char* tl_last_error(void);
 int tl_version(void);
+
+/* The launchers' tuning knobs (environment variables TL_SMALL_LDS, TL_TILE_GROUP, TL_QUAD_SHARE, TL_LW,
+ * TL_SPMV_SHARE, TL_SPMV_WIDE, TL_SMALL_MT, TL_SPMV_DIRECT, TL_BLOCK_SET, TL_ROWS_SPLIT; unset = the
+ * launcher's own choice) are read once per process.  This reads them again -- for tests and tuning runs
+ * that change them between calls. */
+int tl_reload_options(void);
 
 /* ======================================================================== */
 /* Host packers: bit-exact replacements of the reference's converters.      */
@@ -116,14 +124,18 @@ int tl_tiled_mcsc_to_dense(const void* merged_row, int index_width, int64_t n_in
 /*     multiple of 16 bytes.                                                */
 /*   - descriptor: +1 count (bits 0-7), -1 count (bits 8-15), dword offset  */
 /*     of the column's runs from the start of the chunk (bits 16-31).       */
+/*   - the rows of a run may come in any order; a row may repeat (it is     */
+/*     then added that many times) and may sit in both runs (it cancels):   */
+/*     a blob built from dense ternary weights holds every row once, one    */
+/*     built from the reference's merged arrays holds what they encode.     */
 /*   - the stream is block-major: all tiles of block 0, then block 1, ...;  */
 /*     chunkstart[block * T + tile] is the dword where a chunk begins       */
 /*     (one extra entry marks the end).                                     */
 /* The blob starts with a tl_layout_header (256 bytes).                     */
 /* ======================================================================== */
 
-#define TL_LAYOUT_MAGIC 0x34474C54u /* "TLG4" */
-#define TL_LAYOUT_VERSION 4
+#define TL_LAYOUT_MAGIC 0x35474C54u /* "TLG5" */
+#define TL_LAYOUT_VERSION 5
 #define TL_BLOCK_COLUMNS 16
 
 typedef struct tl_layout_header {
@@ -143,7 +155,8 @@ typedef struct tl_layout_header {
     uint64_t total_bytes;    /* bytes of the blob that are in use, multiple of 256                        */
     uint32_t max_run_dwords; /* largest (+1 run dwords + -1 run dwords) of any (column, tile)             */
     uint32_t mean_run_dwords_x16; /* mean of the same, times 16, rounded up                               */
-    uint32_t reserved[42];
+    uint64_t checksum;       /* FNV-1a (64-bit, one step per dword) over the chunk table and the stream   */
+    uint32_t reserved[40];
 } tl_layout_header;
 
 /* Bytes of the blob that tl_layout_build will write for these tiled-CSC arrays
@@ -163,10 +176,25 @@ int tl_layout_build(const int32_t* neg_row, const int32_t* neg_off_tiled,
 int tl_layout_from_dense(const int32_t* w, int columns, int inners, int tile_rows,
                          void* blob, int64_t* blob_bytes);
 
-/* Validates a host copy of a blob (header, bounds, monotone offsets, sentinel use). */
+/* Builds the blob straight from the reference's merged tiled-CSC arrays
+ * (convert_to_ter_tiled_mcsc, ter_spmm_wrapper.cu:156-315; index_width 2 = int16 as
+ * TernaryLinear stores them, TernaryLinear.py:110, or 4), so that the product through
+ * it is what the reference kernels' walk of those arrays adds up
+ * (ter_spmm_kernel.cuh:197-300): per tile the pairs (+x[p] - x[n]) over
+ * [off0, off1), then sign * x[c] over [off1, off2).  A row that the arrays name
+ * several times (possible with padded arrays) is added that many times.
+ * `uniformed` != 0 leaves the [off1, off2) part out, as the reference's kernels do
+ * when that flag is set (ter_spmm_kernel.cuh:59,249).
+ * Call with blob == NULL to get blob_bytes only. */
+int tl_layout_from_mcsc(const void* merged_row, int index_width, int64_t n_index,
+                        const int32_t* merged_off, int columns, int inners, int tile_k,
+                        int uniformed, int tile_rows, void* blob, int64_t* blob_bytes);
+
+/* Validates a host copy of a blob (header, bounds, monotone offsets, row range, sentinel use, checksum). */
 int tl_layout_validate(const void* blob, int64_t blob_bytes);
 
-/* Decodes a host blob back to dense int32 [inners][columns] (round-trip check). */
+/* Decodes a host blob back to dense int32 [inners][columns] (round-trip check): an entry is the
+ * number of times its row sits in the column's +1 run minus the times it sits in the -1 run. */
 int tl_layout_to_dense(const void* blob, int64_t blob_bytes, int32_t* w_out);
 
 /* ======================================================================== */

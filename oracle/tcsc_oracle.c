@@ -239,8 +239,10 @@ void orc_dense_product(const double *x, const int32_t *w, double *y, int M, int 
 /* (+x[p] - x[n]) over [off0, off1), then sign * sum x[c] over [off1, off2). */
 /* Every gather uses the tile's row offset (the SpMV remainder loop at :63   */
 /* omits it; that omission is a defect, not part of the format).             */
+/* uniformed != 0: the [off1, off2) part is skipped, as both kernels do under */
+/* their UNIFORMED template flag (ter_spmm_kernel.cuh:59, :249).              */
 void orc_mcsc_product(const double *x, const int32_t *merged_row, const int32_t *merged_off,
-                      double *y, int M, int N, int K, int tile_k)
+                      double *y, int M, int N, int K, int tile_k, int uniformed)
 {
     const int T = ceil_div(K, tile_k);
     for (int m = 0; m < M; m++)
@@ -251,6 +253,7 @@ void orc_mcsc_product(const double *x, const int32_t *merged_row, const int32_t 
                 const double *xt = x + (size_t)m * K + (size_t)t * tile_k;
                 for (int i = o[0]; i < o[1]; i += 2)
                     acc += xt[merged_row[i]] - xt[merged_row[i + 1]];
+                if (uniformed) continue;
                 double part = 0.0;
                 for (int i = o[1]; i < o[2]; i++) part += xt[merged_row[i]];
                 acc += (double)o[3] * part;

@@ -108,14 +108,15 @@ def dense_product(x, w):
     return y
 
 
-def mcsc_product(x, merged_row, merged_off, N, tile_k):
+def mcsc_product(x, merged_row, merged_off, N, tile_k, uniformed=False):
+    """What the reference kernels add up when they walk merged arrays (ter_spmm_kernel.cuh:197-300)."""
     x = np.ascontiguousarray(x, dtype=np.float64)
     M, K = x.shape
     merged_row = np.ascontiguousarray(merged_row, dtype=np.int32)
     merged_off = np.ascontiguousarray(merged_off, dtype=np.int32)
     y = np.zeros((M, N), np.float64)
     lib().orc_mcsc_product(_p(x, ctypes.c_double), _p(merged_row, ctypes.c_int32), _p(merged_off, ctypes.c_int32),
-                           _p(y, ctypes.c_double), M, N, K, tile_k)
+                           _p(y, ctypes.c_double), M, N, K, tile_k, int(bool(uniformed)))
     return y
 
 

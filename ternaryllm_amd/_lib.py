@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(_DIR, "libternary_spmm.so")
 TL_F32, TL_F16 = 0, 1
 TL_X_ROW_MAJOR, TL_X_K_MAJOR = 0, 1
 TL_ACT_SILU_GATE = 1
-TL_LAYOUT_MAGIC = 0x34474C54
+TL_LAYOUT_MAGIC = 0x35474C54
 
 ERROR_NAMES = {
     -1: "TL_ERR_ARG", -2: "TL_ERR_SHAPE", -3: "TL_ERR_DTYPE", -4: "TL_ERR_ALIGN", -5: "TL_ERR_UNSUPPORTED",
@@ -34,7 +34,7 @@ class LayoutHeader(ctypes.Structure):
         ("off_chunkstart", ctypes.c_uint64), ("off_stream", ctypes.c_uint64),
         ("stream_bytes", ctypes.c_uint64), ("total_bytes", ctypes.c_uint64),
         ("max_run_dwords", ctypes.c_uint32), ("mean_run_dwords_x16", ctypes.c_uint32),
-        ("reserved", ctypes.c_uint32 * 42),
+        ("checksum", ctypes.c_uint64), ("reserved", ctypes.c_uint32 * 40),
     ]
 
 
@@ -51,6 +51,7 @@ _I64 = ctypes.c_int64
 SIGNATURES = {
     "tl_last_error": (ctypes.c_char_p, []),
     "tl_version": (_INT, []),
+    "tl_reload_options": (_INT, []),
     "tl_count_nnz": (_INT, [_I32P, _INT, _INT, _I64P, _I64P]),
     "tl_convert_to_ter_csc": (_INT, [_I32P, _INT, _INT, _INT, _INT, _I32P, _I32P, _I32P, _I32P]),
     "tl_convert_to_ter_tiled_csc": (_INT, [_I32P, _INT, _INT, _INT, _INT, _INT, _I32P, _I32P, _I32P, _I32P]),
@@ -60,6 +61,7 @@ SIGNATURES = {
     "tl_layout_size": (_INT, [_I32P, _I32P, _INT, _INT, _INT, _INT, _I64P]),
     "tl_layout_build": (_INT, [_I32P, _I32P, _I32P, _I32P, _INT, _INT, _INT, _INT, _VP, _I64]),
     "tl_layout_from_dense": (_INT, [_I32P, _INT, _INT, _INT, _VP, _I64P]),
+    "tl_layout_from_mcsc": (_INT, [_VP, _INT, _I64, _I32P, _INT, _INT, _INT, _INT, _INT, _VP, _I64P]),
     "tl_layout_validate": (_INT, [_VP, _I64]),
     "tl_layout_to_dense": (_INT, [_VP, _I64, _I32P]),
     "tl_spmm_workspace": (_INT, [_HDRP, _I64, _INT, _INT, _I64P]),

@@ -1,8 +1,11 @@
-"""LlamaTernaryAttention: four ternary projections around dense causal attention
+"""LlamaTernaryAttention: four ternary projections around dense softmax attention, with the
+constructor and the forward contract of the reference's module
 (ternaryLLM_GPU/TernaryLLM/TernaryAttn.py:15-127).  The reference borrows rotary embedding,
-repeat_kv and the KV cache from the `transformers` package; here they are a textbook RoPE, an
-expand, and a plain (k, v) tuple, and the softmax attention is torch's
-scaled_dot_product_attention."""
+repeat_kv and the KV cache from the `transformers` package; here the rotary embedding is a
+textbook rotate-half RoPE, repeat_kv an expand, and the cache may be a `transformers` Cache
+(anything with its `update(key, value, layer_idx, cache_kwargs)`) or a plain (k, v) tuple."""
+import math
+
 import torch
 from torch import nn
 
@@ -18,10 +21,12 @@ def rope_tables(positions, head_dim, theta, dtype, device):
 
 
 def apply_rope(x, cos, sin):
-    """x: [batch, heads, seq, head_dim]."""
+    """x: [batch, heads, seq, head_dim]; cos/sin: [seq, head_dim] or [batch, seq, head_dim]."""
     half = x.shape[-1] // 2
     rot = torch.cat([-x[..., half:], x[..., :half]], dim=-1)
-    return x * cos[None, None] + rot * sin[None, None]
+    if cos.dim() == 2:
+        cos, sin = cos[None], sin[None]
+    return x * cos[:, None] + rot * sin[:, None]
 
 
 class LlamaTernaryAttention(nn.Module):
@@ -31,11 +36,16 @@ class LlamaTernaryAttention(nn.Module):
         self.layer_idx = layer_idx
         self.hidden_size = config.hidden_size
         self.num_heads = config.num_attention_heads
-        self.head_dim = self.hidden_size // self.num_heads
+        self.head_dim = getattr(config, "head_dim", None) or self.hidden_size // self.num_heads
         self.num_key_value_heads = config.num_key_value_heads
         self.num_key_value_groups = self.num_heads // self.num_key_value_heads
+        self.max_position_embeddings = getattr(config, "max_position_embeddings", None)
         self.rope_theta = config.rope_theta
         self.attention_dropout = config.attention_dropout
+        # The reference sets this and never reads it: it applies whatever mask the caller passes and none
+        # when there is no mask (TernaryAttn.py:38,103-105).  Here a forward without a mask is causal
+        # while this is True; set it to False for the reference's literal behaviour.
+        self.is_causal = True
 
         def make(k, n):
             return TernaryLinear(k, n, sparsity=config.sparsity, uniform=config.uniform_sparsity,
@@ -48,29 +58,94 @@ class LlamaTernaryAttention(nn.Module):
         self.v_proj = make(self.hidden_size, self.num_key_value_heads * self.head_dim)
         self.o_proj = make(self.num_heads * self.head_dim, self.hidden_size)
 
-    def forward(self, hidden_states, past_key_value=None, position_offset=0, use_cache=False):
-        """hidden_states: [batch, seq, hidden]; past_key_value: optional (k, v) of
-        [batch, kv_heads, past, head_dim].  Returns (output, present) with present = (k, v) or None."""
+    def _rotary(self, position_ids, position_embeddings, q_len, past_len, dtype, device):
+        if position_embeddings is not None:   # computed by the model, as newer `transformers` do
+            cos, sin = position_embeddings
+            return cos.to(dtype), sin.to(dtype)
+        if position_ids is None:
+            position_ids = torch.arange(past_len, past_len + q_len, device=device)
+        if position_ids.dim() == 1:
+            return rope_tables(position_ids, self.head_dim, self.rope_theta, dtype, device)
+        cos, sin = rope_tables(position_ids.reshape(-1), self.head_dim, self.rope_theta, dtype, device)
+        return cos.view(*position_ids.shape, -1), sin.view(*position_ids.shape, -1)
+
+    def forward(self, hidden_states, attention_mask=None, position_ids=None, past_key_value=None, output_attentions=False,
+                use_cache=False, cache_position=None, position_embeddings=None, *, position_offset=None, **kwargs):
+        """The reference's signature and 3-tuple result (TernaryAttn.py:59-70,127):
+        (attn_output [batch, seq, hidden], attn_weights or None, past_key_value).
+
+        attention_mask: additive, broadcastable to [batch, heads, q_len, kv_len]; longer masks are cut to
+        the key length as in the reference (:103-105).  position_embeddings: (cos, sin) of
+        [batch or 1, q_len, head_dim], else they are computed from position_ids ([q_len] or
+        [batch, q_len]), else from the cache length.  past_key_value: a `transformers` Cache (updated in
+        place with `layer_idx`; newer versions pass it as `past_key_values`) or a (k, v) tuple of
+        [batch, kv_heads, past, head_dim]; with a tuple, or with use_cache and no cache, the third
+        result is the new (k, v) tuple.  position_offset: position of the first token when neither
+        position_ids nor position_embeddings are given (default: the tuple cache's length)."""
+        if past_key_value is None:
+            past_key_value = kwargs.pop("past_key_values", None)
         bsz, q_len, _ = hidden_states.shape
-        q = self.q_proj(hidden_states).view(bsz, q_len, self.num_heads, self.head_dim).transpose(1, 2)
-        k = self.k_proj(hidden_states).view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
-        v = self.v_proj(hidden_states).view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
-        pos = torch.arange(position_offset, position_offset + q_len, device=hidden_states.device)
-        cos, sin = rope_tables(pos, self.head_dim, self.rope_theta, q.dtype, q.device)
+        q = self.q_proj(hidden_states).view(bsz, q_len, -1, self.head_dim).transpose(1, 2)
+        k = self.k_proj(hidden_states).view(bsz, q_len, -1, self.head_dim).transpose(1, 2)
+        v = self.v_proj(hidden_states).view(bsz, q_len, -1, self.head_dim).transpose(1, 2)
+        is_tuple = isinstance(past_key_value, (tuple, list))
+        past_len = position_offset
+        if past_len is None:
+            past_len = past_key_value[0].shape[2] if is_tuple else 0
+        cos, sin = self._rotary(position_ids, position_embeddings, q_len, past_len, q.dtype, q.device)
         q, k = apply_rope(q, cos, sin), apply_rope(k, cos, sin)
-        if past_key_value is not None:
+        if is_tuple:
             k = torch.cat([past_key_value[0], k], dim=2)
             v = torch.cat([past_key_value[1], v], dim=2)
-        present = (k, v) if use_cache else None
+            past_key_value = (k, v)
+        elif past_key_value is not None:
+            k, v = past_key_value.update(k, v, self.layer_idx, {"sin": sin, "cos": cos, "cache_position": cache_position})
+        elif use_cache:
+            past_key_value = (k, v)
+        kv_len = k.shape[2]
         if self.num_key_value_groups > 1:
             k = k.repeat_interleave(self.num_key_value_groups, dim=1)
             v = v.repeat_interleave(self.num_key_value_groups, dim=1)
-        causal = past_key_value is None and q_len > 1
-        if past_key_value is not None and q_len > 1:
-            raise ValueError("a multi-token step on top of a cache is not supported")
-        attn = torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=causal)
-        attn = attn.transpose(1, 2).reshape(bsz, q_len, self.num_heads * self.head_dim)
-        return self.o_proj(attn), present
+        if attention_mask is not None:
+            mask = attention_mask[..., :kv_len]
+            if mask.dtype != torch.bool:
+                mask = mask.to(q.dtype)
+        elif self.is_causal and q_len > 1:
+            # query i sits at key position kv_len - q_len + i
+            mask = torch.ones((q_len, kv_len), dtype=torch.bool, device=q.device).tril(kv_len - q_len)
+        else:
+            mask = None
+        dropout = self.attention_dropout if self.training else 0.0
+        if output_attentions:
+            # the reference's eager form (TernaryAttn.py:101-110): scores, fp32 softmax, weights returned
+            scores = torch.matmul(q, k.transpose(2, 3)) / math.sqrt(self.head_dim)
+            if mask is not None:
+                scores = scores.masked_fill(~mask, float("-inf")) if mask.dtype == torch.bool else scores + mask
+            attn_weights = torch.softmax(scores, dim=-1, dtype=torch.float32).to(q.dtype)
+            attn = torch.matmul(nn.functional.dropout(attn_weights, p=dropout, training=self.training), v)
+        else:
+            attn_weights = None
+            attn = nn.functional.scaled_dot_product_attention(q, k, v, attn_mask=mask, dropout_p=dropout)
+        attn = attn.transpose(1, 2).reshape(bsz, q_len, -1)
+        return self.o_proj(attn), attn_weights, past_key_value
 
 
-__all__ = ["LlamaTernaryAttention", "rope_tables", "apply_rope"]
+def collect_attn_linear_layers(model):
+    """(name, module) of the nn.Linear attention projections under `model` (TernaryAttn.py:134-140)."""
+    return [(name, m) for name, m in model.named_modules()
+            if isinstance(m, nn.Linear) and any(tag in name for tag in ("q_proj", "k_proj", "v_proj", "o_proj"))]
+
+
+def replace_linear_layers(layers, attn, sparsity=0.8, *, generator=None, reference_buffers=False):
+    """Puts a random TernaryLinear of the same shape in the place of each listed projection of the
+    attention module `attn` and moves it to the GPU (TernaryAttn.py:142-147; `layers` as returned by
+    collect_attn_linear_layers(attn))."""
+    for name, module in layers:
+        ternary = TernaryLinear(module.in_features, module.out_features, sparsity, False, generator=generator,
+                                reference_buffers=reference_buffers).to("cuda")
+        parent_name, _, leaf = name.rpartition(".")
+        setattr(attn.get_submodule(parent_name) if parent_name else attn, leaf, ternary)
+    torch.cuda.empty_cache()
+
+
+__all__ = ["LlamaTernaryAttention", "rope_tables", "apply_rope", "collect_attn_linear_layers", "replace_linear_layers"]

@@ -26,6 +26,8 @@
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
+#include <atomic>
 #include <cstdlib>
 #include <cstring>
 #include <type_traits>
@@ -768,7 +770,8 @@ struct RunFetcher {
 #pragma unroll
         for (int c = 0; c < C; ++c) d[c] = dp[c];
     }
-    // Reads past the wave's piece stay inside the blob (it ends with spare bytes) and are never used.
+    // NPRE * 64 dwords from the start of the wave's piece, whatever its length: what lies past the piece is
+    // never used, and past the stream's end the blob keeps as many spare bytes (tl_layout.cpp, kStreamSpareBytes).
     __device__ __forceinline__ void indices(WaveRuns<C>& r, uint32_t chunk) const
     {
         r.base = chunk + (r.d[0] >> 16);
@@ -1248,10 +1251,54 @@ constexpr int kRowsColsPlain = 8;  // columns per wave of the plain kernel: an a
 
 inline int rows_mtile(int x_dtype) { return x_dtype == TL_F16 ? 256 : 128; }
 
-int env_int(const char* name, int fallback)
+// Tuning knobs (environment variables of the same names).  They are read once, at the first launch of the
+// process; tl_reload_options() reads them again.  A knob that is not set leaves the launcher's own choice.
+enum Knob { TL_SMALL_LDS, TL_TILE_GROUP, TL_QUAD_SHARE, TL_LW, TL_SPMV_SHARE, TL_SPMV_WIDE, TL_SMALL_MT, TL_SPMV_DIRECT,
+            TL_BLOCK_SET, TL_ROWS_SPLIT, kKnobCount };
+const char* const kKnobNames[kKnobCount] = {"TL_SMALL_LDS", "TL_TILE_GROUP", "TL_QUAD_SHARE", "TL_LW", "TL_SPMV_SHARE", "TL_SPMV_WIDE",
+                                            "TL_SMALL_MT", "TL_SPMV_DIRECT", "TL_BLOCK_SET", "TL_ROWS_SPLIT"};
+struct Knobs {
+    bool set[kKnobCount];
+    int value[kKnobCount];
+};
+std::atomic<const Knobs*> g_knobs{nullptr};
+
+const Knobs* read_knobs()
 {
-    const char* v = std::getenv(name);
-    return v && *v ? std::atoi(v) : fallback;
+    Knobs* k = new Knobs;
+    for (int i = 0; i < kKnobCount; ++i) {
+        const char* v = std::getenv(kKnobNames[i]);
+        k->set[i] = v && *v;
+        k->value[i] = k->set[i] ? std::atoi(v) : 0;
+    }
+    return k;
+}
+
+int knob(Knob which, int fallback)
+{
+    const Knobs* k = g_knobs.load(std::memory_order_acquire);
+    if (!k) {
+        const Knobs* fresh = read_knobs();
+        if (g_knobs.compare_exchange_strong(k, fresh, std::memory_order_acq_rel)) k = fresh;
+        else delete fresh;  // another thread was first; k now holds its table
+    }
+    return k->set[which] ? k->value[which] : fallback;
+}
+
+// Compute units of the current device, asked once per device.  Launch shapes are sized by it; the row
+// kernel's one-workgroup-per-unit launch is capped at kMaxComputeUnits, which sizes its partial-sum area.
+constexpr int kMaxComputeUnits = 256;
+int compute_units()
+{
+    static std::atomic<int> cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return kMaxComputeUnits;
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = kMaxComputeUnits;
+        cached[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
 }
 
 WeightPtrs weight_ptrs(const tl_layout_header* h, const void* blob_dev, const void* scale)
@@ -1307,7 +1354,6 @@ inline int64_t small_kmajor_bytes(const tl_layout_header* h, int64_t M, int x_dt
 // with no more workgroups than compute units lets each have (nearly) all of it.
 constexpr int kSmallLdsShared = 78 * 1024;
 constexpr int kSmallLdsAlone = 158 * 1024;
-constexpr int kComputeUnits = 256;
 
 template <int MT, bool XF16>
 int launch_block_kernel(KernelArgs a, const tl_layout_header* h, hipStream_t st)
@@ -1318,14 +1364,14 @@ int launch_block_kernel(KernelArgs a, const tl_layout_header* h, hipStream_t st)
     const int64_t chunk_bytes = (int64_t)h->max_chunk_dwords * 4;
     if (chunk_bytes * a.block_set > Shape::kStreamCap) return fail(TL_ERR_UNSUPPORTED, "a tile's chunks do not fit the staging registers");
     const unsigned gx = (unsigned)ceil_div(a.NB, a.block_set), gy = (unsigned)ceil_div(a.M, MT);
-    const int budget = env_int("TL_SMALL_LDS", (int64_t)gx * gy <= kComputeUnits ? kSmallLdsAlone : kSmallLdsShared);
+    const int budget = knob(TL_SMALL_LDS, (int64_t)gx * gy <= compute_units() ? kSmallLdsAlone : kSmallLdsShared);
     // tiles per group: bounded by the registers of the staging (Shape), by the LDS budget shared between
     // the activation image and the chunk copies, and by the stream bytes one group may hold
     const int per_tile = tile_bytes + (int)chunk_bytes * a.block_set;
     int tg = std::min(Shape::kTiles, (budget - 1024) / per_tile);
     tg = std::min(tg, (int)(Shape::kStreamCap / (chunk_bytes * a.block_set)));
     tg = std::max(1, std::min(std::min(tg, a.T), 255));
-    tg = std::max(1, std::min(tg, env_int("TL_TILE_GROUP", tg)));
+    tg = std::max(1, std::min(tg, knob(TL_TILE_GROUP, tg)));
     tg = (int)ceil_div(a.T, ceil_div(a.T, tg));  // same number of groups, evened out
     a.tiles_per_group = tg;
     a.xs_bytes = tg * tile_bytes;
@@ -1360,10 +1406,10 @@ int launch_quad_kernel(KernelArgs a, const tl_layout_header* h, hipStream_t st)
     const int tile_bytes = kTileSlots * MT * es;
     const int chunk_bytes = (int)h->max_chunk_dwords * 4;
     const unsigned gx = (unsigned)a.NB, gy = (unsigned)ceil_div(a.M, MT);
-    const int share = std::max(1, std::min(env_int("TL_QUAD_SHARE", 4), (int)ceil_div((int64_t)gx * gy, kComputeUnits)));
+    const int share = std::max(1, std::min(knob(TL_QUAD_SHARE, 4), (int)ceil_div((int64_t)gx * gy, compute_units())));
     const int budget = 160 * 1024 / share - 1024;
     int tg = std::max(1, std::min(a.T, (budget - 256) / (2 * (tile_bytes + chunk_bytes))));
-    tg = std::max(1, std::min(tg, env_int("TL_TILE_GROUP", tg)));
+    tg = std::max(1, std::min(tg, knob(TL_TILE_GROUP, tg)));
     tg = (int)ceil_div(a.T, ceil_div(a.T, tg));  // same number of groups, evened out
     a.tiles_per_group = tg;
     a.xs_bytes = tg * tile_bytes;
@@ -1376,7 +1422,7 @@ int launch_quad_kernel(KernelArgs a, const tl_layout_header* h, hipStream_t st)
     int lw = 2;
     while (lw < groups && lw * 8 < mean_run) lw *= 2;
     while (groups / lw > tg) lw *= 2;
-    lw = std::min(env_int("TL_LW", lw), groups);
+    lw = std::min(knob(TL_LW, lw), groups);
     if (lw < 1 || (lw & (lw - 1))) return fail(TL_ERR_ARG, "TL_LW=%d (a power of two expected)", lw);
     a.lpc_shift = log2_exact(groups);
     a.lw_shift = log2_exact(lw);
@@ -1398,11 +1444,11 @@ int launch_spmv_direct_nt(KernelArgs a, const tl_layout_header* h, hipStream_t s
     constexpr int es = XF16 ? 2 : 4;
     const int tile_bytes = kTileSlots * es;
     const int chunk_bytes = (int)h->max_chunk_dwords * 4;
-    const int share = std::max(1, std::min(env_int("TL_SPMV_SHARE", 4), (int)ceil_div(a.NB, kComputeUnits)));
+    const int share = std::max(1, std::min(knob(TL_SPMV_SHARE, 4), (int)ceil_div(a.NB, compute_units())));
     const int budget = 160 * 1024 / share - 1024;
     int tg = a.T;
     if ((int64_t)a.T * (tile_bytes + chunk_bytes) + 256 > budget) tg = std::max(1, (budget - 256) / (2 * (tile_bytes + chunk_bytes)));
-    tg = std::max(1, std::min(tg, env_int("TL_TILE_GROUP", tg)));
+    tg = std::max(1, std::min(tg, knob(TL_TILE_GROUP, tg)));
     tg = (int)ceil_div(a.T, ceil_div(a.T, tg));  // same number of groups, evened out
     a.tiles_per_group = tg;
     a.xs_bytes = tg * tile_bytes;
@@ -1414,7 +1460,7 @@ int launch_spmv_direct_nt(KernelArgs a, const tl_layout_header* h, hipStream_t s
     const double mean_run = h->mean_run_dwords_x16 / 16.0;
     int lw = 4;
     while (lw < lpc && lw * 3 < mean_run) lw *= 2;
-    lw = std::min(env_int("TL_LW", lw), lpc);
+    lw = std::min(knob(TL_LW, lw), lpc);
     if (lw < 1 || (lw & (lw - 1))) return fail(TL_ERR_ARG, "TL_LW=%d (a power of two expected)", lw);
     a.lpc_shift = log2_exact(lpc);
     a.lw_shift = log2_exact(lw);
@@ -1433,7 +1479,7 @@ int launch_spmv_direct_nt(KernelArgs a, const tl_layout_header* h, hipStream_t s
 template <bool XF16>
 int launch_spmv_direct(const KernelArgs& a, const tl_layout_header* h, hipStream_t st)
 {
-    const bool wide = env_int("TL_SPMV_WIDE", a.NB <= kComputeUnits ? 1 : 0) != 0;
+    const bool wide = knob(TL_SPMV_WIDE, a.NB <= compute_units() ? 1 : 0) != 0;
     return wide ? launch_spmv_direct_nt<XF16, 1024>(a, h, st) : launch_spmv_direct_nt<XF16, kBlockThreads>(a, h, st);
 }
 
@@ -1449,8 +1495,8 @@ int launch_small(KernelArgs a, const tl_layout_header* h, int x_dtype, void* wor
     while (mt < a.M && mt < 16) mt *= 2;
     // 16-row slots with no more workgroups than compute units: 8-row slots give twice the workgroups,
     // each with half the LDS image, so that two share a compute unit and hide each other's waits.
-    if (mt == 16 && (int64_t)a.NB * ceil_div(a.M, 16) <= kComputeUnits) mt = 8;
-    mt = env_int("TL_SMALL_MT", mt);
+    if (mt == 16 && (int64_t)a.NB * ceil_div(a.M, 16) <= compute_units()) mt = 8;
+    mt = knob(TL_SMALL_MT, mt);
     if (mt != 1 && mt != 2 && mt != 4 && mt != 8 && mt != 16) return fail(TL_ERR_ARG, "TL_SMALL_MT=%d (1, 2, 4, 8 or 16 expected)", mt);
     const int es = x_dtype == TL_F16 ? 2 : 4;
     a.x_sm = a.x_kmajor ? 1 : a.ldx;
@@ -1484,20 +1530,21 @@ int launch_small(KernelArgs a, const tl_layout_header* h, int x_dtype, void* wor
     }
     // one contiguous aligned row whose tiles are whole 16-byte pieces: straight copies into LDS
     if (mt == 1 && a.x_sk == 1 && reinterpret_cast<uintptr_t>(a.X) % 16 == 0 && h->tile_rows % (16 / es) == 0 && a.K % (16 / es) == 0 &&
-        env_int("TL_SPMV_DIRECT", 1))
+        knob(TL_SPMV_DIRECT, 1))
         return a.x_f16 ? launch_spmv_direct<true>(a, h, st) : launch_spmv_direct<false>(a, h, st);
     // Column blocks per workgroup.  A compute unit works through ceil(workgroups / 256) workgroups of
     // `set` blocks each: the narrowest set that keeps that product smallest.
     int set = 1;
     {
         int64_t best = -1;
+        const int cus = compute_units();
         for (int cand = 1; cand <= kMaxBlockSet; cand *= 2) {
             if ((int64_t)h->max_chunk_dwords * 4 * cand > BlockShape<1, 2, kBlockThreads>::kStreamCap) break;
-            const int64_t cost = ceil_div(ceil_div(a.NB, cand), kComputeUnits) * cand;
+            const int64_t cost = ceil_div(ceil_div(a.NB, cand), cus) * cand;
             if (best < 0 || cost < best) { best = cost; set = cand; }
         }
     }
-    set = env_int("TL_BLOCK_SET", set);
+    set = knob(TL_BLOCK_SET, set);
     if (set != 1 && set != 2 && set != 4) return fail(TL_ERR_ARG, "TL_BLOCK_SET=%d (1, 2 or 4 expected)", set);
     a.block_set = set;
     const int lpc = kBlockThreads / (TL_BLOCK_COLUMNS * set);
@@ -1506,7 +1553,7 @@ int launch_small(KernelArgs a, const tl_layout_header* h, int x_dtype, void* wor
     const double mean_run = h->mean_run_dwords_x16 / 16.0;
     int lw = 4;
     while (lw < lpc && lw * 3 < mean_run) lw *= 2;
-    lw = std::min(env_int("TL_LW", lw), lpc);
+    lw = std::min(knob(TL_LW, lw), lpc);
     if (lw != 1 && lw != 2 && lw != 4 && lw != 8 && lw != 16 && lw != 32) return fail(TL_ERR_ARG, "TL_LW=%d (a power of two up to 32 expected)", lw);
     a.lpc_shift = log2_exact(lpc);
     a.lw_shift = log2_exact(lw);
@@ -1530,7 +1577,7 @@ int launch_small(KernelArgs a, const tl_layout_header* h, int x_dtype, void* wor
 
 // Bytes of partial sums the row kernel may leave when K tiles are shared out (both weight sets of the
 // fused gate/up kernel): two slots per workgroup of a one-workgroup-per-compute-unit launch.
-constexpr int64_t kRowsPartialBytes = (int64_t)kComputeUnits * 2 * 2 * kRowsWaves * kRowsCols * 4 * 64 * sizeof(float);
+constexpr int64_t kRowsPartialBytes = (int64_t)kMaxComputeUnits * 2 * 2 * kRowsWaves * kRowsCols * 4 * 64 * sizeof(float);
 static_assert(kRowsColsPlain == 2 * kRowsCols, "one accumulator set of the plain kernel is as large as the fused kernel's two");
 
 template <typename XT, int R, bool GATED>
@@ -1555,16 +1602,17 @@ int launch_rows_t(KernelArgs a, void* partial, int64_t partial_bytes, hipStream_
     // unit is launched instead: each works through an equal number of whole output tiles, the tiles
     // left over are shared out by (output tile, K tile) steps, and a second small launch adds up the
     // partial sums of those.
-    const int64_t rounds = ceil_div(units, kComputeUnits);
-    const bool uneven = (double)rounds * kComputeUnits > 1.06 * (double)units;
-    const bool want = env_int("TL_ROWS_SPLIT", uneven && units * a.T >= 4 * kComputeUnits ? 1 : 0) != 0;
-    const int64_t leftover = units % kComputeUnits;  // output tiles beyond an equal number of whole ones per workgroup
+    const int G = std::min(compute_units(), kMaxComputeUnits);  // workgroups of a one-per-compute-unit launch
+    const int64_t rounds = ceil_div(units, G);
+    const bool uneven = (double)rounds * G > 1.06 * (double)units;
+    const bool want = knob(TL_ROWS_SPLIT, uneven && units * a.T >= 4 * G ? 1 : 0) != 0;
+    const int64_t leftover = units % G;  // output tiles beyond an equal number of whole ones per workgroup
     if (want && leftover && partial && partial_bytes >= kRowsPartialBytes && reinterpret_cast<uintptr_t>(partial) % 16 == 0 && a.T >= 2) {
-        a.whole_units = (int)(units / kComputeUnits);
-        a.split_first_unit = a.whole_units * kComputeUnits;
+        a.whole_units = (int)(units / G);
+        a.split_first_unit = a.whole_units * G;
         a.split_steps = leftover * a.T;
         a.partial = static_cast<float*>(partial);
-        hipLaunchKernelGGL(kernel, dim3(kComputeUnits), dim3(kRowsWaves * 64), lds, st, a);
+        hipLaunchKernelGGL(kernel, dim3((unsigned)G), dim3(kRowsWaves * 64), lds, st, a);
         // LDS of the fix-up: the staged output tile (fp32 at most, padded rows)
         const size_t fix_lds = (size_t)MTILE * (kRowsWaves * COLS * 4 + 16);
         auto fixup = tl_rows_fixup<XT, R, COLS, kRowsWaves, GATED>;
@@ -1573,7 +1621,7 @@ int launch_rows_t(KernelArgs a, void* partial, int64_t partial_bytes, hipStream_
             if (int rc = raise_lds_limit(fixup, fix_lds)) return rc;
             fix_raised = true;
         }
-        hipLaunchKernelGGL(fixup, dim3((unsigned)leftover), dim3(kRowsWaves * 64), fix_lds, st, a, kComputeUnits);
+        hipLaunchKernelGGL(fixup, dim3((unsigned)leftover), dim3(kRowsWaves * 64), fix_lds, st, a, G);
         return TL_OK;
     }
     a.split_steps = 0;
@@ -1660,6 +1708,13 @@ int check_io(const void* blob_dev, const void* X, void* Y, int x_dtype, int x_la
 }
 
 }  // namespace
+
+extern "C" int tl_reload_options(void)
+{
+    const Knobs* old = g_knobs.exchange(read_knobs(), std::memory_order_acq_rel);
+    (void)old;  // a launch on another thread may still be reading it: the few bytes are left alone
+    return TL_OK;
+}
 
 extern "C" int tl_spmm_workspace(const tl_layout_header* header, int64_t M, int x_dtype, int x_layout, int64_t* workspace_bytes)
 {

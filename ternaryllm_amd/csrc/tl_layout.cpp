@@ -11,6 +11,7 @@
 //   - groups columns in blocks of 16 and stores, block-major, one self-describing chunk per
 //     (block, tile): 16 descriptors followed by the block's runs.  What a workgroup needs
 //     for a range of tiles is then a single contiguous piece of memory.
+#include <climits>
 #include <cstring>
 #include <algorithm>
 #include <vector>
@@ -43,6 +44,12 @@ int pick_geometry(int columns, int inners, int tile_rows, Geometry* g)
     return TL_OK;
 }
 
+// What kernels may read past the end of the stream: 192 dwords from the start of a wave's piece
+// (the piece may be empty and start at the stream's last dword) or 63 dwords past a piece's end.
+constexpr int kSparePrefetchDwords = 192;
+constexpr int64_t kStreamSpareBytes = 1024;
+static_assert(kStreamSpareBytes >= kSparePrefetchDwords * 4, "the spare must cover the index prefetch");
+
 struct Sections {
     int64_t off_chunkstart, off_stream, total;
 };
@@ -52,8 +59,9 @@ Sections place_sections(const Geometry& g, int64_t stream_bytes)
     Sections s;
     s.off_chunkstart = 256;
     s.off_stream = s.off_chunkstart + round_up(((int64_t)g.n_tiles * g.n_blocks + 1) * 4, 256);
-    // 512 spare bytes behind the stream: kernels fetch whole vectors past a chunk's end.
-    s.total = s.off_stream + round_up(stream_bytes, 256) + 512;
+    // Spare bytes behind the stream: the row kernel requests a wave's first kSparePrefetchDwords index
+    // dwords from wherever its piece starts, also when the piece is the stream's last and shorter.
+    s.total = s.off_stream + round_up(stream_bytes, 256) + kStreamSpareBytes;
     return s;
 }
 
@@ -78,10 +86,21 @@ int count_device_tiles(const int32_t* row, const int32_t* off_tiled, int columns
                 const int64_t k = (int64_t)t * tile_k + row[i];
                 if (row[i] < 0 || row[i] >= tile_k || k >= inners)
                     return fail(TL_ERR_FORMAT, "column %d tile %d: local row %d out of range", y, t, row[i]);
-                (*counts)[(size_t)(k / g.tile_rows) * columns + y]++;
+                uint16_t& c = (*counts)[(size_t)(k / g.tile_rows) * columns + y];
+                if (c == 0xffffu) return fail(TL_ERR_UNSUPPORTED, "column %d: more than 65535 entries in one tile", y);
+                ++c;
             }
         }
     return TL_OK;
+}
+
+// FNV-1a, 64-bit, one step per dword, over the chunk table (with its end entry) and the stream.
+uint64_t content_checksum(const uint32_t* chunkstart, size_t n_table, const uint32_t* stream, size_t n_stream)
+{
+    uint64_t h = 0xcbf29ce484222325ull;
+    for (size_t i = 0; i < n_table; ++i) h = (h ^ chunkstart[i]) * 0x100000001b3ull;
+    for (size_t i = 0; i < n_stream; ++i) h = (h ^ stream[i]) * 0x100000001b3ull;
+    return h;
 }
 
 // Last "end" entry of a tiled-CSC offset array = number of stored rows of that sign.
@@ -150,7 +169,8 @@ extern "C" int tl_layout_build(const int32_t* neg_row, const int32_t* neg_off_ti
                     p = cp[(size_t)t * columns + y];
                     n = cn[(size_t)t * columns + y];
                 }
-                if (p > 255 || n > 255) return fail(TL_ERR_FORMAT, "column %d tile %d holds %u/%u rows of one sign", y, t, p, n);
+                if (p > 255 || n > 255)
+                    return fail(TL_ERR_UNSUPPORTED, "column %d tile %d names %u/%u rows of one sign (255 at most)", y, t, p, n);
                 if ((dwords + j) * 4 >= (uint64_t)reserve) return fail(TL_ERR_SIZE, "stream reserve exceeded");
                 desc[j] = make_desc(p, n, in_chunk);
                 const uint32_t run = (p + 3) / 4 + (n + 3) / 4;
@@ -216,6 +236,7 @@ extern "C" int tl_layout_build(const int32_t* neg_row, const int32_t* neg_off_ti
     h.total_bytes = (uint64_t)place_sections(g, (int64_t)dwords * 4).total;
     h.max_run_dwords = run_max;
     h.mean_run_dwords_x16 = (uint32_t)ceil_div((int64_t)run_sum * 16, (int64_t)columns * T);
+    h.checksum = content_checksum(chunkstart, (size_t)NB * T + 1, stream, (size_t)dwords);
     std::memcpy(blob, &h, sizeof(h));
     return TL_OK;
 }
@@ -246,6 +267,56 @@ extern "C" int tl_layout_from_dense(const int32_t* w, int columns, int inners, i
     if (*blob_bytes < need) return fail(TL_ERR_SIZE, "blob has %lld bytes, %lld needed", (long long)*blob_bytes, (long long)need);
     return tl_layout_build(neg_row.data(), neg_off.data(), pos_row.data(), pos_off.data(), columns, inners, g.tile_rows,
                            g.tile_rows, blob, *blob_bytes);
+}
+
+extern "C" int tl_layout_from_mcsc(const void* merged_row, int index_width, int64_t n_index,
+                                   const int32_t* merged_off, int columns, int inners, int tile_k,
+                                   int uniformed, int tile_rows, void* blob, int64_t* blob_bytes)
+{
+    if (!merged_off || !blob_bytes || (n_index > 0 && !merged_row)) return fail(TL_ERR_ARG, "null pointer");
+    if (columns <= 0 || inners <= 0 || tile_k <= 0) return fail(TL_ERR_SHAPE, "bad dimensions");
+    if (index_width != 2 && index_width != 4) return fail(TL_ERR_DTYPE, "index_width=%d (2 or 4 expected)", index_width);
+    const int T = (int)ceil_div(inners, tile_k);
+    const int16_t* r16 = static_cast<const int16_t*>(merged_row);
+    const int32_t* r32 = static_cast<const int32_t*>(merged_row);
+    auto at = [&](int64_t i) -> int32_t { return index_width == 2 ? (int32_t)r16[i] : r32[i]; };
+    // The walk of the reference kernels, turned into the two row lists of every (column, tile):
+    // tiled CSC whose rows may repeat and come in the order the merged stream names them.
+    std::vector<int32_t> pos_off((size_t)columns * T * 2), neg_off((size_t)columns * T * 2);
+    std::vector<int32_t> pos_row, neg_row;
+    for (int y = 0; y < columns; ++y)
+        for (int t = 0; t < T; ++t) {
+            const int32_t* o = merged_off + ((size_t)y * T + t) * 4;
+            if (o[0] < 0 || o[1] < o[0] || o[2] < o[1] || o[2] > n_index || ((o[1] - o[0]) & 1) || (o[3] != 1 && o[3] != -1))
+                return fail(TL_ERR_FORMAT, "column %d tile %d: offsets [%d,%d,%d,%d] are not a merged tile", y, t, o[0],
+                            o[1], o[2], o[3]);
+            const size_t c = ((size_t)y * T + t) * 2;
+            pos_off[c] = (int32_t)pos_row.size();
+            neg_off[c] = (int32_t)neg_row.size();
+            const int64_t end = uniformed ? o[1] : o[2];
+            for (int64_t i = o[0]; i < end; ++i) {
+                const int32_t r = at(i);
+                if (r < 0 || r >= tile_k || (int64_t)t * tile_k + r >= inners)
+                    return fail(TL_ERR_FORMAT, "column %d tile %d: row index %d out of range", y, t, r);
+                const bool plus = i < o[1] ? ((i - o[0]) & 1) == 0 : o[3] > 0;
+                (plus ? pos_row : neg_row).push_back(r);
+            }
+            if (pos_row.size() > (size_t)INT32_MAX || neg_row.size() > (size_t)INT32_MAX)
+                return fail(TL_ERR_UNSUPPORTED, "more than 2^31 entries of one sign");
+            pos_off[c + 1] = (int32_t)pos_row.size();
+            neg_off[c + 1] = (int32_t)neg_row.size();
+        }
+    int64_t need = 0;
+    if (int rc = tl_layout_size(neg_off.data(), pos_off.data(), columns, inners, tile_k, tile_rows, &need)) return rc;
+    if (!blob) {
+        *blob_bytes = need;
+        return TL_OK;
+    }
+    if (*blob_bytes < need) return fail(TL_ERR_SIZE, "blob has %lld bytes, %lld needed", (long long)*blob_bytes, (long long)need);
+    pos_row.push_back(0);  // never read; keeps data() non-null for an all-zero weight
+    neg_row.push_back(0);
+    return tl_layout_build(neg_row.data(), neg_off.data(), pos_row.data(), pos_off.data(), columns, inners, tile_k, tile_rows,
+                           blob, *blob_bytes);
 }
 
 extern "C" int tl_layout_validate(const void* blob, int64_t blob_bytes)
@@ -292,8 +363,7 @@ extern "C" int tl_layout_validate(const void* blob, int64_t blob_bytes)
                     const uint32_t cnt = sign ? n : p, padded = sign ? 4 * nd : 4 * pd;
                     for (uint32_t i = 0; i < padded; ++i) {
                         if (i < cnt) {
-                            if (r[i] >= rows_here || (i > 0 && r[i] <= r[i - 1]))
-                                return fail(TL_ERR_FORMAT, "tile %u column %u: rows not ascending / out of range", t, y);
+                            if (r[i] >= rows_here) return fail(TL_ERR_FORMAT, "tile %u column %u: row out of range", t, y);
                         } else if (r[i] != kSentinel) {
                             return fail(TL_ERR_FORMAT, "tile %u column %u: padding byte is not the sentinel", t, y);
                         }
@@ -314,6 +384,8 @@ extern "C" int tl_layout_validate(const void* blob, int64_t blob_bytes)
         return fail(TL_ERR_FORMAT, "stream length does not match the chunk table");
     if (np != h.nnz_pos || nn != h.nnz_neg || run_max != h.max_run_dwords || chunk_max != h.max_chunk_dwords)
         return fail(TL_ERR_FORMAT, "header totals do not match the streams");
+    if (content_checksum(chunkstart, (size_t)T * NB + 1, stream, (size_t)expect_start) != h.checksum)
+        return fail(TL_ERR_FORMAT, "checksum of the chunk table and the stream does not match the header");
     return TL_OK;
 }
 
@@ -332,9 +404,9 @@ extern "C" int tl_layout_to_dense(const void* blob, int64_t blob_bytes, int32_t*
             const uint32_t* chunk = stream + chunkstart[(size_t)(y / kBlock) * h.n_tiles + t];
             const uint32_t d = chunk[y % kBlock], p = d & 0xff, n = (d >> 8) & 0xff;
             const uint8_t* run = reinterpret_cast<const uint8_t*>(chunk + (d >> 16));
-            for (uint32_t i = 0; i < p; ++i) w_out[((size_t)t * h.tile_rows + run[i]) * h.columns + y] = 1;
+            for (uint32_t i = 0; i < p; ++i) w_out[((size_t)t * h.tile_rows + run[i]) * h.columns + y] += 1;
             run += ((p + 3) / 4) * 4;
-            for (uint32_t i = 0; i < n; ++i) w_out[((size_t)t * h.tile_rows + run[i]) * h.columns + y] = -1;
+            for (uint32_t i = 0; i < n; ++i) w_out[((size_t)t * h.tile_rows + run[i]) * h.columns + y] -= 1;
         }
     return TL_OK;
 }

@@ -5,8 +5,9 @@ It stands where the reference patches a Hugging Face Llama with its ternary modu
 (ternaryLLM_GPU/TernaryLLM/TernaryLlama.py:69-75) and drives it with `generate`
 (ternaryLLM_GPU/benchmark_ternary_llama.py:81-105); the CPU twin of the same structure is
 ternaryLLM_CPU/src/LlamaModel.hpp:457-527.  Weights are random ternary matrices, drawn as the
-reference draws them; every product runs in libternary_spmm.so.  Normalisation, rotary embedding
-and attention are torch operators.
+reference draws them; every product runs in libternary_spmm.so.  A prefill pass uses torch operators
+for normalisation, rotary embedding and attention; a single-token step uses the library's kernels
+for them (rotary + cache update, attention over the cache, residual add + RMSNorm, SiLU gate).
 
 The decode step has static shapes (the cache has its full length, a mask hides what is not
 written yet, position and token live in device tensors), so it can be captured once in a HIP graph

@@ -144,6 +144,27 @@ class PackedWeight:
                                      inners, TILE_K, tile_rows, blob.ctypes.data, size.value))
         return cls(blob)
 
+    @classmethod
+    def from_mcsc(cls, merged_row, merged_off, columns, inners, TILE_K, uniformed=False, tile_rows=0):
+        """From the merged arrays convert_to_ter_tiled_mcsc returns (int16 or int32 indices): the blob
+        multiplies by exactly what the reference kernels' walk of those arrays adds up, rows named
+        several times included; `uniformed` leaves the same-sign part of every tile out, as the
+        reference's kernels do under that flag (ter_spmm_kernel.cuh:59,249)."""
+        merged_row = np.ascontiguousarray(merged_row)
+        if merged_row.dtype not in (np.int16, np.int32):
+            raise ValueError("merged_row must be int16 or int32")
+        merged_off = np.ascontiguousarray(merged_off, dtype=np.int32)
+        if TILE_K <= 0 or merged_off.size != columns * (-(-inners // TILE_K)) * 4:
+            raise ValueError("merged_off must hold columns * ceil(inners / TILE_K) * 4 entries")
+        size = ctypes.c_int64(0)
+        L = _lib.lib()
+        args = (merged_row.ctypes.data, merged_row.dtype.itemsize, merged_row.size, _lib.i32p(merged_off), columns, inners,
+                TILE_K, int(bool(uniformed)), tile_rows)
+        _lib.check(L.tl_layout_from_mcsc(*args, None, ctypes.byref(size)))
+        blob = np.zeros(size.value, np.uint8)
+        _lib.check(L.tl_layout_from_mcsc(*args, blob.ctypes.data, ctypes.byref(size)))
+        return cls(blob)
+
     def validate(self):
         _lib.check(_lib.lib().tl_layout_validate(self.blob.ctypes.data, self.blob.size))
 

@@ -10,15 +10,10 @@ TernaryLinear.py:19-20), without bias.  The model is any torch module tree; `tra
 import torch
 from torch import nn
 
+from .attention import collect_attn_linear_layers  # noqa: F401  (TernaryAttn.py:134-140; re-exported here)
 from .linear import TernaryLinear
 
 _ATTN_NAMES = ("q_proj", "k_proj", "v_proj", "o_proj")
-
-
-def collect_attn_linear_layers(model):
-    """(name, module) of the nn.Linear attention projections of `model` (TernaryAttn.py:134-140)."""
-    return [(name, m) for name, m in model.named_modules()
-            if isinstance(m, nn.Linear) and any(tag in name for tag in _ATTN_NAMES)]
 
 
 def collect_linear_layers(model, config):

@@ -6,6 +6,13 @@ import torch
 
 pytestmark = pytest.mark.gpu
 
+# Logit error of the fp16 pipeline against the fp32 restatement, relative to the largest logit.  An fp16
+# rounding is 2^-11 = 4.9e-4 relative; a logit sums thousands of rounded O(1) values with random signs, and a
+# layer rounds its activations about ten times.  The bounds are about twice what was measured on MI355X:
+# 1.3e-3 for TINY (2 layers x 256 wide), 1.7e-3 for FULL_WIDTH (2 layers x 4096 wide, 512 + 4 positions).
+TINY_TOL = 3e-3
+FULL_WIDTH_TOL = 4e-3
+
 
 def _reference_logits(model, tokens):
     """fp32 forward over the whole sequence with dense weights; returns logits [B, S, vocab]."""
@@ -60,14 +67,53 @@ def test_prefill_and_decode_match_fp32_reference(tiny, cuda):
     ref = _reference_logits(tiny, tokens)                       # [B, S + extra, V]
     scale = ref.abs().max().item()
     got = tiny.prefill(tokens[:, :S]).float()                   # 140 rows: the row-parallel kernel
-    assert (got - ref[:, S - 1]).abs().max().item() <= 2e-2 * scale
+    worst = (got - ref[:, S - 1]).abs().max().item() / scale
     st = tiny._decode_state(B)
     for j in range(extra):                                      # teacher-forced single-token steps: the small-M kernel
         st["token"].copy_(tokens[:, S + j])
         st["pos"].fill_(S + j)
         st["mask"].copy_((torch.arange(tiny.max_seq_len, device=cuda) <= S + j)[None, None, None])
         logits = tiny._decode_step(st["token"], st["pos"], st["mask"]).float()
-        assert (logits - ref[:, S + j]).abs().max().item() <= 2e-2 * scale
+        worst = max(worst, (logits - ref[:, S + j]).abs().max().item() / scale)
+    print(f"  tiny decoder: max |logit - ref| / max |ref| = {worst:.3e}", flush=True)
+    assert worst <= TINY_TOL
+
+
+@pytest.fixture(scope="module")
+def full_width(cuda):
+    """Two layers of BASELINE config 5's decoder at its real width: hidden 4096, FFN 11008, 32 heads x 128,
+    vocabulary 32000, 66 % sparsity."""
+    from ternaryllm_amd import TernaryConfig
+    from ternaryllm_amd.llama import TernaryLlamaDecoder
+    cfg = TernaryConfig(hidden_size=4096, intermediate_size=11008, num_hidden_layers=2, num_attention_heads=32,
+                        num_key_value_heads=32, vocab_size=32000, max_position_embeddings=528, sparsity=0.66)
+    return TernaryLlamaDecoder(cfg, seed=11, device=cuda, pack_threads=8)
+
+
+@pytest.mark.parametrize("batch", [1, 16])
+def test_full_width_prefill_512_and_decode_steps(full_width, cuda, batch):
+    """Config 5's shapes (prefill of 512 tokens, then single-token steps, batch 1 and 16) on the two-layer
+    full-width model against the fp32 restatement on dense weights: the prefill's logits and four
+    teacher-forced decode steps."""
+    model = full_width
+    g = torch.Generator().manual_seed(20 + batch)
+    S, extra = 512, 4
+    tokens = torch.randint(0, model.config.vocab_size, (batch, S + extra), generator=g).to(cuda)
+    print(f"case full-width decoder batch={batch}", flush=True)
+    ref = _reference_logits(model, tokens)[:, S - 1:].clone()          # [B, 1 + extra, V]
+    scale = ref.abs().max().item()
+    got = model.prefill(tokens[:, :S]).float()
+    worst = (got - ref[:, 0]).abs().max().item() / scale
+    st = model._decode_state(batch)
+    for j in range(extra):
+        st["token"].copy_(tokens[:, S + j])
+        st["pos"].fill_(S + j)
+        st["mask"].copy_((torch.arange(model.max_seq_len, device=cuda) <= S + j)[None, None, None])
+        logits = model._decode_step(st["token"], st["pos"], st["mask"]).float()
+        worst = max(worst, (logits - ref[:, 1 + j]).abs().max().item() / scale)
+    print(f"  max |logit - ref| / max |ref| = {worst:.3e}", flush=True)
+    model._state = None
+    assert worst <= FULL_WIDTH_TOL
 
 
 def test_native_decode_step_matches_torch_operators(tiny, cuda):

@@ -3,7 +3,7 @@ import numpy as np
 import pytest
 import torch
 
-from tests.util import FP16_TOL, FP32_TOL, activations, max_rel_err, ternary_weight
+from tests.util import FP16_TOL, FP32_TOL, activations, knobs, max_rel_err, ternary_weight
 
 pytestmark = pytest.mark.gpu
 
@@ -144,7 +144,7 @@ def test_small_m_activation_layouts(cuda, oracle, M, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
-def test_rows_kernel_with_and_without_shared_out_tiles(cuda, oracle, dtype, monkeypatch):
+def test_rows_kernel_with_and_without_shared_out_tiles(cuda, oracle, dtype):
     """The row-parallel kernel in both launch modes (one workgroup per output tile; K tiles shared out
     among one workgroup per compute unit, partial sums added by the fix-up launch), plain and fused."""
     from ternaryllm_amd import ops
@@ -162,15 +162,14 @@ def test_rows_kernel_with_and_without_shared_out_tiles(cuda, oracle, dtype, monk
         ref_fused = (torch.nn.functional.silu(g) * u).numpy()
         fused = {}
         for mode in ("0", "1"):
-            monkeypatch.setenv("TL_ROWS_SPLIT", mode)
             print(f"case M={M} K={K} N={N} dtype={dtype} split={mode}", flush=True)
-            y = ops.spmm(dg, x.to(cuda), out_dtype=torch.float32).cpu().numpy()
+            with knobs(TL_ROWS_SPLIT=mode):
+                y = ops.spmm(dg, x.to(cuda), out_dtype=torch.float32).cpu().numpy()
+                h = ops.mlp_gate_up(dg, du, xf.to(cuda), sg.to(cuda), sg.to(cuda), out_dtype=torch.float32).cpu().numpy()
             assert np.array_equal(y.astype(np.float64), ref), (M, K, N, mode)
-            h = ops.mlp_gate_up(dg, du, xf.to(cuda), sg.to(cuda), sg.to(cuda), out_dtype=torch.float32).cpu().numpy()
             scale = np.abs(ref_fused).max()
             assert np.abs(h - ref_fused).max() <= (FP16_TOL if dtype == torch.float16 else 1e-4) * scale, (M, K, N, mode)
             fused[mode] = h
-        monkeypatch.delenv("TL_ROWS_SPLIT")
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
@@ -198,7 +197,7 @@ def test_output_into_a_strided_buffer(cuda, oracle, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
-def test_small_m_kernels_in_every_mode(cuda, oracle, dtype, monkeypatch):
+def test_small_m_kernels_in_every_mode(cuda, oracle, dtype):
     """The direct-load kernels in the modes a default launch of a small shape does not reach: 8- and 16-row
     slots, one group of tiles or two alternating buffers, several lane groups per run or one, 512 or 1024
     threads for a single row; and the register-staged kernel on a single row."""
@@ -213,10 +212,7 @@ def test_small_m_kernels_in_every_mode(cuda, oracle, dtype, monkeypatch):
         ref = oracle.fast_product(x.double().numpy(), w)
         extra = [{"TL_SPMV_DIRECT": "0"}, {"TL_SPMV_WIDE": "0"}, {"TL_SPMV_WIDE": "1"}, {"TL_SPMV_WIDE": "1", "TL_TILE_GROUP": "2"}] if M == 1 else [{"TL_SMALL_MT": "8"}, {"TL_SMALL_MT": "16"}, {"TL_SMALL_MT": "16", "TL_TILE_GROUP": "2"}]
         for env in settings + extra:
-            for key, value in env.items():
-                monkeypatch.setenv(key, value)
             print(f"case M={M} dtype={dtype} env={env}", flush=True)
-            y = ops.spmm(dw, x.to(cuda), out_dtype=torch.float32).cpu().numpy()
-            for key in env:
-                monkeypatch.delenv(key)
+            with knobs(**env):
+                y = ops.spmm(dw, x.to(cuda), out_dtype=torch.float32).cpu().numpy()
             assert np.array_equal(y.astype(np.float64), ref), (M, env)

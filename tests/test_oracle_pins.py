@@ -105,6 +105,28 @@ def test_mcsc_hand_worked_tiles(oracle, case):
     assert tiles.tolist() == case["col_tile_idx"]
 
 
+@pytest.mark.parametrize("case", hand_cases(), ids=lambda c: c["name"][:40])
+def test_mcsc_product_hand_worked(oracle, case):
+    """orc_mcsc_product against the hand-worked sums of the fixture (ter_spmm_kernel.cuh:197-300): pairs,
+    the same-sign part with its sign, the row offset of a second tile, dropped and mis-signed rows of the
+    lossy tiles, a row named twice by padded arrays."""
+    x = np.array(case["x"], np.float64)[None, :]
+    assert sum(s * case["x"][r] for s, r in case["product_terms"]) == case["product"]
+    rows = np.array(case["merged_row_idx"], np.int32)
+    off = np.array(case["merged_off"], np.int32)
+    assert oracle.mcsc_product(x, rows, off, 1, case["tile_k"])[0, 0] == case["product"]
+    # under the kernels' UNIFORMED flag only the pair part counts: the terms whose position lies before off1
+    o = off.reshape(-1, 4)
+    n_pair_terms = int((o[:, 1] - o[:, 0]).sum())
+    pairs_only = sum(s * case["x"][r] for s, r in case["product_terms"][:n_pair_terms])
+    assert oracle.mcsc_product(x, rows, off, 1, case["tile_k"], uniformed=True)[0, 0] == pairs_only
+    # a second activation row must not leak into the first, nor the first into the second
+    x2 = np.vstack([x, 2.0 * x + 1.0])
+    both = oracle.mcsc_product(x2, rows, off, 1, case["tile_k"])
+    signs = sum(s for s, _ in case["product_terms"])
+    assert both[0, 0] == case["product"] and both[1, 0] == 2 * case["product"] + signs
+
+
 def test_mcsc_reduces_to_interleave_when_balanced(oracle):
     """Every tile with p == n and p even: the alignment rule is a no-op and the merged stream is the plain
     interleave of the tiled-CSC streams (the clean format of the reference's TernaryCSC.py:97-156)."""

@@ -98,6 +98,81 @@ def test_mcsc_decodes_to_the_matrix_it_encodes(oracle):
         packing.tiled_mcsc_to_dense(rows.astype(np.int16), off[:-4], 24, 256, 64)
 
 
+def _hand_cases():
+    import json
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "mcsc_hand_cases.json")) as f:
+        return json.load(f)["cases"]
+
+
+@pytest.mark.parametrize("case", _hand_cases(), ids=lambda c: c["name"][:40])
+def test_blob_from_merged_arrays_encodes_the_hand_worked_terms(case):
+    """tl_layout_from_mcsc on the fixture's arrays: the integer matrix the blob decodes to is the sum of the
+    hand-worked terms (a row named twice counts twice), also with the same-sign part left out."""
+    rows = np.array(case["merged_row_idx"], np.int16)
+    off = np.array(case["merged_off"], np.int32)
+    K, tk = case["inners"], case["tile_k"]
+    o = off.reshape(-1, 4)
+    n_pair_terms = int((o[:, 1] - o[:, 0]).sum())
+    for uniformed, terms in ((False, case["product_terms"]), (True, case["product_terms"][:n_pair_terms])):
+        want = np.zeros((K, 1), np.int32)
+        for s, r in terms:
+            want[r, 0] += s
+        pw = packing.PackedWeight.from_mcsc(rows, off, 1, K, tk, uniformed)
+        pw.validate()
+        assert np.array_equal(pw.to_dense(), want)
+    if np.abs(want).max() <= 1 and not case["padding"]:
+        assert np.array_equal(packing.tiled_mcsc_to_dense(rows, off, 1, K, tk), packing.PackedWeight.from_mcsc(rows, off, 1, K, tk).to_dense())
+
+
+@pytest.mark.parametrize("padding", [False, True])
+def test_blob_from_merged_arrays_matches_the_oracle_walk(oracle, padding):
+    rng = np.random.default_rng(4)
+    K, N, tk = 512, 40, 256
+    w = ternary_weight(K, N, 0.7, 15)
+    cp, cn = packing.count_nnz(w)
+    rows, off, _ = packing.convert_to_ter_tiled_mcsc(w, N, K, cp, cn, tk, padding, 4)
+    x = rng.integers(-8, 9, (3, K)).astype(np.float64)
+    for uniformed in (False, True):
+        pw = packing.PackedWeight.from_mcsc(rows.astype(np.int16), off, N, K, tk, uniformed)
+        pw.validate()
+        assert np.array_equal(x @ pw.to_dense().astype(np.float64), oracle.mcsc_product(x, rows, off, N, tk, uniformed))
+    with pytest.raises(ValueError):
+        bad = rows.copy()
+        bad[off[0]] = tk  # a row index outside its tile
+        packing.PackedWeight.from_mcsc(bad, off, N, K, tk)
+
+
+@pytest.mark.parametrize("K,N,s,seed", [(4096, 11008, 0.8, 1237), (2048, 2048, 0.9, 3), (256, 16, 0.99, 1), (4096, 48, 0.0, 2)])
+def test_index_prefetch_stays_inside_the_blob(K, N, s, seed):
+    """The row kernel requests 192 index dwords from the start of every wave's piece of a chunk (a wave owns 4 or
+    8 neighbouring columns) and, for longer pieces, whole 64-dword groups up to 63 dwords past the piece's end:
+    the furthest byte either touches must lie inside the blob as trimmed to header.total_bytes."""
+    if K * N > 1 << 24:
+        rng = np.random.default_rng(seed)   # the torch generator is slow at this size
+        r = rng.random((K, N), dtype=np.float32)
+        w = np.zeros((K, N), np.int32)
+        w[r >= s] = -1
+        w[r >= (s + 1) / 2] = 1
+    else:
+        w = ternary_weight(K, N, s, seed)
+    pw = packing.PackedWeight.from_dense(w)
+    h = pw.header
+    assert pw.blob.size == h.total_bytes
+    stream = pw.blob[h.off_stream:].view(np.uint32)
+    cs = pw.blob[h.off_chunkstart:h.off_chunkstart + (h.n_tiles * h.n_blocks + 1) * 4].view(np.uint32).astype(np.int64)
+    room = (h.total_bytes - h.off_stream) // 4   # dwords from the stream's start to the blob's end
+    for C in (4, 8):
+        subs = np.arange(0, 16, C)
+        d_first = stream[cs[:-1, None] + subs[None, :]].astype(np.int64)             # descriptor of a wave's first column
+        d_last = stream[cs[:-1, None] + subs[None, :] + C - 1].astype(np.int64)      # ... and of its last
+        base = cs[:-1, None] + (d_first >> 16)
+        end = cs[:-1, None] + (d_last >> 16) + ((d_last & 0xff) + 3) // 4 + (((d_last >> 8) & 0xff) + 3) // 4
+        total = end - base
+        assert (base + 192).max() <= room
+        groups = -(-total // 64)
+        assert (base + np.maximum(groups, 3) * 64).max() <= room
+
+
 def test_error_behaviour():
     w = ternary_weight(64, 8, 0.5, 1)
     cp, cn = packing.count_nnz(w)

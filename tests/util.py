@@ -1,6 +1,29 @@
 """Shared helpers of the tests: seeded inputs and the error measure."""
+import contextlib
+import os
+
 import numpy as np
 import torch
+
+
+@contextlib.contextmanager
+def knobs(**env):
+    """Sets the library's tuning knobs (TL_* environment variables) for the block and has the library read
+    them again (it reads the environment once per process otherwise); restores both on the way out."""
+    from ternaryllm_amd import _lib
+    old = {k: os.environ.get(k) for k in env}
+    try:
+        for k, v in env.items():
+            os.environ[k] = str(v)
+        _lib.lib().tl_reload_options()
+        yield
+    finally:
+        for k, v in old.items():
+            if v is None:
+                os.environ.pop(k, None)
+            else:
+                os.environ[k] = v
+        _lib.lib().tl_reload_options()
 
 
 def ternary_weight(K, N, sparsity, seed):
