@@ -223,6 +223,20 @@ int tl_spmm(const tl_layout_header* header, const void* blob_dev,
             const void* scale, int scale_dtype,
             void* workspace, int64_t workspace_bytes, void* stream);
 
+/* tl_spmm for callers that cannot allocate or pass a workspace: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same
+ * arguments and result as tl_spmm, minus the workspace: what tl_spmm stages there (the K-major image of the
+ * activations) goes into a 32 MiB array inside the library's device code, one copy per GPU, held until
+ * the process ends.  The call allocates and frees nothing.  TL_ERR_SIZE when the image would not fit
+ * (e.g. 1024 x 11008 fp16 fits, 1024 x 11008 fp32 does not).  The kernels write every byte of the array
+ * before they read it, so nothing is cleared between calls; all calls on one GPU share the array, so
+ * calls that may overlap on one GPU (different streams) race -- keep them on one stream or use tl_spmm.
+ * The first call on a device looks the array's address up; make it outside graph capture. */
+int tl_spmm_noalloc(const tl_layout_header* header, const void* blob_dev,
+                    const void* X, int x_dtype, int x_layout, int64_t ldx, int64_t M,
+                    void* Y, int y_dtype, int64_t ldy,
+                    const void* scale, int scale_dtype, void* stream);
+
 /* H[M][N] = act(X*Wg * sg, X*Wu * su): the gate and up projections of the
  * reference's LlamaTernaryMLP (TernaryLLM/TernaryMLP.py:33-35) in one pass over X
  * with the SiLU-gate product fused into the epilogue (the reference runs two

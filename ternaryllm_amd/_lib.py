@@ -66,6 +66,7 @@ SIGNATURES = {
     "tl_layout_to_dense": (_INT, [_VP, _I64, _I32P]),
     "tl_spmm_workspace": (_INT, [_HDRP, _I64, _INT, _INT, _I64P]),
     "tl_spmm": (_INT, [_HDRP, _VP, _VP, _INT, _INT, _I64, _I64, _VP, _INT, _I64, _VP, _INT, _VP, _I64, _VP]),
+    "tl_spmm_noalloc": (_INT, [_HDRP, _VP, _VP, _INT, _INT, _I64, _I64, _VP, _INT, _I64, _VP, _INT, _VP]),
     "tl_mlp_gate_up": (_INT, [_HDRP, _VP, _HDRP, _VP, _VP, _INT, _INT, _I64, _I64, _VP, _INT, _I64, _VP, _VP, _INT, _INT,
                               _VP, _I64, _VP]),
     "tl_spmm_time": (_INT, [_HDRP, _VP, _VP, _INT, _INT, _I64, _I64, _VP, _INT, _I64, _VP, _INT, _VP, _I64, _VP, _INT,

@@ -1756,6 +1756,52 @@ extern "C" int tl_spmm(const tl_layout_header* header, const void* blob_dev,
     return finish_launch();
 }
 
+// Scratch of tl_spmm_noalloc: device memory that belongs to the library's code object, one copy per GPU,
+// there from the moment the library is loaded on a device until the process ends.
+constexpr int64_t kStaticScratchBytes = 32ll << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+// Device address of `scratch` on the current device.  In host code the array's name is only a handle
+// for the runtime; the address comes from hipGetSymbolAddress, asked once per device with that device
+// current, and differs from GPU to GPU.
+int static_scratch(void** out)
+{
+    static std::atomic<void*> address[64];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(TL_ERR_LAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= 64) return fail(TL_ERR_UNSUPPORTED, "device ordinal %d: the static scratch serves ordinals 0 to 63", dev);
+    void* p = address[dev].load(std::memory_order_acquire);
+    if (!p) {
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) return fail(TL_ERR_LAUNCH, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+        address[dev].store(p, std::memory_order_release);
+    }
+    *out = p;
+    return TL_OK;
+}
+}  // namespace
+
+extern "C" int tl_spmm_noalloc(const tl_layout_header* header, const void* blob_dev,
+                               const void* X, int x_dtype, int x_layout, int64_t ldx, int64_t M,
+                               void* Y, int y_dtype, int64_t ldy,
+                               const void* scale, int scale_dtype, void* stream)
+{
+    if (int rc = check_header(header)) return rc;
+    if (int rc = check_dtype(x_dtype, "x")) return rc;
+    if (M <= 0) return fail(TL_ERR_SHAPE, "M=%lld must be positive", (long long)M);
+    // what the kernels stage in the scratch: the K-major image of the activations (none for 4 rows and fewer).
+    // Room for partial sums is not offered, so the row kernel gives every output tile a workgroup of its own.
+    const int64_t need = M <= kSmallMaxM ? small_kmajor_bytes(header, M, x_dtype) : rows_relayout_bytes(header->inners, M, x_dtype);
+    if (need > kStaticScratchBytes)
+        return fail(TL_ERR_SIZE, "M=%lld rows of K=%u need %lld bytes of scratch; tl_spmm_noalloc has %lld (use tl_spmm with a workspace)",
+                    (long long)M, header->inners, (long long)need, (long long)kStaticScratchBytes);
+    void* ws = nullptr;
+    if (int rc = static_scratch(&ws)) return rc;
+    return tl_spmm(header, blob_dev, X, x_dtype, x_layout, ldx, M, Y, y_dtype, ldy, scale, scale_dtype, ws, need, stream);
+}
+
 extern "C" int tl_mlp_gate_up(const tl_layout_header* gate_header, const void* gate_blob_dev,
                               const tl_layout_header* up_header, const void* up_blob_dev,
                               const void* X, int x_dtype, int x_layout, int64_t ldx, int64_t M,
