@@ -128,6 +128,8 @@ int tl_tiled_mcsc_to_dense(const void* merged_row, int index_width, int64_t n_in
 /*     then added that many times) and may sit in both runs (it cancels):   */
 /*     a blob built from dense ternary weights holds every row once, one    */
 /*     built from the reference's merged arrays holds what they encode.     */
+/*     The builder orders the rows of a run so that the single-row kernel's */
+/*     LDS reads spread over the banks.                                     */
 /*   - the stream is block-major: all tiles of block 0, then block 1, ...;  */
 /*     chunkstart[block * T + tile] is the dword where a chunk begins       */
 /*     (one extra entry marks the end).                                     */
@@ -155,8 +157,9 @@ typedef struct tl_layout_header {
     uint64_t total_bytes;    /* bytes of the blob that are in use, multiple of 256                        */
     uint32_t max_run_dwords; /* largest (+1 run dwords + -1 run dwords) of any (column, tile)             */
     uint32_t mean_run_dwords_x16; /* mean of the same, times 16, rounded up                               */
-    uint64_t checksum;       /* FNV-1a (64-bit, one step per dword) over the chunk table and the stream   */
-    uint32_t reserved[40];
+    uint64_t checksum;       /* FNV-1a (64-bit, one step per dword) over chunk table, run order and stream */
+    uint64_t off_runorder;   /* byte offset of uint16 runorder[NB][T * 16], or 0 when T * 16 >= 65536       */
+    uint32_t reserved[38];
 } tl_layout_header;
 
 /* Bytes of the blob that tl_layout_build will write for these tiled-CSC arrays

@@ -25,5 +25,9 @@ inline uint32_t make_desc(uint32_t n_pos, uint32_t n_neg, uint32_t dword_off)
 constexpr int kSentinel = 255;       // index byte that addresses the always-zero slot of a tile
 constexpr int kTileSlots = 256;      // slots a staged tile occupies (tile_rows real rows + zeros)
 constexpr int kMaxTileRows = 255;
+// The single-row kernel lays the LDS images of consecutive tiles kTileSlots slots + this many bytes apart, so that
+// equal slots of neighbouring tiles (the zero slot among them) fall on different LDS banks; the packer orders
+// the rows of a run with that placement in mind.
+constexpr int kSpmvImageSkew = 16;
 
 }  // namespace tl

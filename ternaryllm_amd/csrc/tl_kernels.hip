@@ -624,7 +624,8 @@ __global__ __launch_bounds__(NT) void tl_spmv_direct(KernelArgs a)
     using XT = typename std::conditional<XF16, __half, float>::type;
     constexpr int ES = (int)sizeof(XT);
     constexpr int VE = 16 / ES;                  // values per 16-byte piece
-    constexpr int PPT = kTileSlots / VE;         // pieces per tile image
+    constexpr int PITCH = kTileSlots + kSpmvImageSkew / ES;  // slots from one tile image to the next: each starts 4 banks further round
+    constexpr int PPT = PITCH / VE;              // pieces per tile image
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int TG = a.tiles_per_group;
@@ -645,7 +646,7 @@ __global__ __launch_bounds__(NT) void tl_spmv_direct(KernelArgs a)
         for (int first = wave * 64; first < vectors; first += NT)
             if (first + lane < vectors)
                 __builtin_amdgcn_global_load_lds((global_ptr)(a.w0.stream + lo + (size_t)(first + lane) * 4), (lds_ptr)(buf + (size_t)first * 16), 16, 0, 0);
-        const int pieces = nt * PPT;  // PPT is 32 or 64: a wave's 64 pieces never straddle the image's end by less than a tile
+        const int pieces = nt * PPT;  // images lie back to back, PPT pieces each (the last one or two of an image only ever hold zeros)
         for (int first = wave * 64; first < pieces; first += NT) {
             const int p = first + lane, tile = p / PPT, k = (t + tile) * a.tile_rows + (p % PPT) * VE;
             if (p < pieces) {
@@ -693,7 +694,7 @@ __global__ __launch_bounds__(NT) void tl_spmv_direct(KernelArgs a)
             for (int u = 0; u < TU; ++u) {
                 const int pd = run_pos_dwords(d[u]), tot = pd + run_neg_dwords(d[u]);
                 if (u > 0 && __builtin_amdgcn_ballot_w64(tot > 0) == 0) continue;  // no lane of the wave has this tile
-                const XT* xt = xs + (size_t)min(tl0 + u * TP, nt - 1) * kTileSlots;
+                const XT* xt = xs + (size_t)min(tl0 + u * TP, nt - 1) * PITCH;
                 gather_add<1, XT>(acc, xt, w[u], lw < pd ? 1.0f : -1.0f);
                 for (int i = lw + LW; i < tot; i += LW)  // runs longer than the lane group
                     gather_add<1, XT>(acc, xt, run[u][i], i < pd ? 1.0f : -1.0f);
@@ -1442,7 +1443,7 @@ template <bool XF16, int NT>
 int launch_spmv_direct_nt(KernelArgs a, const tl_layout_header* h, hipStream_t st)
 {
     constexpr int es = XF16 ? 2 : 4;
-    const int tile_bytes = kTileSlots * es;
+    const int tile_bytes = kTileSlots * es + kSpmvImageSkew;
     const int chunk_bytes = (int)h->max_chunk_dwords * 4;
     const int share = std::max(1, std::min(knob(TL_SPMV_SHARE, 4), (int)ceil_div(a.NB, compute_units())));
     const int budget = 160 * 1024 / share - 1024;

@@ -94,6 +94,115 @@ int count_device_tiles(const int32_t* row, const int32_t* off_tiled, int columns
     return TL_OK;
 }
 
+// Order of the rows inside runs.  The sum does not depend on it; the single-row kernel's speed does: a lane
+// reads one activation per index from the LDS image of its tile, 64 lanes at a time, and reads that fall on
+// one LDS bank (of 32, four bytes wide) but on different words are served one after the other.  That kernel
+// works on neighbouring tiles of a column side by side, four lanes to a run (lane l on dwords l, l + 4, ... of
+// the +1 run followed by the -1 run); all lanes read byte b of their k-th dword together.  So the rows of
+// a group of 8 tiles (32 lanes) are dealt out read by read: each lane takes from what is left of its run the
+// row whose bank the read has used least so far (the padding bytes, which read the tile's zero slot, are
+// counted first); then rows are swapped between the reads of a run while that lowers the number of lanes
+// that share a bank.  Blobs whose runs are longer on average get more lanes per run from the kernel; the
+// order is then no better than any other, and no worse.
+struct RunRef {
+    uint8_t* bytes;  // start of the +1 run (the -1 run follows its padded end)
+    int n_pos, n_neg;
+    int tile;
+};
+
+constexpr int kLanesPerRun = 4;
+constexpr int kSpreadSweeps = 1;
+
+// LDS bank of a row's activation in the single-row kernel: fp16 values, two to a bank word; the image of
+// tile t starts kSpmvImageSkew bytes further round the banks than that of tile t - 1 (tl_common.h).
+inline int bank_of(uint8_t row, int tile) { return ((row >> 1) + tile * (kSpmvImageSkew / 4)) & 31; }
+
+void spread_over_banks(const RunRef* runs, int n_runs, int sweeps)
+{
+    // read q = pass * 4 + byte; run r, lane l holds dword pass * 4 + l of the combined run
+    int longest = 0;
+    for (int r = 0; r < n_runs; ++r) longest = std::max(longest, (runs[r].n_pos + 3) / 4 + (runs[r].n_neg + 3) / 4);
+    if (longest == 0) return;
+    const int passes = (longest + kLanesPerRun - 1) / kLanesPerRun, reads = passes * 4;
+    std::vector<int> load((size_t)reads * 32, 0);
+    std::vector<uint8_t> pool[2];
+    auto position = [&](const RunRef& run, int q, int l, bool* neg, int* e) {
+        const int pd = (run.n_pos + 3) / 4;
+        const int i = (q >> 2) * kLanesPerRun + l;
+        *neg = i >= pd;
+        *e = 4 * (*neg ? i - pd : i) + (q & 3);
+        return *e < (*neg ? run.n_neg : run.n_pos);
+    };
+    for (int r = 0; r < n_runs; ++r) {
+        const RunRef& run = runs[r];
+        const int pd = (run.n_pos + 3) / 4;
+        pool[0].assign(run.bytes, run.bytes + run.n_pos);
+        pool[1].assign(run.bytes + 4 * pd, run.bytes + 4 * pd + run.n_neg);
+        // the padding bytes of the two last dwords read the tile's zero slot: loads that are there whatever the order
+        for (int sign = 0; sign < 2; ++sign) {
+            const int n = sign ? run.n_neg : run.n_pos;
+            for (int e = n; e < (n + 3) / 4 * 4; ++e)
+                ++load[(size_t)((((sign ? pd : 0) + e / 4) / kLanesPerRun) * 4 + (e & 3)) * 32 + bank_of(kSentinel, run.tile)];
+        }
+        for (int q = 0; q < reads; ++q)
+            for (int l = 0; l < kLanesPerRun; ++l) {
+                bool neg;
+                int e;
+                if (!position(run, q, l, &neg, &e)) continue;
+                std::vector<uint8_t>& left = pool[neg ? 1 : 0];
+                const int* ld = &load[(size_t)q * 32];
+                size_t best = 0;
+                for (size_t c = 1; c < left.size(); ++c) {
+                    const int lb = ld[bank_of(left[best], run.tile)], lc = ld[bank_of(left[c], run.tile)];
+                    if (lc < lb || (lc == lb && left[c] < left[best])) best = c;
+                }
+                const uint8_t row = left[best];
+                left[best] = left.back();
+                left.pop_back();
+                ++load[(size_t)q * 32 + bank_of(row, run.tile)];
+                run.bytes[(neg ? 4 * pd : 0) + e] = row;
+            }
+    }
+    // swaps inside a run, between two of its reads, that lower the sum of squared bank loads
+    for (int sweep = 0; sweep < sweeps; ++sweep) {
+        bool any = false;
+        for (int r = 0; r < n_runs; ++r) {
+            const RunRef& run = runs[r];
+            const int pd = (run.n_pos + 3) / 4;
+            for (int sign = 0; sign < 2; ++sign) {
+                uint8_t* rows = run.bytes + (sign ? 4 * pd : 0);
+                const int n = sign ? run.n_neg : run.n_pos;
+                const int first_dword = sign ? pd : 0;
+                auto read_of = [&](int e) { return ((first_dword + e / 4) / kLanesPerRun) * 4 + (e & 3); };
+                for (int e1 = 0; e1 < n; ++e1) {
+                    const int q1 = read_of(e1), b1 = bank_of(rows[e1], run.tile);
+                    if (load[(size_t)q1 * 32 + b1] < 2) continue;  // alone on its bank: nothing to gain
+                    int best = -1, best_gain = 0;
+                    for (int e2 = 0; e2 < n; ++e2) {
+                        const int q2 = read_of(e2);
+                        if (q2 == q1) continue;
+                        const int b2 = bank_of(rows[e2], run.tile);
+                        if (b1 == b2) continue;
+                        // before: l(q1,b1), l(q1,b2), l(q2,b1), l(q2,b2); moving b1 to q2 and b2 to q1
+                        const int a = load[(size_t)q1 * 32 + b1], b = load[(size_t)q1 * 32 + b2];
+                        const int c = load[(size_t)q2 * 32 + b1], d = load[(size_t)q2 * 32 + b2];
+                        const int gain = 2 * (a - 1 - b) + 2 * (d - 1 - c);  // decrease of the sum of squares
+                        if (gain > best_gain) { best_gain = gain; best = e2; }
+                    }
+                    if (best >= 0) {
+                        const int q2 = read_of(best), b2 = bank_of(rows[best], run.tile);
+                        --load[(size_t)q1 * 32 + b1]; ++load[(size_t)q1 * 32 + b2];
+                        --load[(size_t)q2 * 32 + b2]; ++load[(size_t)q2 * 32 + b1];
+                        std::swap(rows[e1], rows[best]);
+                        any = true;
+                    }
+                }
+            }
+        }
+        if (!any) break;
+    }
+}
+
 // FNV-1a, 64-bit, one step per dword, over the chunk table (with its end entry) and the stream.
 uint64_t content_checksum(const uint32_t* chunkstart, size_t n_table, const uint32_t* stream, size_t n_stream)
 {
@@ -196,6 +305,7 @@ extern "C" int tl_layout_build(const int32_t* neg_row, const int32_t* neg_off_ti
         }
     std::vector<uint64_t> cursor((size_t)T * 2);
     uint8_t* bytes = reinterpret_cast<uint8_t*>(stream);
+    std::vector<RunRef> runs(8);
     for (int y = 0; y < columns; ++y) {
         const int nb = y / kBlock, j = y % kBlock;
         for (int t = 0; t < T; ++t) {
@@ -213,6 +323,17 @@ extern "C" int tl_layout_build(const int32_t* neg_row, const int32_t* neg_off_ti
                     const int k = t * tile_k + row[i];
                     bytes[cursor[2 * (k / g.tile_rows) + sign]++] = (uint8_t)(k % g.tile_rows);
                 }
+        }
+        // the column is complete: order the rows inside every group of 8 neighbouring tiles (the 32 lanes that
+        // the single-row kernel puts on them read together)
+        for (int t0 = 0; t0 < T; t0 += 8) {
+            const int gsz = std::min(8, T - t0);
+            for (int i = 0; i < gsz; ++i) {
+                const uint64_t c0 = chunkstart[(size_t)nb * T + t0 + i];
+                const uint32_t d = stream[c0 + j];
+                runs[i] = RunRef{bytes + (c0 + (d >> 16)) * 4, (int)(d & 0xff), (int)((d >> 8) & 0xff), t0 + i};
+            }
+            spread_over_banks(runs.data(), gsz, kSpreadSweeps);
         }
     }
 
