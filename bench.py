@@ -51,6 +51,17 @@ def weight_and_packed(K, N, sparsity, seed, device):
     return w, pw, ops.DeviceWeight(pw, device)
 
 
+def kernel_source_hash():
+    """sha256 over the sources the measured kernels are built from: a traffic figure recorded for other
+    sources is not reported."""
+    import hashlib
+    h = hashlib.sha256()
+    for name in ("tl_kernels.hip", "tl_layout.cpp", "tl_common.h"):
+        with open(os.path.join(ROOT, "ternaryllm_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
 def best_k_mean(samples, k):
     s = sorted(samples)[:k]
     return sum(s) / len(s)
@@ -72,11 +83,40 @@ def time_spmm(dw, x, scale, steps, warmup, x_layout=0):
     return wall_ms, ev_ms
 
 
+def graph_us_per_node(fn, nodes, replays):
+    """Median, 10th percentile and best-10 mean of the time per node of a HIP graph of fn(0) ... fn(nodes - 1),
+    replayed `replays` times (launch gaps are then the hardware's, not the interpreter's)."""
+    import torch
+    for i in range(2):
+        fn(i)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for i in range(nodes):
+                fn(i)
+    torch.cuda.synchronize()
+    for _ in range(2):
+        graph.replay()
+    torch.cuda.synchronize()
+    samples = []
+    for _ in range(replays):
+        t0 = time.perf_counter()
+        graph.replay()
+        torch.cuda.synchronize()
+        samples.append((time.perf_counter() - t0) / nodes)
+    samples.sort()
+    return samples[len(samples) // 2], samples[len(samples) // 10], best_k_mean(samples, 10)
+
+
 def cold_decode_leg(dev, K=4096, N=4096, sparsity=0.66, copies=48, calls=1000, M=1):
-    """Config 2 as the decoder meets it: 1000 SpMV calls with a fresh x each, over `copies` distinct
-    copies of the weight (about 300 MB, more than the last-level cache holds), issued as HIP-graph
-    replays so that launch gaps are the hardware's, not the interpreter's.  With M > 1: the same for a
-    batch of M rows (row-major, so the K-major image is made by the library's pre-pass)."""
+    """Config 2 as the decoder meets it: `calls` SpMV calls, each with an x of its own, over `copies` distinct
+    copies of the weight (about 300 MB, more than the last-level cache holds), captured as one HIP graph
+    and replayed.  With M > 1: the same for a batch of M rows (row-major, so the K-major image is made by
+    the library's pre-pass).  Beside it, what a plain device copy of as many bytes as one weight copy takes
+    under the same replay: the box's own floor for a call that must stream that much memory."""
     import torch
     from ternaryllm_amd import ops
     w, pw, dw = weight_and_packed(K, N, sparsity, 1244, dev)
@@ -86,40 +126,49 @@ def cold_decode_leg(dev, K=4096, N=4096, sparsity=0.66, copies=48, calls=1000, M
         c.header, c.blob = dw.header, dw.blob.clone()
         ws.append(c)
     g = torch.Generator().manual_seed(1245)
-    xs = torch.randn((copies, M, K), generator=g).to(torch.float16).to(dev)  # a fresh x per call of the graph
-    ys = torch.empty((copies, M, N), dtype=torch.float16, device=dev)
-    for i in range(2):
-        ops.spmm(ws[i], xs[i], out=ys[i])
-    torch.cuda.synchronize()
-    side = torch.cuda.Stream()
-    side.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(side):
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            for i in range(copies):
-                ops.spmm(ws[i], xs[i], out=ys[i])
-    torch.cuda.synchronize()
-    replays = max(1, calls // copies)
-    for _ in range(2):
-        graph.replay()
-    torch.cuda.synchronize()
-    samples = []
-    for _ in range(replays):
-        t0 = time.perf_counter()
-        graph.replay()
-        torch.cuda.synchronize()
-        samples.append((time.perf_counter() - t0) / copies)
-    # parity of the last replay's first call
-    ref = xs[0].double().cpu().numpy() @ w.double().numpy()
-    err = float(abs(ys[0].double().cpu().numpy() - ref).max() / max(1e-9, abs(ref).max()))
-    samples.sort()
-    med = samples[len(samples) // 2]
+    xs = torch.randn((calls, M, K), generator=g).to(torch.float16).to(dev)  # a fresh x for every call of the graph
+    ys = torch.empty((calls, M, N), dtype=torch.float16, device=dev)
+    med, p10, best = graph_us_per_node(lambda i: ops.spmm(ws[i % copies], xs[i], out=ys[i]), calls, 10)
+    # parity of the last replay: first and last call
+    err = 0.0
+    for i in (0, calls - 1):
+        ref = xs[i].double().cpu().numpy() @ w.double().numpy()
+        err = max(err, float(abs(ys[i].double().cpu().numpy() - ref).max() / max(1e-9, abs(ref).max())))
+    dst = torch.empty_like(dw.blob)
+    copy_med, _, _ = graph_us_per_node(lambda i: dst.copy_(ws[i % copies].blob), min(calls, 4 * copies), 10)
     B = pw.algorithmic_bytes(M, 2, 2)
-    return {"M": M, "K": K, "N": N, "sparsity": sparsity, "weight_copies": copies, "calls": replays * copies,
-            "us_per_call_median": round(med * 1e6, 3), "us_per_call_p10": round(samples[len(samples) // 10] * 1e6, 3),
-            "us_per_call_best10_mean": round(best_k_mean(samples, 10) * 1e6, 3),
+    return {"M": M, "K": K, "N": N, "sparsity": sparsity, "weight_copies": copies, "calls_per_replay": calls, "distinct_x": calls,
+            "us_per_call_median": round(med * 1e6, 3), "us_per_call_p10": round(p10 * 1e6, 3),
+            "us_per_call_best10_mean": round(best * 1e6, 3),
             "GB_per_s": round(B / med / 1e9, 1), "pct_hbm_peak": round(100 * B / med / 1e9 / HBM_PEAK_GBS, 2),
-            "tokens_per_s": round(M / med, 1), "max_err_over_max": err}
+            "tokens_per_s": round(M / med, 1), "max_err_over_max": err,
+            "plain_copy_of_one_weight_us": round(copy_med * 1e6, 3), "weight_bytes": int(dw.blob.numel()),
+            "time_over_plain_copy": round(med / copy_med, 2)}
+
+
+def balanced_leg(dev, steps, warmup):
+    """Block-balanced weights (the reference's `uniform=True` generator, TernaryLinear.py:39-77: every block of a
+    column holds the same number of +1 and of -1) against i.i.d. weights with the same number of non-zeros, on
+    config 2's and config 3's shapes: the reference's kernels have a path of their own for balanced weights
+    (no same-sign remainder, ter_spmm_kernel.cuh:59,249); here both run through the same kernels."""
+    import torch
+    from ternaryllm_amd import ops
+    from ternaryllm_amd.linear import random_ternary_weights
+    from ternaryllm_amd.packing import PackedWeight
+    out = []
+    for name, M, K, N, s in (("config 2 (M=1)", 1, 4096, 4096, 0.66), ("config 3 gate (M=1024)", 1024, 4096, 11008, 0.8)):
+        g = torch.Generator().manual_seed(1250)
+        x = torch.randn((M, K), generator=g).to(torch.float16).to(dev)
+        row = {"shape": name}
+        for kind, uniform in (("iid", False), ("balanced_blocks_of_256", True)):
+            w = random_ternary_weights((K, N), s, uniform, 256, generator=g)
+            pw = PackedWeight.from_dense(w)
+            dw = ops.DeviceWeight(pw, dev)
+            _, ev_ms = time_spmm(dw, x, None, max(steps, 50), warmup)
+            row[kind] = {"nnz": int(pw.nnz), "stream_bytes": int(pw.header.stream_bytes), "kernel_ms": round(ev_ms, 5)}
+        row["balanced_over_iid"] = round(row["balanced_blocks_of_256"]["kernel_ms"] / row["iid"]["kernel_ms"], 4)
+        out.append(row)
+    return out
 
 
 def decoder_leg(dev, prompt=512, new_tokens=128):
@@ -192,11 +241,13 @@ def main():
     x = torch.randn((M, K), generator=g).to(torch.float16)
     scale = (0.5 + torch.rand(N, generator=g)).to(torch.float16)
     xd, sd = x.to(dev), scale.to(dev)
-    # the kernel's native activation layout ([K][M], M contiguous): the timed launch is then the SpMM kernel alone
+    # row-major [M][K] activations, what TernaryLinear.forward passes: one call is the re-layout pre-pass, the row
+    # kernel and its fix-up launch
+    wall_ms, ev_ms = time_spmm(dw, xd, sd, args.steps, args.warmup)
+    # beside it: activations already in the kernel's own layout ([K][M], M contiguous), no pre-pass
     xk = xd.t().contiguous()
-    wall_ms, ev_ms = time_spmm(dw, xk, sd, args.steps, args.warmup, x_layout=_lib.TL_X_K_MAJOR)
-    wall_rm_ms, ev_rm_ms = time_spmm(dw, xd, sd, args.steps, args.warmup)  # row-major input: adds the re-layout pre-pass
-    y = ops.spmm(dw, xk, sd, x_layout=_lib.TL_X_K_MAJOR)
+    wall_km_ms, ev_km_ms = time_spmm(dw, xk, sd, args.steps, args.warmup, x_layout=_lib.TL_X_K_MAJOR)
+    y = ops.spmm(dw, xd, sd)
     ref = (x.double().numpy() @ w.double().numpy()) * scale.double().numpy()[None, :]
     err = np.abs(y.float().cpu().numpy() - ref)
     floor = np.linalg.norm(x.double().numpy(), axis=1, keepdims=True) * np.sqrt(1 - sparsity)
@@ -207,11 +258,17 @@ def main():
     B = pw.algorithmic_bytes(M, 2, 2, 2)
     nnz = pw.nnz
     gbs = B / (wall_ms * 1e-3) / 1e9
-    traffic = None
+    # HBM bytes per call from rocprofv3's FETCH_SIZE / WRITE_SIZE (profiles/): reported only while the kernels are
+    # still the ones it was recorded for
+    traffic, traffic_note = None, "no traffic record"
     tpath = os.path.join(ROOT, "profiles", "spmm_rows_c3_gate_traffic.json")
     if os.path.exists(tpath):
         with open(tpath) as f:
-            traffic = json.load(f).get("hbm_bytes_per_launch")
+            rec = json.load(f)
+        if rec.get("kernel_source_sha16") == kernel_source_hash():
+            traffic, traffic_note = rec.get("hbm_bytes_per_launch"), "rocprofv3 FETCH_SIZE + WRITE_SIZE, profiles/spmm_rows_c3_gate_traffic.json"
+        else:
+            traffic_note = "profiles/spmm_rows_c3_gate_traffic.json was recorded for other kernel sources (%s)" % rec.get("kernel_source_sha16")
     out = {
         "metric": "ternary SpMM GB/s (% HBM peak) + tokens/s, Llama-2-7B ternary MLP shape",
         "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -220,23 +277,25 @@ def main():
         "config": {"workload": "Llama-2-7B ternary MLP gate projection SpMM: M=1024 (8x128 tokens), K=4096, N=11008, "
                                "80% sparsity, fp16 activations, per-output fp16 scale, u8 tile-local indices",
                    "M": M, "K": K, "N": N, "sparsity": sparsity, "nnz": int(nnz), "algorithmic_bytes": int(B),
-                   "x_layout": "K-major [K][M]", "max_rel_err": max_rel},
+                   "x_layout": "row-major [M][K]", "max_rel_err": max_rel},
         "pct_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 3),
         "tokens_per_s": round(M / (wall_ms * 1e-3), 1),
         "roofline": {"bound": "hbm", "achieved": round(B / (ev_ms * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(B / (ev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 5), "traffic": traffic,
-                     "kernel": "tl_spmm_rows<__half, 4, 8, 16, false> + tl_rows_fixup<__half, 4, 8, 16, false> (the two launches of one tl_spmm call)",
+                     "frac": round(B / (ev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 5), "traffic": traffic, "traffic_note": traffic_note,
+                     "kernel": "tl_relayout_x<__half> + tl_spmm_rows<__half, 4, 8, 16, false> + tl_rows_fixup<__half, 4, 8, 16, false> "
+                               "(the three launches of one tl_spmm call on row-major activations)",
                      "kernel_ms": round(ev_ms, 5)},
     }
     extra = {
         "gadd_per_s": round(M * nnz / (ev_ms * 1e-3) / 1e9, 1),
         "valu_add_roofline_frac": round(M * nnz / (ev_ms * 1e-3) / 1e9 / VALU_PEAK_GADDS, 4),
         "gop_equiv_per_s": round(2.0 * M * K * N / (ev_ms * 1e-3) / 1e9, 1),
-        "row_major_input_ms_per_step": round(wall_rm_ms, 5),
+        "k_major_input": {"ms_per_step": round(wall_km_ms, 5), "kernel_ms": round(ev_km_ms, 5),
+                          "note": "activations handed over as [K][M]: no re-layout pre-pass"},
     }
     # the reference's own statistic (benchmark_ternary_mlp.py:51-53,98): 100 single calls timed one by one,
     # mean of the fastest 10; median and 10th percentile beside it
-    singles = sorted(ops.spmm_time(dw, xk, 1, sd, x_layout=_lib.TL_X_K_MAJOR)[0] for _ in range(100))
+    singles = sorted(ops.spmm_time(dw, xd, 1, sd)[0] for _ in range(100))
     extra["headline_single_call_ms"] = {"best10_of_100_mean": round(best_k_mean(singles, 10), 5), "median": round(singles[50], 5),
                                         "p10": round(singles[10], 5)}
 
@@ -301,6 +360,7 @@ def main():
         mlp_ms = (time.perf_counter() - t0) * 1e3 / 10
         extra["c3_mlp_block_fused"] = {"ms": round(mlp_ms, 4), "tokens_per_s": round(M / (mlp_ms * 1e-3), 1)}
     if not args.no_extra:
+        extra["balanced_vs_iid_weights"] = balanced_leg(dev, args.steps, args.warmup)
         extra["c2_decode_cold_weights_graph"] = cold_decode_leg(dev)
         if not args.no_cpu:
             try:  # the reference's decode kernel (ported) on the host's cores, same W, beside config 2
