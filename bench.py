@@ -35,6 +35,8 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--no-decoder", action="store_true", help="skip the 32-layer decoder (prefill 512 + 128 greedy steps)")
+    ap.add_argument("--only-decoder", action="store_true", help="of the secondary workloads run the 32-layer decoder alone (for profiling it)")
+    ap.add_argument("--only-decode-shapes", action="store_true", help="of the secondary workloads run the cold decode shapes alone (for profiling them)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one plain 256 MiB device copy (reference for scaling rocprof's FETCH_SIZE / WRITE_SIZE)")
     return ap.parse_args()
@@ -314,7 +316,8 @@ def main():
             out["cpu_baseline"] = {"value": None, "unit": "GB/s", "cores": 0, "kind": "port", "sample": "failed: %s" % e}
 
     # ---- the other regimes of the path ---------------------------------------
-    if not args.no_extra:
+    only = args.only_decoder or args.only_decode_shapes
+    if not args.no_extra and not only:
         # what a plain device copy reaches on this box, beside the 8 TB/s the fractions are quoted against
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
         dst = torch.empty_like(src)
@@ -359,10 +362,11 @@ def main():
         torch.cuda.synchronize()
         mlp_ms = (time.perf_counter() - t0) * 1e3 / 10
         extra["c3_mlp_block_fused"] = {"ms": round(mlp_ms, 4), "tokens_per_s": round(M / (mlp_ms * 1e-3), 1)}
-    if not args.no_extra:
-        extra["balanced_vs_iid_weights"] = balanced_leg(dev, args.steps, args.warmup)
+    if not args.no_extra and not args.only_decoder:
+        if not only:
+            extra["balanced_vs_iid_weights"] = balanced_leg(dev, args.steps, args.warmup)
         extra["c2_decode_cold_weights_graph"] = cold_decode_leg(dev)
-        if not args.no_cpu:
+        if not args.no_cpu and not only:
             try:  # the reference's decode kernel (ported) on the host's cores, same W, beside config 2
                 from oracle import cpu_baseline
                 w2, pw2, _ = weight_and_packed(4096, 4096, 0.66, 1244, dev)
@@ -377,7 +381,7 @@ def main():
         extra["decode_cold_shapes"] = [cold_decode_leg(dev, K, N, copies=24, calls=240, M=M)
                                        for K, N in ((4096, 4096), (4096, 11008), (11008, 4096)) for M in (1, 16)]
     # ---- whole decoder: 32 layers, every linear ternary at 66 % sparsity -------
-    if not args.no_extra and not args.no_decoder:
+    if not args.no_extra and not args.no_decoder and not args.only_decode_shapes:
         extra["c5_decoder"] = decoder_leg(dev)
     out["extra"] = extra
     print(json.dumps(out))

@@ -51,6 +51,9 @@ extern "C" {
 #define TL_X_K_MAJOR 1   /* X is [K][ldx], M contiguous (what the reference kernel itself reads, */
                          /* ter_spmm_kernel.cuh:173)                                            */
 
+#define TL_PRODUCER_SILU_GATE 1   /* tl_spmv_fused: x = silu(in[:K]) * in[K:]                  */
+#define TL_PRODUCER_ADD_RMSNORM 2 /* tl_spmv_fused: x = RMSNorm(in + in2) * norm_weight        */
+
 #define TL_ACT_NONE 0
 #define TL_ACT_SILU_GATE 1 /* out = silu(gate) * up, for tl_mlp_gate_up */
 
@@ -292,6 +295,21 @@ int tl_rope_cache_update(const void* qkv, int dtype, int64_t batch, int heads, i
 int tl_decode_attention(const void* q, const void* k_cache, const void* v_cache, int dtype,
                         int64_t batch, int heads, int head_dim, int64_t max_seq,
                         const int64_t* pos_dev, void* out, int64_t out_kmajor_ld, void* stream);
+
+/* Y[N] = (x * W) * scale for ONE activation row x that the call produces itself, so that a decode step
+ * needs neither a launch nor a trip through memory for the producer (the reference leaves these steps to
+ * separate torch operators, TernaryLLM/TernaryMLP.py:34 and the Hugging Face decoder layer it patches):
+ *   TL_PRODUCER_SILU_GATE    x[k] = silu(in[k]) * in[K + k], `in` a side-by-side gate | up row of 2K values
+ *                            (tl_silu_mul followed by tl_spmm); in2, norm_weight, sum_out must be NULL
+ *   TL_PRODUCER_ADD_RMSNORM  s = in + in2 (in2 may be NULL), x = s * rsqrt(mean(s^2) + eps) * norm_weight;
+ *                            s is also written to sum_out when that is not NULL (tl_add_rmsnorm followed
+ *                            by tl_spmm).  sum_out must not alias in or in2.
+ * in, in2, norm_weight, sum_out are of x_dtype, K values each (2K for the gate | up row), 16-byte aligned.
+ * Roundings are those of the separate kernels.  TL_ERR_UNSUPPORTED when K or the blob's tile height is not
+ * a whole number of 16-byte pieces (use the separate kernels then). */
+int tl_spmv_fused(const tl_layout_header* header, const void* blob_dev, int producer,
+                  const void* in, const void* in2, const void* norm_weight, float eps, void* sum_out, int x_dtype,
+                  void* Y, int y_dtype, const void* scale, int scale_dtype, void* stream);
 
 /* x_out = x + y, h_out = RMSNorm(x_out) * weight, row by row ([rows][width], one dtype): the residual
  * add of a decoder layer fused with the normalisation that follows (the reference leaves both to the

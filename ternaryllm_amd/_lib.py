@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(_DIR, "libternary_spmm.so")
 TL_F32, TL_F16 = 0, 1
 TL_X_ROW_MAJOR, TL_X_K_MAJOR = 0, 1
 TL_ACT_SILU_GATE = 1
+TL_PRODUCER_SILU_GATE, TL_PRODUCER_ADD_RMSNORM = 1, 2
 TL_LAYOUT_MAGIC = 0x35474C54
 
 ERROR_NAMES = {
@@ -67,6 +68,7 @@ SIGNATURES = {
     "tl_spmm_workspace": (_INT, [_HDRP, _I64, _INT, _INT, _I64P]),
     "tl_spmm": (_INT, [_HDRP, _VP, _VP, _INT, _INT, _I64, _I64, _VP, _INT, _I64, _VP, _INT, _VP, _I64, _VP]),
     "tl_spmm_noalloc": (_INT, [_HDRP, _VP, _VP, _INT, _INT, _I64, _I64, _VP, _INT, _I64, _VP, _INT, _VP]),
+    "tl_spmv_fused": (_INT, [_HDRP, _VP, _INT, _VP, _VP, _VP, ctypes.c_float, _VP, _INT, _VP, _INT, _VP, _INT, _VP]),
     "tl_mlp_gate_up": (_INT, [_HDRP, _VP, _HDRP, _VP, _VP, _INT, _INT, _I64, _I64, _VP, _INT, _I64, _VP, _VP, _INT, _INT,
                               _VP, _I64, _VP]),
     "tl_spmm_time": (_INT, [_HDRP, _VP, _VP, _INT, _INT, _I64, _I64, _VP, _INT, _I64, _VP, _INT, _VP, _I64, _VP, _INT,

@@ -73,6 +73,11 @@ struct KernelArgs {
     int split_first_unit;   // row kernel: first output tile of those whose steps are shared out
     float* partial;         // row kernel: partial sums of output tiles whose K tiles were shared out
     float one;  // 1.0f, passed in so that the fp16 -> fp32 accumulate stays a single mixed-precision fma
+    // single-row kernel with a fused producer of its input (tl_spmv_fused)
+    const void* X2;       // second summand of the residual add, or null
+    const void* norm_w;   // RMSNorm weight [K]
+    void* sum_out;        // where the first workgroup writes X + X2, or null
+    float eps;
 };
 
 __device__ __forceinline__ float load_scale(const void* scale, int is_f16, int n)
@@ -617,7 +622,25 @@ __global__ __launch_bounds__(kBlockThreads) void tl_spmm_quad(KernelArgs a)
 // (TP tiles side by side, LW lanes per run, one dword per lane and pass, two tiles' reads issued
 // together), and fold their sums with cross-lane shuffles.  When all of K fits the LDS there is a
 // single group: every load of the workgroup is in flight at once and nothing is staged twice.
-template <bool XF16, int NT>
+//
+// PRO names what produces the row: kProNone, the row lies in memory (copied by direct loads); with the other
+// two the workgroup computes it while the chunks are on their way, every workgroup for itself (a row is a
+// few thousand values), so that the producer needs no launch and no trip through memory of its own:
+//   kProSiluGate  x[k] = silu(in[k]) * in[K + k] for a side-by-side gate | up row `in` of 2K values;
+//   kProAddNorm   s = in + in2 (in2 may be null), x = s * rsqrt(mean(s^2) + eps) * norm_w; the first workgroup
+//                 also writes s to sum_out (the residual stream of a decoder layer).
+// Roundings are those of the separate kernels (tl_silu_mul, tl_add_rmsnorm): s, the SiLU and x are rounded to
+// the activation type.
+constexpr int kProNone = 0, kProSiluGate = 1, kProAddNorm = 2;
+
+template <bool F16>
+__device__ __forceinline__ float round_to_x(float v)
+{
+    if constexpr (F16) return __half2float(__float2half(v));
+    else return v;
+}
+
+template <bool XF16, int NT, int PRO = kProNone>
 __global__ __launch_bounds__(NT) void tl_spmv_direct(KernelArgs a)
 {
     extern __shared__ __align__(16) unsigned char lds[];
@@ -637,6 +660,38 @@ __global__ __launch_bounds__(NT) void tl_spmv_direct(KernelArgs a)
     const unsigned char* Xb = static_cast<const unsigned char*>(a.X);
     using global_ptr = const __attribute__((address_space(1))) void*;
     using lds_ptr = __attribute__((address_space(3))) void*;
+    float inv_rms = 1.0f;  // kProAddNorm: rsqrt(mean(s^2) + eps), known before any tile is staged
+
+    // the 16-byte piece of the row that starts at value k, as the producer makes it
+    auto produce = [&](int k) -> u32x4 {
+        u32x4 out;
+        XT* o = reinterpret_cast<XT*>(&out);
+        if constexpr (PRO == kProSiluGate) {
+            const u32x4 gv = *reinterpret_cast<const u32x4*>(Xb + (size_t)k * ES);
+            const u32x4 uv = *reinterpret_cast<const u32x4*>(Xb + ((size_t)a.K + k) * ES);
+            const XT* g = reinterpret_cast<const XT*>(&gv);
+            const XT* u = reinterpret_cast<const XT*>(&uv);
+#pragma unroll
+            for (int e = 0; e < VE; ++e) {
+                const float gf = (float)g[e];
+                o[e] = XT(round_to_x<XF16>(gf / (1.0f + __expf(-gf))) * (float)u[e]);
+            }
+        } else {
+            const u32x4 xv = *reinterpret_cast<const u32x4*>(Xb + (size_t)k * ES);
+            const u32x4 wv = *reinterpret_cast<const u32x4*>(static_cast<const unsigned char*>(a.norm_w) + (size_t)k * ES);
+            u32x4 yv = u32x4{0u, 0u, 0u, 0u};
+            if (a.X2) yv = *reinterpret_cast<const u32x4*>(static_cast<const unsigned char*>(a.X2) + (size_t)k * ES);
+            const XT* x = reinterpret_cast<const XT*>(&xv);
+            const XT* y = reinterpret_cast<const XT*>(&yv);
+            const XT* w = reinterpret_cast<const XT*>(&wv);
+#pragma unroll
+            for (int e = 0; e < VE; ++e) {
+                const float sv = a.X2 ? round_to_x<XF16>((float)x[e] + (float)y[e]) : (float)x[e];
+                o[e] = XT(sv * inv_rms * (float)w[e]);
+            }
+        }
+        return out;
+    };
 
     auto issue = [&](int t, int nt, int which) {
         unsigned char* xs = lds + which * stage_bytes;
@@ -646,17 +701,26 @@ __global__ __launch_bounds__(NT) void tl_spmv_direct(KernelArgs a)
         for (int first = wave * 64; first < vectors; first += NT)
             if (first + lane < vectors)
                 __builtin_amdgcn_global_load_lds((global_ptr)(a.w0.stream + lo + (size_t)(first + lane) * 4), (lds_ptr)(buf + (size_t)first * 16), 16, 0, 0);
+        if (tid <= nt) cst[which * (TG + 1) + tid] = cs[t + tid] - lo;
+    };
+    // the tile images of the group: copies of the row's pieces (or what the producer makes of them), zeros behind a tile's rows
+    auto stage_row = [&](int t, int nt, int which) {
+        unsigned char* xs = lds + which * stage_bytes;
         const int pieces = nt * PPT;  // images lie back to back, PPT pieces each (the last one or two of an image only ever hold zeros)
         for (int first = wave * 64; first < pieces; first += NT) {
             const int p = first + lane, tile = p / PPT, k = (t + tile) * a.tile_rows + (p % PPT) * VE;
             if (p < pieces) {
-                if ((p % PPT) * VE < a.tile_rows && k < a.K)
-                    __builtin_amdgcn_global_load_lds((global_ptr)(Xb + (size_t)k * ES), (lds_ptr)(xs + (size_t)first * 16), 16, 0, 0);
-                else
-                    *reinterpret_cast<u32x4*>(xs + (size_t)p * 16) = u32x4{0u, 0u, 0u, 0u};
+                const bool real = (p % PPT) * VE < a.tile_rows && k < a.K;
+                if constexpr (PRO == kProNone) {
+                    if (real)
+                        __builtin_amdgcn_global_load_lds((global_ptr)(Xb + (size_t)k * ES), (lds_ptr)(xs + (size_t)first * 16), 16, 0, 0);
+                    else
+                        *reinterpret_cast<u32x4*>(xs + (size_t)p * 16) = u32x4{0u, 0u, 0u, 0u};
+                } else {
+                    *reinterpret_cast<u32x4*>(xs + (size_t)p * 16) = real ? produce(k) : u32x4{0u, 0u, 0u, 0u};
+                }
             }
         }
-        if (tid <= nt) cst[which * (TG + 1) + tid] = cs[t + tid] - lo;
     };
 
     const int lpc_shift = a.lpc_shift, lw_shift = a.lw_shift;
@@ -667,12 +731,45 @@ __global__ __launch_bounds__(NT) void tl_spmv_direct(KernelArgs a)
     constexpr int TU = 2;  // tiles of one lane whose LDS reads are issued together
 
     issue(0, min(TG, a.T), 0);
+    if constexpr (PRO == kProAddNorm) {
+        // mean square of s = in + in2 over the row, while the chunks are on their way; the first workgroup keeps s
+        float* red = reinterpret_cast<float*>(cst + buffers * (TG + 1));  // [NT / 64]
+        float ss = 0.f;
+        for (int v = tid; v < a.K / VE; v += NT) {
+            const u32x4 xv = *reinterpret_cast<const u32x4*>(Xb + (size_t)v * 16);
+            u32x4 sv = xv;
+            if (a.X2) {
+                const u32x4 yv = *reinterpret_cast<const u32x4*>(static_cast<const unsigned char*>(a.X2) + (size_t)v * 16);
+                const XT* x = reinterpret_cast<const XT*>(&xv);
+                const XT* y = reinterpret_cast<const XT*>(&yv);
+                XT* o = reinterpret_cast<XT*>(&sv);
+#pragma unroll
+                for (int e = 0; e < VE; ++e) o[e] = XT((float)x[e] + (float)y[e]);
+            }
+            const XT* sp = reinterpret_cast<const XT*>(&sv);
+#pragma unroll
+            for (int e = 0; e < VE; ++e) ss = fmaf((float)sp[e], (float)sp[e], ss);
+            if (nb == 0 && a.sum_out) *reinterpret_cast<u32x4*>(static_cast<unsigned char*>(a.sum_out) + (size_t)v * 16) = sv;
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+        if (lane == 0) red[wave] = ss;
+        __syncthreads();
+        float total = 0.f;
+#pragma unroll
+        for (int v = 0; v < NT / 64; ++v) total += red[v];
+        inv_rms = rsqrtf(total / (float)a.K + a.eps);
+    }
+    stage_row(0, min(TG, a.T), 0);
     int which = 0;
     for (int t = 0; t < a.T; t += TG, which ^= 1) {
         const int nt = min(TG, a.T - t);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        if (t + TG < a.T) issue(t + TG, min(TG, a.T - t - TG), which ^ 1);
+        if (t + TG < a.T) {
+            issue(t + TG, min(TG, a.T - t - TG), which ^ 1);
+            stage_row(t + TG, min(TG, a.T - t - TG), which ^ 1);
+        }
         const XT* xs = reinterpret_cast<const XT*>(lds + which * stage_bytes);
         const uint32_t* buf = reinterpret_cast<const uint32_t*>(lds + which * stage_bytes + a.xs_bytes);
         const uint32_t* my_cst = cst + which * (TG + 1);
@@ -1439,7 +1536,7 @@ int launch_quad_kernel(KernelArgs a, const tl_layout_header* h, hipStream_t st)
 
 // The direct-load kernel for one activation row.  All of K in one group when `share` workgroups of that
 // size fit a compute unit, else two alternating buffers of TG tiles.
-template <bool XF16, int NT>
+template <bool XF16, int NT, int PRO = kProNone>
 int launch_spmv_direct_nt(KernelArgs a, const tl_layout_header* h, hipStream_t st)
 {
     constexpr int es = XF16 ? 2 : 4;
@@ -1455,7 +1552,7 @@ int launch_spmv_direct_nt(KernelArgs a, const tl_layout_header* h, hipStream_t s
     a.xs_bytes = tg * tile_bytes;
     a.buf_bytes = (int)round_up((int64_t)tg * chunk_bytes, 16);
     const int buffers = tg < a.T ? 2 : 1;
-    const size_t lds = (size_t)buffers * ((size_t)a.xs_bytes + a.buf_bytes) + (size_t)buffers * (tg + 1) * 4;
+    const size_t lds = (size_t)buffers * ((size_t)a.xs_bytes + a.buf_bytes) + (size_t)buffers * (tg + 1) * 4 + (NT / 64) * 4;  // + the waves' partial mean squares
     if (lds > 160 * 1024) return fail(TL_ERR_UNSUPPORTED, "one tile needs %zu bytes of LDS", lds);
     const int lpc = NT / TL_BLOCK_COLUMNS;
     const double mean_run = h->mean_run_dwords_x16 / 16.0;
@@ -1465,7 +1562,7 @@ int launch_spmv_direct_nt(KernelArgs a, const tl_layout_header* h, hipStream_t s
     if (lw < 1 || (lw & (lw - 1))) return fail(TL_ERR_ARG, "TL_LW=%d (a power of two expected)", lw);
     a.lpc_shift = log2_exact(lpc);
     a.lw_shift = log2_exact(lw);
-    auto kernel = tl_spmv_direct<XF16, NT>;
+    auto kernel = tl_spmv_direct<XF16, NT, PRO>;
     static bool raised = false;  // per instantiation; a repeated or racing call is harmless
     if (!raised) {
         if (int rc = raise_lds_limit(kernel, 160 * 1024)) return rc;
@@ -1477,11 +1574,11 @@ int launch_spmv_direct_nt(KernelArgs a, const tl_layout_header* h, hipStream_t s
 
 // With no more blocks than compute units a workgroup has its compute unit to itself: 1024 threads
 // (64 lanes per column) then keep more gathers in flight than 512 do.
-template <bool XF16>
+template <bool XF16, int PRO = kProNone>
 int launch_spmv_direct(const KernelArgs& a, const tl_layout_header* h, hipStream_t st)
 {
     const bool wide = knob(TL_SPMV_WIDE, a.NB <= compute_units() ? 1 : 0) != 0;
-    return wide ? launch_spmv_direct_nt<XF16, 1024>(a, h, st) : launch_spmv_direct_nt<XF16, kBlockThreads>(a, h, st);
+    return wide ? launch_spmv_direct_nt<XF16, 1024, PRO>(a, h, st) : launch_spmv_direct_nt<XF16, kBlockThreads, PRO>(a, h, st);
 }
 
 template <int MT>
@@ -1801,6 +1898,47 @@ extern "C" int tl_spmm_noalloc(const tl_layout_header* header, const void* blob_
     void* ws = nullptr;
     if (int rc = static_scratch(&ws)) return rc;
     return tl_spmm(header, blob_dev, X, x_dtype, x_layout, ldx, M, Y, y_dtype, ldy, scale, scale_dtype, ws, need, stream);
+}
+
+extern "C" int tl_spmv_fused(const tl_layout_header* header, const void* blob_dev, int producer,
+                             const void* in, const void* in2, const void* norm_weight, float eps, void* sum_out, int x_dtype,
+                             void* Y, int y_dtype, const void* scale, int scale_dtype, void* stream)
+{
+    if (int rc = check_header(header)) return rc;
+    if (int rc = check_dtype(x_dtype, "x")) return rc;
+    if (int rc = check_dtype(y_dtype, "y")) return rc;
+    if (scale)
+        if (int rc = check_dtype(scale_dtype, "scale")) return rc;
+    if (producer != TL_PRODUCER_SILU_GATE && producer != TL_PRODUCER_ADD_RMSNORM) return fail(TL_ERR_ARG, "producer code %d unknown", producer);
+    if (!blob_dev || !in || !Y) return fail(TL_ERR_ARG, "device pointer is null");
+    if (reinterpret_cast<uintptr_t>(blob_dev) % 256) return fail(TL_ERR_ALIGN, "weight blob must be 256-byte aligned");
+    if (producer == TL_PRODUCER_ADD_RMSNORM && !norm_weight) return fail(TL_ERR_ARG, "norm_weight is null");
+    if (producer == TL_PRODUCER_SILU_GATE && (in2 || sum_out)) return fail(TL_ERR_ARG, "in2 and sum_out belong to TL_PRODUCER_ADD_RMSNORM");
+    if (sum_out && (sum_out == in || sum_out == in2)) return fail(TL_ERR_ARG, "sum_out must not be one of the inputs: other workgroups still read them");
+    const int es = x_dtype == TL_F16 ? 2 : 4, ve = 16 / es;
+    // what the direct-load kernel needs of a row: whole aligned 16-byte pieces per tile
+    if (header->tile_rows % ve || header->inners % ve)
+        return fail(TL_ERR_UNSUPPORTED, "K=%u, tile height %u: the fused single-row kernel needs whole 16-byte pieces per tile", header->inners, header->tile_rows);
+    for (const void* p : {in, in2, norm_weight, static_cast<const void*>(sum_out)})
+        if (reinterpret_cast<uintptr_t>(p) % 16) return fail(TL_ERR_ALIGN, "in, in2, norm_weight and sum_out must be 16-byte aligned");
+    KernelArgs a;
+    std::memset(&a, 0, sizeof(a));
+    a.w0 = weight_ptrs(header, blob_dev, scale);
+    a.X = in; a.X2 = in2; a.norm_w = norm_weight; a.sum_out = sum_out; a.eps = eps;
+    a.Y = Y;
+    a.ldx = header->inners; a.ldy = header->columns;
+    a.M = 1; a.N = (int)header->columns; a.K = (int)header->inners; a.T = (int)header->n_tiles; a.tile_rows = (int)header->tile_rows;
+    a.NB = (int)header->n_blocks;
+    a.x_f16 = x_dtype == TL_F16; a.y_f16 = y_dtype == TL_F16; a.scale_f16 = scale_dtype == TL_F16;
+    a.one = 1.0f;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    int rc;
+    if (producer == TL_PRODUCER_SILU_GATE)
+        rc = a.x_f16 ? launch_spmv_direct<true, kProSiluGate>(a, header, st) : launch_spmv_direct<false, kProSiluGate>(a, header, st);
+    else
+        rc = a.x_f16 ? launch_spmv_direct<true, kProAddNorm>(a, header, st) : launch_spmv_direct<false, kProAddNorm>(a, header, st);
+    if (rc) return rc;
+    return finish_launch();
 }
 
 extern "C" int tl_mlp_gate_up(const tl_layout_header* gate_header, const void* gate_blob_dev,

@@ -121,6 +121,12 @@ class TernaryLlamaDecoder(nn.Module):
         self._graph = None
         # single-token steps use the library's rotary / cache / attention kernels; False keeps them on torch operators
         self.native_decode = config.head_dim in (64, 128, 256) and self.max_seq_len * 4 <= 120 * 1024
+        # single-row steps fold the norms and the SiLU gate into the products' kernels; that kernel wants rows and
+        # tiles of whole 16-byte pieces
+        self.fused_decode = all(m._header.tile_rows % 8 == 0 and m.in_features % 8 == 0
+                                for layer in self.layers for m in (layer.qkv_proj, layer.gate_up_proj, layer.down_proj)) and \
+            self.lm_head._header.tile_rows % 8 == 0 and H % 8 == 0
+        self._layer_index = {id(layer): i for i, layer in enumerate(self.layers)}
 
     # -- pieces ------------------------------------------------------------------------------
     @staticmethod
@@ -208,6 +214,8 @@ class TernaryLlamaDecoder(nn.Module):
         eps = c.rms_norm_eps
         # 5 to 48 rows: the products read a K-major image, so whatever feeds one writes it in that layout
         # (its transpose as a view) and no re-layout pass runs in front of the products
+        if B == 1 and self.fused_decode:
+            return self._decode_step_fused(x, pos, q)
         km = 5 <= B <= 48 and c.hidden_size != B and c.intermediate_size != B
         _, h = ops.add_rmsnorm(x, None, self.layers[0].input_layernorm.weight, eps, kmajor=km)
         for li, layer in enumerate(self.layers):
@@ -219,6 +227,26 @@ class TernaryLlamaDecoder(nn.Module):
             nxt = self.layers[li + 1].input_layernorm.weight if li + 1 < len(self.layers) else self.norm.weight
             x, h = ops.add_rmsnorm(x, y, nxt, eps, kmajor=km)  # the residual add, and the norm the next layer (or the head) starts with
         return self.lm_head(h)
+
+    def _decode_step_fused(self, x, pos, q):
+        """One row: the residual add + RMSNorm in front of the q|k|v and gate|up products and the SiLU gate in
+        front of the down projection are computed inside those products' kernels (tl_spmv_fused), six launches
+        per layer instead of nine."""
+        eps = self.config.rms_norm_eps
+        y = None   # what the previous block still has to add to the residual stream
+        for layer in self.layers:
+            qkv, x = ops.spmv_fused(layer.qkv_proj.device_weight(), "add_rmsnorm", x, y, layer.input_layernorm.weight, eps,
+                                    layer.qkv_proj.w_scale, want_sum=True)
+            ops.rope_cache_update(qkv, self.rope_cos, self.rope_sin, pos, q, self._cache_of(layer, 0), self._cache_of(layer, 1))
+            a = ops.decode_attention(q, self._cache_of(layer, 0), self._cache_of(layer, 1), pos)
+            o = layer.o_proj(a)
+            gu, x = ops.spmv_fused(layer.gate_up_proj.device_weight(), "add_rmsnorm", x, o, layer.post_attention_layernorm.weight, eps,
+                                   layer.gate_up_proj.w_scale, want_sum=True)
+            y = ops.spmv_fused(layer.down_proj.device_weight(), "silu_gate", gu, scale=layer.down_proj.w_scale)
+        return ops.spmv_fused(self.lm_head.device_weight(), "add_rmsnorm", x, y, self.norm.weight, eps, self.lm_head.w_scale)
+
+    def _cache_of(self, layer, which):
+        return self._cache[self._layer_index[id(layer)], which]
 
     @torch.no_grad()
     def generate(self, tokens, new_tokens, use_graph=True):

@@ -160,6 +160,36 @@ def mlp_gate_up(gate, up, x, gate_scale=None, up_scale=None, out_dtype=None):
     return h
 
 
+def spmv_fused(weight, producer, inp, inp2=None, norm_weight=None, eps=0.0, scale=None, out_dtype=None, want_sum=False):
+    """y[1, N] = (x @ W) * scale for one activation row x that the call produces itself (tl_spmv_fused):
+    producer "silu_gate": x = silu(inp[:K]) * inp[K:] for a gate | up row inp of 2K values;
+    producer "add_rmsnorm": s = inp + inp2 (inp2 may be None), x = rmsnorm(s) * norm_weight; with want_sum the
+    call also returns s (a new tensor).  Returns y, or (y, s).  Raises RuntimeError (TL_ERR_UNSUPPORTED) where the
+    fused kernel does not apply (K or the tile height not whole 16-byte pieces); callers then use the separate operators."""
+    K, N = weight.inners, weight.columns
+    code = {"silu_gate": _lib.TL_PRODUCER_SILU_GATE, "add_rmsnorm": _lib.TL_PRODUCER_ADD_RMSNORM}[producer]
+    x_code = _code(inp.dtype, "inp")
+    need = 2 * K if producer == "silu_gate" else K
+    tensors = [inp] + [t for t in (inp2, norm_weight) if t is not None]
+    for t in tensors:
+        if t.numel() != (need if t is inp else K) or not t.is_contiguous() or t.dtype != inp.dtype or t.device != weight.device:
+            raise ValueError("inputs must be contiguous rows of the weight's K (2K for a gate | up row), one dtype, on the weight's device")
+    if producer == "add_rmsnorm" and norm_weight is None:
+        raise ValueError("add_rmsnorm needs norm_weight")
+    out_dtype = out_dtype or inp.dtype
+    y = torch.empty((1, N), dtype=out_dtype, device=inp.device)
+    s_out = torch.empty(K, dtype=inp.dtype, device=inp.device).view(inp.shape) if (want_sum and producer == "add_rmsnorm") else None
+    scale, s_code = _scale_args(scale, N, inp.device)
+    with torch.cuda.device(inp.device):
+        rc = _lib.lib().tl_spmv_fused(ctypes.byref(weight.header), weight.blob.data_ptr(), code, inp.data_ptr(),
+                                      inp2.data_ptr() if inp2 is not None else None,
+                                      norm_weight.data_ptr() if norm_weight is not None else None, float(eps),
+                                      s_out.data_ptr() if s_out is not None else None, x_code, y.data_ptr(), _code(out_dtype, "out_dtype"),
+                                      scale.data_ptr() if scale is not None else None, s_code, _stream_ptr(inp.device))
+    _lib.check(rc)
+    return (y, s_out) if want_sum else y
+
+
 def spmm_time(weight, x, iters, scale=None, out_dtype=None, x_layout=_lib.TL_X_ROW_MAJOR):
     """Mean milliseconds per tl_spmm call over `iters` back-to-back calls, timed with HIP events
     recorded on the stream the kernels run on.  Returns (ms, y)."""

@@ -240,6 +240,76 @@ def test_add_rmsnorm_and_silu_mul(cuda):
             assert torch.equal(ops.silu_mul(gu, kmajor=True).t(), out)
 
 
+@pytest.mark.parametrize("dtype,tol", [(torch.float16, 2e-3), (torch.float32, 1e-5)])
+def test_fused_producers_of_the_single_row_product(cuda, oracle, dtype, tol):
+    """tl_spmv_fused: the residual add + RMSNorm and the SiLU gate computed inside the product's kernel, against a
+    float64 restatement and against the separate kernels followed by the plain product."""
+    from tests.util import max_rel_err, ternary_weight
+    from ternaryllm_amd import ops
+    from ternaryllm_amd.packing import PackedWeight
+    g = torch.Generator().manual_seed(14)
+    for K, N in ((4096, 272), (11008, 96), (1000, 40)):   # one group of tiles; many tiles; a ragged last tile and block
+        w = ternary_weight(K, N, 0.7, K + N)
+        dw = ops.DeviceWeight(PackedWeight.from_dense(w), cuda)
+        sc = (0.5 + torch.rand(N, generator=g)).to(dtype).to(cuda)
+        x = torch.randn(K, generator=g).to(dtype).to(cuda)
+        y = torch.randn(K, generator=g).to(dtype).to(cuda)
+        nw = (1 + 0.1 * torch.randn(K, generator=g)).to(dtype).to(cuda)
+        gu = torch.randn(2 * K, generator=g).to(dtype).to(cuda)
+        wd = w.astype("float64")
+        for second in (y, None):
+            out, s = ops.spmv_fused(dw, "add_rmsnorm", x, second, nw, 1e-5, sc, want_sum=True)
+            s_ref = (x + second) if second is not None else x
+            assert torch.equal(s, s_ref)
+            h64 = s_ref.double() * torch.rsqrt(s_ref.double().pow(2).mean() + 1e-5) * nw.double()
+            ref = (h64.cpu().numpy()[None, :] @ wd) * sc.double().cpu().numpy()[None, :]
+            # the activation row is rounded to its type before the product: allow for that rounding on top of the product's
+            assert max_rel_err(out.double().cpu().numpy(), ref, h64.cpu().numpy()[None, :], w) <= 2 * tol
+            _, h = ops.add_rmsnorm(x[None], second[None] if second is not None else None, nw, 1e-5)
+            unfused = ops.spmm(dw, h, sc)
+            assert max_rel_err(out.double().cpu().numpy(), unfused.double().cpu().numpy(), h.double().cpu().numpy(), w) <= tol
+        out = ops.spmv_fused(dw, "silu_gate", gu, scale=sc)
+        a64 = torch.nn.functional.silu(gu[:K].double()) * gu[K:].double()
+        ref = (a64.cpu().numpy()[None, :] @ wd) * sc.double().cpu().numpy()[None, :]
+        assert max_rel_err(out.double().cpu().numpy(), ref, a64.cpu().numpy()[None, :], w) <= 2 * tol
+        unfused = ops.spmm(dw, ops.silu_mul(gu[None]), sc)
+        assert torch.equal(out, unfused)   # same roundings, same kernel behind the staging: bit for bit
+    with pytest.raises(RuntimeError, match="UNSUPPORTED"):   # a tile height that is not whole 16-byte pieces: the separate kernels are the way then
+        odd = ops.DeviceWeight(PackedWeight.from_dense(ternary_weight(1000, 40, 0.7, 3), tile_rows=250), cuda)
+        ops.spmv_fused(odd, "silu_gate", torch.zeros(2000, dtype=dtype, device=cuda))
+
+
+def test_fused_single_row_step_equals_the_unfused_one(tiny, cuda):
+    """Batch 1: the step with the norms and the SiLU gate folded into the products against the same step on
+    separate kernels, eager and as a replayed graph."""
+    g = torch.Generator().manual_seed(21)
+    tokens = torch.randint(0, tiny.config.vocab_size, (1, 30), generator=g).to(cuda)
+    assert tiny.fused_decode
+    outs = {}
+    for fused in (False, True):
+        tiny.fused_decode = fused
+        tiny._graph = None
+        tiny.prefill(tokens[:, :28])
+        st = tiny._decode_state(1)
+        logits = []
+        for j in range(2):
+            st["token"].copy_(tokens[:, 28 + j])
+            st["pos"].fill_(28 + j)
+            st["mask"].copy_((torch.arange(tiny.max_seq_len, device=cuda) <= 28 + j)[None, None, None])
+            logits.append(tiny._decode_step(st["token"], st["pos"], st["mask"]).float())
+        outs[fused] = torch.stack(logits)
+    tiny.fused_decode = True
+    tiny._state = None
+    tiny._graph = None
+    assert (outs[True] - outs[False]).abs().max().item() <= 2e-3 * outs[False].abs().max().item()
+    eager = tiny.generate(tokens, 10, use_graph=False)
+    graphed = tiny.generate(tokens, 10, use_graph=True)
+    again = tiny.generate(tokens, 10, use_graph=True)
+    assert torch.equal(eager, graphed) and torch.equal(eager, again)
+    tiny._graph = None
+    tiny._state = None
+
+
 def test_graph_replay_equals_eager_decode(tiny, cuda):
     g = torch.Generator().manual_seed(4)
     tokens = torch.randint(0, tiny.config.vocab_size, (3, 40), generator=g).to(cuda)
