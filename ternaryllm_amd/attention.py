@@ -130,6 +130,20 @@ class LlamaTernaryAttention(nn.Module):
         return self.o_proj(attn), attn_weights, past_key_value
 
 
+class TwoResultAttention(nn.Module):
+    """Adapter for `transformers` releases whose decoder layer unpacks two results from `self_attn`
+    (attn_output, attn_weights) and hands the cache over as `past_key_values`: wraps a LlamaTernaryAttention,
+    which keeps the three results of the release the reference was written against (4.45)."""
+
+    def __init__(self, attention):
+        super().__init__()
+        self.attention = attention
+
+    def forward(self, *args, **kwargs):
+        out = self.attention(*args, **kwargs)
+        return out[0], out[1]
+
+
 def collect_attn_linear_layers(model):
     """(name, module) of the nn.Linear attention projections under `model` (TernaryAttn.py:134-140)."""
     return [(name, m) for name, m in model.named_modules()
@@ -148,4 +162,5 @@ def replace_linear_layers(layers, attn, sparsity=0.8, *, generator=None, referen
     torch.cuda.empty_cache()
 
 
-__all__ = ["LlamaTernaryAttention", "rope_tables", "apply_rope", "collect_attn_linear_layers", "replace_linear_layers"]
+__all__ = ["LlamaTernaryAttention", "TwoResultAttention", "rope_tables", "apply_rope", "collect_attn_linear_layers",
+           "replace_linear_layers"]

@@ -295,6 +295,51 @@ def test_surgery_on_a_hugging_face_llama(cuda):
     assert (got - ref).abs().max().item() <= 1e-3 * ref.abs().max().item()
 
 
+def test_attention_module_as_self_attn_of_a_hugging_face_llama(cuda):
+    """LlamaTernaryAttention in the place of `self_attn` of a transformers Llama built from a local config (what
+    the reference does to the model it patches, TernaryLlama.py:69-75): the decoder layer calls it with its own
+    keyword arguments (mask, position embeddings, cache); logits of a forward pass and of a cached two-step
+    continuation must equal those of the same model with dense projections holding the ternary weights."""
+    transformers = pytest.importorskip("transformers")
+    import copy
+    import inspect
+    from ternaryllm_amd import LlamaTernaryAttention, TernaryConfig
+    from ternaryllm_amd.attention import TwoResultAttention, collect_attn_linear_layers, replace_linear_layers
+    torch.manual_seed(21)
+    hf_cfg = transformers.LlamaConfig(hidden_size=128, intermediate_size=256, num_hidden_layers=2, num_attention_heads=4,
+                                      num_key_value_heads=2, vocab_size=120, max_position_embeddings=64)
+    model = transformers.LlamaForCausalLM(hf_cfg).eval().to(cuda)
+    dense = copy.deepcopy(model)
+    theta = getattr(hf_cfg, "rope_theta", None) or hf_cfg.rope_parameters["rope_theta"]
+    cfg = TernaryConfig(hidden_size=128, num_attention_heads=4, num_key_value_heads=2, sparsity=0.6, rope_theta=theta)
+    two_results = "past_key_values" in inspect.signature(type(model.model.layers[0].self_attn).forward).parameters
+    g = torch.Generator().manual_seed(22)
+    for li, layer in enumerate(model.model.layers):
+        attn = LlamaTernaryAttention(cfg, layer_idx=li, generator=g, reference_buffers=False).to(cuda)
+        layer.self_attn = TwoResultAttention(attn) if two_results else attn
+        twin = dense.model.layers[li].self_attn
+        for name in ("q_proj", "k_proj", "v_proj", "o_proj"):
+            getattr(twin, name).weight.data = getattr(attn, name).ternary_weight.t().float().contiguous().to(cuda)
+    ids = torch.randint(0, 120, (2, 20), generator=torch.Generator().manual_seed(23)).to(cuda)
+    with torch.no_grad():
+        got = model(ids).logits.float()
+        ref = dense(ids).logits.float()
+        assert torch.isfinite(ref).all()
+        assert (got - ref).abs().max().item() <= 1e-3 * ref.abs().max().item()
+        # prefill 18 tokens with a cache, then two single-token steps on top of it
+        out = model(ids[:, :18], use_cache=True)
+        cache = out.past_key_values
+        for j in (18, 19):
+            out = model(ids[:, j:j + 1], past_key_values=cache, use_cache=True)
+            cache = out.past_key_values
+            assert (out.logits[:, 0].float() - ref[:, j]).abs().max().item() <= 1e-3 * ref.abs().max().item()
+    # the reference's per-module helper: swap the nn.Linear projections of one attention module for random ternary ones
+    twin = dense.model.layers[0].self_attn
+    replace_linear_layers(collect_attn_linear_layers(twin), twin, 0.8)
+    from ternaryllm_amd import TernaryLinear
+    assert all(isinstance(getattr(twin, n), TernaryLinear) for n in ("q_proj", "k_proj", "v_proj", "o_proj"))
+
+
 @pytest.mark.parametrize("name,M,K,N,s,dtype", [
     ("config 1", 16, 4096, 4096, 0.5, torch.float32),
     ("config 2", 1, 4096, 4096, 0.66, torch.float16),
