@@ -519,15 +519,10 @@ __global__ __launch_bounds__(kBlockThreads) void tl_spmm_quad(KernelArgs a)
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int TG = a.tiles_per_group;
-    // The workgroup owns BS neighbouring blocks: the activation image of a group of tiles, by far the larger
-    // part of what is staged, then serves BS * 16 columns.
-    const int BS = a.block_set;
-    const int nb0 = blockIdx.x * BS, m0 = blockIdx.y * MT;
-    const int bs = min(BS, a.NB - nb0);  // blocks this workgroup really has
+    const int nb = blockIdx.x, m0 = blockIdx.y * MT;
     const int stage_bytes = a.xs_bytes + a.buf_bytes;
-    const int block_buf_bytes = a.buf_bytes / BS;  // chunk copies of one block and group (a multiple of 16)
-    uint32_t* cst = reinterpret_cast<uint32_t*>(lds + 2 * stage_bytes);  // [2][BS][TG + 1] chunk starts inside a block's chunk copies
-    const_u32_ptr cs = as_const(a.w0.chunkstart) + (size_t)nb0 * a.T;
+    uint32_t* cst = reinterpret_cast<uint32_t*>(lds + 2 * stage_bytes);  // [2][TG + 1] chunk starts inside a buffer's chunk copies
+    const_u32_ptr cs = as_const(a.w0.chunkstart) + (size_t)nb * a.T;
     const unsigned char* Xb = static_cast<const unsigned char*>(a.X) + (size_t)m0 * ES;
     const size_t row_bytes = (size_t)a.ldx * ES;
     using global_ptr = const __attribute__((address_space(1))) void*;
@@ -546,23 +541,17 @@ __global__ __launch_bounds__(kBlockThreads) void tl_spmm_quad(KernelArgs a)
             else
                 *reinterpret_cast<u32x4*>(xs + (size_t)p * 16) = u32x4{0u, 0u, 0u, 0u};
         }
-        for (int j = 0; j < bs; ++j) {
-            const_u32_ptr csj = cs + (size_t)j * a.T;
-            const uint32_t lo = csj[t];
-            const int vectors = (int)((csj[t + nt] - lo) / 4);
-            unsigned char* bufj = buf + (size_t)j * block_buf_bytes;
-            for (int first = wave * 64; first < vectors; first += NT)
-                if (first + lane < vectors)
-                    __builtin_amdgcn_global_load_lds((global_ptr)(a.w0.stream + lo + (size_t)(first + lane) * 4), (lds_ptr)(bufj + (size_t)first * 16), 16, 0, 0);
-            if (tid <= nt) cst[(which * BS + j) * (TG + 1) + tid] = csj[t + tid] - lo;
-        }
+        const uint32_t lo = cs[t];
+        const int vectors = (int)((cs[t + nt] - lo) / 4);
+        for (int first = wave * 64; first < vectors; first += NT)
+            if (first + lane < vectors)
+                __builtin_amdgcn_global_load_lds((global_ptr)(a.w0.stream + lo + (size_t)(first + lane) * 4), (lds_ptr)(buf + (size_t)first * 16), 16, 0, 0);
+        if (tid <= nt) cst[which * (TG + 1) + tid] = cs[t + tid] - lo;
     };
 
     const int lw_shift = a.lw_shift;
     const int LPC = 1 << a.lpc_shift, LW = 1 << lw_shift, TP = LPC >> lw_shift;
-    const int cols = TL_BLOCK_COLUMNS * BS;
-    const int q = tid % Q, col = (tid / Q) % cols, lig = tid / (Q * cols);
-    const int blk = col / TL_BLOCK_COLUMNS, c16 = col % TL_BLOCK_COLUMNS;
+    const int q = tid % Q, c16 = (tid / Q) & 15, lig = tid / (Q * TL_BLOCK_COLUMNS);
     const int tp = lig >> lw_shift, lw = lig & (LW - 1);
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
 
@@ -575,31 +564,29 @@ __global__ __launch_bounds__(kBlockThreads) void tl_spmm_quad(KernelArgs a)
         __syncthreads();
         if (t + TG < a.T) issue(t + TG, min(TG, a.T - t - TG), which ^ 1);
         const unsigned char* xs = lds + which * stage_bytes;
-        const uint32_t* buf = reinterpret_cast<const uint32_t*>(xs + a.xs_bytes + (size_t)blk * block_buf_bytes);
-        const uint32_t* my_cst = cst + (which * BS + blk) * (TG + 1);
-        if (blk < bs) {
-            for (int tl = tp; tl < nt; tl += TP) {
-                const uint32_t* chunk = buf + my_cst[tl];
-                const uint32_t d = chunk[c16];
-                const uint32_t* run = chunk + (d >> 16);
-                const int pd = run_pos_dwords(d), tot = pd + run_neg_dwords(d);
-                const XT* xq = reinterpret_cast<const XT*>(xs) + (size_t)tl * kTileSlots * MT + q * 4;
-                int i = lw;
-                for (; i + 3 * LW < tot; i += 4 * LW) {
-                    const uint32_t w0 = run[i], w1 = run[i + LW], w2 = run[i + 2 * LW], w3 = run[i + 3 * LW];
-                    gather_add_quad<MT, XT>(acc, xq, w0, i < pd ? 1.0f : -1.0f);
-                    gather_add_quad<MT, XT>(acc, xq, w1, i + LW < pd ? 1.0f : -1.0f);
-                    gather_add_quad<MT, XT>(acc, xq, w2, i + 2 * LW < pd ? 1.0f : -1.0f);
-                    gather_add_quad<MT, XT>(acc, xq, w3, i + 3 * LW < pd ? 1.0f : -1.0f);
-                }
-                if (i + LW < tot) {
-                    const uint32_t w0 = run[i], w1 = run[i + LW];
-                    gather_add_quad<MT, XT>(acc, xq, w0, i < pd ? 1.0f : -1.0f);
-                    gather_add_quad<MT, XT>(acc, xq, w1, i + LW < pd ? 1.0f : -1.0f);
-                    i += 2 * LW;
-                }
-                if (i < tot) gather_add_quad<MT, XT>(acc, xq, run[i], i < pd ? 1.0f : -1.0f);
+        const uint32_t* buf = reinterpret_cast<const uint32_t*>(xs + a.xs_bytes);
+        const uint32_t* my_cst = cst + which * (TG + 1);
+        for (int tl = tp; tl < nt; tl += TP) {
+            const uint32_t* chunk = buf + my_cst[tl];
+            const uint32_t d = chunk[c16];
+            const uint32_t* run = chunk + (d >> 16);
+            const int pd = run_pos_dwords(d), tot = pd + run_neg_dwords(d);
+            const XT* xq = reinterpret_cast<const XT*>(xs) + (size_t)tl * kTileSlots * MT + q * 4;
+            int i = lw;
+            for (; i + 3 * LW < tot; i += 4 * LW) {
+                const uint32_t w0 = run[i], w1 = run[i + LW], w2 = run[i + 2 * LW], w3 = run[i + 3 * LW];
+                gather_add_quad<MT, XT>(acc, xq, w0, i < pd ? 1.0f : -1.0f);
+                gather_add_quad<MT, XT>(acc, xq, w1, i + LW < pd ? 1.0f : -1.0f);
+                gather_add_quad<MT, XT>(acc, xq, w2, i + 2 * LW < pd ? 1.0f : -1.0f);
+                gather_add_quad<MT, XT>(acc, xq, w3, i + 3 * LW < pd ? 1.0f : -1.0f);
             }
+            if (i + LW < tot) {
+                const uint32_t w0 = run[i], w1 = run[i + LW];
+                gather_add_quad<MT, XT>(acc, xq, w0, i < pd ? 1.0f : -1.0f);
+                gather_add_quad<MT, XT>(acc, xq, w1, i + LW < pd ? 1.0f : -1.0f);
+                i += 2 * LW;
+            }
+            if (i < tot) gather_add_quad<MT, XT>(acc, xq, run[i], i < pd ? 1.0f : -1.0f);
         }
     }
     // fold the LPC partial sums of each (column, row quad) through LDS
@@ -607,7 +594,7 @@ __global__ __launch_bounds__(kBlockThreads) void tl_spmm_quad(KernelArgs a)
     float4* red = reinterpret_cast<float4*>(lds);
     red[tid] = make_float4(acc[0], acc[1], acc[2], acc[3]);
     __syncthreads();
-    const int per_group = cols * Q;  // threads of one lane group
+    constexpr int per_group = TL_BLOCK_COLUMNS * Q;  // threads of one lane group
     if (tid < per_group) {
         float4 sum = red[tid];
 #pragma unroll 4
@@ -615,8 +602,8 @@ __global__ __launch_bounds__(kBlockThreads) void tl_spmm_quad(KernelArgs a)
             const float4 o = red[l * per_group + tid];
             sum.x += o.x; sum.y += o.y; sum.z += o.z; sum.w += o.w;
         }
-        const int n = (nb0 + blk) * TL_BLOCK_COLUMNS + c16;
-        if (blk < bs && n < a.N) {
+        const int n = nb * TL_BLOCK_COLUMNS + c16;
+        if (n < a.N) {
             const float sc = load_scale(a.w0.scale, a.scale_f16, n);
             const float out[4] = {sum.x, sum.y, sum.z, sum.w};
 #pragma unroll
@@ -1365,9 +1352,9 @@ inline int rows_mtile(int x_dtype) { return x_dtype == TL_F16 ? 256 : 128; }
 // Tuning knobs (environment variables of the same names).  They are read once, at the first launch of the
 // process; tl_reload_options() reads them again.  A knob that is not set leaves the launcher's own choice.
 enum Knob { TL_SMALL_LDS, TL_TILE_GROUP, TL_QUAD_SHARE, TL_LW, TL_SPMV_SHARE, TL_SPMV_WIDE, TL_SMALL_MT, TL_SPMV_DIRECT,
-            TL_BLOCK_SET, TL_ROWS_SPLIT, TL_QUAD_BLOCKS, kKnobCount };
+            TL_BLOCK_SET, TL_ROWS_SPLIT, kKnobCount };
 const char* const kKnobNames[kKnobCount] = {"TL_SMALL_LDS", "TL_TILE_GROUP", "TL_QUAD_SHARE", "TL_LW", "TL_SPMV_SHARE", "TL_SPMV_WIDE",
-                                            "TL_SMALL_MT", "TL_SPMV_DIRECT", "TL_BLOCK_SET", "TL_ROWS_SPLIT", "TL_QUAD_BLOCKS"};
+                                            "TL_SMALL_MT", "TL_SPMV_DIRECT", "TL_BLOCK_SET", "TL_ROWS_SPLIT"};
 struct Knobs {
     bool set[kKnobCount];
     int value[kKnobCount];
@@ -1463,7 +1450,6 @@ inline int64_t small_kmajor_bytes(const tl_layout_header* h, int64_t M, int x_dt
 
 // LDS one workgroup of the small-M kernel may use: two workgroups fit a compute unit's 160 KB; a launch
 // with no more workgroups than compute units lets each have (nearly) all of it.
-constexpr int kQuadFill = 2;  // workgroups per compute unit below which tl_spmm_quad does not widen its block set
 constexpr int kSmallLdsShared = 78 * 1024;
 constexpr int kSmallLdsAlone = 158 * 1024;
 
@@ -1514,29 +1500,19 @@ template <int MT, bool XF16>
 int launch_quad_kernel(KernelArgs a, const tl_layout_header* h, hipStream_t st)
 {
     constexpr int es = XF16 ? 2 : 4;
+    constexpr int groups = kBlockThreads / (TL_BLOCK_COLUMNS * (MT / 4));  // lane groups per column
     const int tile_bytes = kTileSlots * MT * es;
     const int chunk_bytes = (int)h->max_chunk_dwords * 4;
-    const unsigned gy = (unsigned)ceil_div(a.M, MT);
-    // Column blocks per workgroup: every workgroup stages the whole activation image of its tiles (8 or 16 KB
-    // a tile against about 1 KB of chunks a block), so blocks that share a workgroup share that work; but the
-    // compute units want at least kQuadFill workgroups each to hide one another's waits.
-    int set = 1;
-    while (set < 4 && ceil_div(a.NB, set * 2) * gy >= (int64_t)kQuadFill * compute_units()) set *= 2;
-    set = knob(TL_QUAD_BLOCKS, set);
-    if (set != 1 && set != 2 && set != 4) return fail(TL_ERR_ARG, "TL_QUAD_BLOCKS=%d (1, 2 or 4 expected)", set);
-    a.block_set = set;
-    const int groups = kBlockThreads / (TL_BLOCK_COLUMNS * set * (MT / 4));  // lane groups per column
-    const unsigned gx = (unsigned)ceil_div(a.NB, set);
+    const unsigned gx = (unsigned)a.NB, gy = (unsigned)ceil_div(a.M, MT);
     const int share = std::max(1, std::min(knob(TL_QUAD_SHARE, 4), (int)ceil_div((int64_t)gx * gy, compute_units())));
     const int budget = 160 * 1024 / share - 1024;
-    const int per_tile = tile_bytes + set * chunk_bytes;
-    int tg = std::max(1, std::min(a.T, (budget - 256) / (2 * per_tile)));
+    int tg = std::max(1, std::min(a.T, (budget - 256) / (2 * (tile_bytes + chunk_bytes))));
     tg = std::max(1, std::min(tg, knob(TL_TILE_GROUP, tg)));
     tg = (int)ceil_div(a.T, ceil_div(a.T, tg));  // same number of groups, evened out
     a.tiles_per_group = tg;
     a.xs_bytes = tg * tile_bytes;
-    a.buf_bytes = set * (int)round_up((int64_t)tg * chunk_bytes, 16);
-    const size_t lds = std::max<size_t>(2 * ((size_t)a.xs_bytes + a.buf_bytes) + 2 * (size_t)set * (tg + 1) * 4, (size_t)kBlockThreads * 16);
+    a.buf_bytes = (int)round_up((int64_t)tg * chunk_bytes, 16);
+    const size_t lds = std::max<size_t>(2 * ((size_t)a.xs_bytes + a.buf_bytes) + 2 * (size_t)(tg + 1) * 4, (size_t)kBlockThreads * 16);
     if (lds > 160 * 1024) return fail(TL_ERR_UNSUPPORTED, "two tiles of %d rows need %zu bytes of LDS", MT, lds);
     // lane groups per run: a run's dwords go round the LW groups, four per group and turn; no more
     // tiles side by side than a group of tiles has
