@@ -915,68 +915,65 @@ struct RunFetcher {
 
 // The inner loop of the row-parallel kernel, written out in assembly.
 //
-// A slot of the staged tile is 512 bytes for both activation types (256 fp16 rows / 128 fp32 rows).
-// Its two halves are fetched with LDS "add-TID" reads: address = M0 + offset + 4 * lane, with
-// M0 = slot * 512 set on the scalar unit, so no vector instruction is spent on addressing.  Lane l thus holds, for fp16, rows {2l, 2l+1} and {128+2l, 129+2l} of the row tile;
-// for fp32, rows l and 64+l.  Per dword of four indices: one v_readlane (the dword sits in a lane of
-// the chunk vector), scalar byte extraction, eight LDS reads, and 16 (fp16) or 8 (fp32) accumulating
-// vector ops.  Two register sets alternate so that the reads of dword i + 1 are in flight while
-// dword i is accumulated; LDS reads complete in issue order, so "lgkmcnt(8)" means everything but
-// the eight reads issued last has arrived.
-// The tile starts at LDS address 0 (the kernel has no other LDS; the launcher checks it), so
-// M0 = slot * 512 = the index byte moved to bits 9..16: one shift and one mask per index.  The scalar
-// op that prepares the next index sits between each write of M0 and the reads that use it (one wait
-// state is required there); the last gap is filled by the loop counter's increment.
-#define TL_ISSUE(W, X0, Y0, X1, Y1, X2, Y2, X3, Y3)                 \
-    "s_lshl_b32 %[t], " W ", 9\n\t"                                  \
-    "s_and_b32 m0, %[t], %[mk]\n\t"                                  \
-    "s_lshl_b32 %[t], " W ", 1\n\t"                                  \
-    "ds_read_addtid_b32 " X0 " offset:0\n\t"                         \
-    "ds_read_addtid_b32 " Y0 " offset:256\n\t"                       \
-    "s_and_b32 m0, %[t], %[mk]\n\t"                                  \
-    "s_lshr_b32 %[t], " W ", 7\n\t"                                  \
-    "ds_read_addtid_b32 " X1 " offset:0\n\t"                         \
-    "ds_read_addtid_b32 " Y1 " offset:256\n\t"                       \
-    "s_and_b32 m0, %[t], %[mk]\n\t"                                  \
-    "s_lshr_b32 %[t], " W ", 15\n\t"                                 \
-    "ds_read_addtid_b32 " X2 " offset:0\n\t"                         \
-    "ds_read_addtid_b32 " Y2 " offset:256\n\t"                       \
-    "s_and_b32 m0, %[t], %[mk]\n\t"                                  \
+// A slot of the staged tile is 512 bytes for both activation types (256 fp16 rows / 128 fp32 rows), and a lane
+// reads its 8 bytes of a slot with one ds_read_b64: rows 4l .. 4l + 3 (fp16) or 2l, 2l + 1 (fp32) of the row
+// tile.  An 8-byte read moves twice the bytes of a 4-byte one in nearly the same LDS time (1.47 against
+// 1.31 ns per wave instruction and compute unit, measured), which is what makes the vector ALU and not the
+// LDS the unit this loop keeps busy.  Per dword of four indices: one v_readlane (the dword sits in a lane of
+// the chunk vector), four scalar byte extractions, four v_lshl_or (address = slot * 512 | 8 * lane, written
+// into the low register of the pair the read then fills), four LDS reads, and 16 (fp16) or 8 (fp32)
+// accumulating vector ops.  Two register sets alternate so that the reads of dword i + 1 are in flight while
+// dword i is accumulated; LDS reads complete in issue order, so "lgkmcnt(4)" means everything but the four
+// reads issued last has arrived.
+// The register pairs are named outright (the halves of a 64-bit asm operand cannot be named), and listed as
+// clobbered so that the compiler keeps them free around the loop.
+#define TL_RUN_CLOBBERS "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123", "v124", "v125", "v126", "v127"
+
+#define TL_ISSUE(L0, H0, L1, H1, L2, H2, L3, H3)                     \
+    "s_bfe_u32 %[t], %[w], 0x80000\n\t"                              \
+    "s_bfe_u32 %[u], %[w], 0x80008\n\t"                              \
+    "v_lshl_or_b32 v" L0 ", %[t], 9, %[l8]\n\t"                      \
+    "s_bfe_u32 %[t], %[w], 0x80010\n\t"                              \
+    "v_lshl_or_b32 v" L1 ", %[u], 9, %[l8]\n\t"                      \
+    "s_lshr_b32 %[u], %[w], 24\n\t"                                  \
+    "ds_read_b64 v[" L0 ":" H0 "], v" L0 "\n\t"                      \
+    "v_lshl_or_b32 v" L2 ", %[t], 9, %[l8]\n\t"                      \
+    "ds_read_b64 v[" L1 ":" H1 "], v" L1 "\n\t"                      \
+    "v_lshl_or_b32 v" L3 ", %[u], 9, %[l8]\n\t"                      \
     "s_add_u32 %[i], %[i], 1\n\t"                                    \
-    "ds_read_addtid_b32 " X3 " offset:0\n\t"                         \
-    "ds_read_addtid_b32 " Y3 " offset:256\n\t"
+    "ds_read_b64 v[" L2 ":" H2 "], v" L2 "\n\t"                      \
+    "ds_read_b64 v[" L3 ":" H3 "], v" L3 "\n\t"
 
 // fp16: a dword holds two rows; the mixed-precision fma converts and accumulates in one op
-#define TL_FMA_H(X, Y)                                                                   \
-    "v_fma_mix_f32 %[c0], " X ", %[sg], %[c0] op_sel_hi:[1,0,0]\n\t"                      \
-    "v_fma_mix_f32 %[c1], " X ", %[sg], %[c1] op_sel:[1,0,0] op_sel_hi:[1,0,0]\n\t"       \
-    "v_fma_mix_f32 %[c2], " Y ", %[sg], %[c2] op_sel_hi:[1,0,0]\n\t"                      \
-    "v_fma_mix_f32 %[c3], " Y ", %[sg], %[c3] op_sel:[1,0,0] op_sel_hi:[1,0,0]\n\t"
-#define TL_FMA_F(X, Y)                              \
-    "v_fma_f32 %[c0], " X ", %[sg], %[c0]\n\t"       \
-    "v_fma_f32 %[c1], " Y ", %[sg], %[c1]\n\t"
+#define TL_FMA_H(L, H)                                                                      \
+    "v_fma_mix_f32 %[c0], v" L ", %[sg], %[c0] op_sel_hi:[1,0,0]\n\t"                        \
+    "v_fma_mix_f32 %[c1], v" L ", %[sg], %[c1] op_sel:[1,0,0] op_sel_hi:[1,0,0]\n\t"         \
+    "v_fma_mix_f32 %[c2], v" H ", %[sg], %[c2] op_sel_hi:[1,0,0]\n\t"                        \
+    "v_fma_mix_f32 %[c3], v" H ", %[sg], %[c3] op_sel:[1,0,0] op_sel_hi:[1,0,0]\n\t"
+#define TL_FMA_F(L, H)                                  \
+    "v_fma_f32 %[c0], v" L ", %[sg], %[c0]\n\t"          \
+    "v_fma_f32 %[c1], v" H ", %[sg], %[c1]\n\t"
 
-#define TL_SET_A "%[a0]", "%[b0]", "%[a1]", "%[b1]", "%[a2]", "%[b2]", "%[a3]", "%[b3]"
-#define TL_SET_B "%[p0]", "%[q0]", "%[p1]", "%[q1]", "%[p2]", "%[q2]", "%[p3]", "%[q3]"
-#define TL_ISSUE_SET(W, ...) TL_ISSUE(W, __VA_ARGS__)
-#define TL_ACC_A(F) F("%[a0]", "%[b0]") F("%[a1]", "%[b1]") F("%[a2]", "%[b2]") F("%[a3]", "%[b3]")
-#define TL_ACC_B(F) F("%[p0]", "%[q0]") F("%[p1]", "%[q1]") F("%[p2]", "%[q2]") F("%[p3]", "%[q3]")
+#define TL_ISSUE_A TL_ISSUE("112", "113", "114", "115", "116", "117", "118", "119")
+#define TL_ISSUE_B TL_ISSUE("120", "121", "122", "123", "124", "125", "126", "127")
+#define TL_ACC_A(F) F("112", "113") F("114", "115") F("116", "117") F("118", "119")
+#define TL_ACC_B(F) F("120", "121") F("122", "123") F("124", "125") F("126", "127")
 
 #define TL_RUN_LOOP(F)                                   \
     "v_readlane_b32 %[w], %[v], %[i]\n\t"                \
-    TL_ISSUE_SET("%[w]", TL_SET_A)                       \
+    TL_ISSUE_A                                           \
     "Ltl_loop%=:\n\t"                                    \
     "s_cmp_lt_u32 %[i], %[hi]\n\t"                       \
     "s_cbranch_scc0 Ltl_lastA%=\n\t"                     \
     "v_readlane_b32 %[w], %[v], %[i]\n\t"                \
-    TL_ISSUE_SET("%[w]", TL_SET_B)                       \
-    "s_waitcnt lgkmcnt(8)\n\t"                           \
+    TL_ISSUE_B                                           \
+    "s_waitcnt lgkmcnt(4)\n\t"                           \
     TL_ACC_A(F)                                          \
     "s_cmp_lt_u32 %[i], %[hi]\n\t"                       \
     "s_cbranch_scc0 Ltl_lastB%=\n\t"                     \
     "v_readlane_b32 %[w], %[v], %[i]\n\t"                \
-    TL_ISSUE_SET("%[w]", TL_SET_A)                       \
-    "s_waitcnt lgkmcnt(8)\n\t"                           \
+    TL_ISSUE_A                                           \
+    "s_waitcnt lgkmcnt(4)\n\t"                           \
     TL_ACC_B(F)                                          \
     "s_branch Ltl_loop%=\n\t"                            \
     "Ltl_lastA%=:\n\t"                                   \
@@ -989,54 +986,77 @@ struct RunFetcher {
     "Ltl_end%=:"
 
 // The dwords [lo, hi) of the chunk vector `v` (dword i sits in lane i), all of one column and one
-// sign: acc += sgn * (rows of the tile at each index).  lo < hi.
+// sign: acc += sgn * (rows of the tile at each index).  lo < hi.  lane8 = 8 * lane.
 template <typename XT, int R>
-__device__ __forceinline__ void rows_run(float (&acc)[R], uint32_t v, int lo, int hi, float sgn_one)
+__device__ __forceinline__ void rows_run(float (&acc)[R], uint32_t v, int lo, int hi, float sgn_one, uint32_t lane8)
 {
-    uint32_t a0, b0, a1, b1, a2, b2, a3, b3, p0, q0, p1, q1, p2, q2, p3, q3, w, t;
+    uint32_t w, t, u;
     uint32_t i = (uint32_t)lo;
     if constexpr (sizeof(XT) == 2) {
         static_assert(R == 4, "fp16 row tiles hold 4 rows per lane");
         asm volatile(TL_RUN_LOOP(TL_FMA_H)
                      : [c0] "+v"(acc[0]), [c1] "+v"(acc[1]), [c2] "+v"(acc[2]), [c3] "+v"(acc[3]), [i] "+s"(i),
-                       [a0] "=&v"(a0), [b0] "=&v"(b0), [a1] "=&v"(a1), [b1] "=&v"(b1), [a2] "=&v"(a2), [b2] "=&v"(b2),
-                       [a3] "=&v"(a3), [b3] "=&v"(b3), [p0] "=&v"(p0), [q0] "=&v"(q0), [p1] "=&v"(p1), [q1] "=&v"(q1),
-                       [p2] "=&v"(p2), [q2] "=&v"(q2), [p3] "=&v"(p3), [q3] "=&v"(q3), [w] "=&s"(w), [t] "=&s"(t)
-                     : [v] "v"(v), [hi] "s"((uint32_t)hi), [mk] "s"(0x1fe00u), [sg] "s"(sgn_one)
-                     : "m0", "scc", "memory");
+                       [w] "=&s"(w), [t] "=&s"(t), [u] "=&s"(u)
+                     : [v] "v"(v), [hi] "s"((uint32_t)hi), [sg] "s"(sgn_one), [l8] "v"(lane8)
+                     : TL_RUN_CLOBBERS, "scc", "memory");
     } else {
         static_assert(R == 2, "fp32 row tiles hold 2 rows per lane");
         asm volatile(TL_RUN_LOOP(TL_FMA_F)
-                     : [c0] "+v"(acc[0]), [c1] "+v"(acc[1]), [i] "+s"(i),
-                       [a0] "=&v"(a0), [b0] "=&v"(b0), [a1] "=&v"(a1), [b1] "=&v"(b1), [a2] "=&v"(a2), [b2] "=&v"(b2),
-                       [a3] "=&v"(a3), [b3] "=&v"(b3), [p0] "=&v"(p0), [q0] "=&v"(q0), [p1] "=&v"(p1), [q1] "=&v"(q1),
-                       [p2] "=&v"(p2), [q2] "=&v"(q2), [p3] "=&v"(p3), [q3] "=&v"(q3), [w] "=&s"(w), [t] "=&s"(t)
-                     : [v] "v"(v), [hi] "s"((uint32_t)hi), [mk] "s"(0x1fe00u), [sg] "s"(sgn_one)
-                     : "m0", "scc", "memory");
+                     : [c0] "+v"(acc[0]), [c1] "+v"(acc[1]), [i] "+s"(i), [w] "=&s"(w), [t] "=&s"(t), [u] "=&s"(u)
+                     : [v] "v"(v), [hi] "s"((uint32_t)hi), [sg] "s"(sgn_one), [l8] "v"(lane8)
+                     : TL_RUN_CLOBBERS, "scc", "memory");
     }
+}
+
+// Wave priority for run `r` of the `total` runs a wave works through per tile.  The issue arbiter serves the
+// oldest wave of a SIMD first, so left alone the four waves of a SIMD drift far apart inside a tile and the
+// early ones idle at the tile's barrier (a quarter of the kernel's time, measured).  Priority that falls with
+// progress holds back the waves that are ahead; the steps shrink towards the end of the tile, because what the
+// waves differ by when they arrive is at most the last step.
+template <int r, int total>
+__device__ __forceinline__ void progress_priority()
+{
+    if constexpr (r * 16 < 7 * total) __builtin_amdgcn_s_setprio(3);
+    else if constexpr (r * 16 < 12 * total) __builtin_amdgcn_s_setprio(2);
+    else if constexpr (r * 16 < 15 * total) __builtin_amdgcn_s_setprio(1);
+    else __builtin_amdgcn_s_setprio(0);
+}
+
+// Column c (of C, counted from compile-time index) of one 64-dword chunk of the wave's piece.
+template <typename XT, int R, int C, int RUN0, int RUNS, int c>
+__device__ __forceinline__ void rows_chunk_column(float (&acc)[C][R], const int (&pb)[C], const int (&pe)[C], const int (&ne)[C],
+                                                  uint32_t v, int cb, float one, uint32_t lane8)
+{
+    int lo = max(pb[c], cb) - cb, hi = min(pe[c], cb + 64) - cb;
+    if (lo < hi) {
+        progress_priority<RUN0 + 2 * c, RUNS>();
+        rows_run<XT, R>(acc[c], v, lo, hi, one, lane8);
+    }
+    lo = max(pe[c], cb) - cb;
+    hi = min(ne[c], cb + 64) - cb;
+    if (lo < hi) {
+        progress_priority<RUN0 + 2 * c + 1, RUNS>();
+        rows_run<XT, R>(acc[c], v, lo, hi, -one, lane8);
+    }
+    if constexpr (c + 1 < C) rows_chunk_column<XT, R, C, RUN0, RUNS, c + 1>(acc, pb, pe, ne, v, cb, one, lane8);
 }
 
 // One 64-dword chunk of the wave's piece: dword i of the piece sits in lane i - cb of `v`
-// and is broadcast from there, so its four row indices are wave-uniform.
-template <typename XT, int R, int C>
+// and is broadcast from there, so its four row indices are wave-uniform.  The wave's runs are numbered
+// RUN0 ... of RUNS per tile (two per column; the fused kernel walks two weights).
+template <typename XT, int R, int C, int RUN0, int RUNS>
 __device__ __forceinline__ void rows_chunk(float (&acc)[C][R], const int (&pb)[C], const int (&pe)[C], const int (&ne)[C],
-                                           uint32_t v, int cb, float one)
+                                           uint32_t v, int cb, float one, uint32_t lane8)
 {
-#pragma unroll
-    for (int c = 0; c < C; ++c) {
-        int lo = max(pb[c], cb) - cb, hi = min(pe[c], cb + 64) - cb;
-        if (lo < hi) rows_run<XT, R>(acc[c], v, lo, hi, one);
-        lo = max(pe[c], cb) - cb;
-        hi = min(ne[c], cb + 64) - cb;
-        if (lo < hi) rows_run<XT, R>(acc[c], v, lo, hi, -one);
-    }
+    rows_chunk_column<XT, R, C, RUN0, RUNS, 0>(acc, pb, pe, ne, v, cb, one, lane8);
 }
 
-template <typename XT, int R, int C>
+template <typename XT, int R, int C, int RUN0, int RUNS>
 __device__ __forceinline__ void rows_consume(float (&acc)[C][R], const WaveRuns<C>& r, const uint32_t* __restrict__ idx,
                                              int lane, float one)
 {
     int pb[C], pe[C], ne[C];
+    const uint32_t lane8 = (uint32_t)lane * 8u;
 #pragma unroll
     for (int c = 0; c < C; ++c) {
         pb[c] = (int)((r.d[c] >> 16) - (r.d[0] >> 16));
@@ -1046,9 +1066,9 @@ __device__ __forceinline__ void rows_consume(float (&acc)[C][R], const WaveRuns<
     const int total = ne[C - 1];
 #pragma unroll
     for (int ch = 0; ch < NPRE; ++ch)
-        if (ch * 64 < total) rows_chunk<XT, R, C>(acc, pb, pe, ne, r.pre[ch], ch * 64, one);
+        if (ch * 64 < total) rows_chunk<XT, R, C, RUN0, RUNS>(acc, pb, pe, ne, r.pre[ch], ch * 64, one, lane8);
     for (int cb = NPRE * 64; cb < total; cb += 64)  // pieces longer than the prefetch window: fetched on demand
-        rows_chunk<XT, R, C>(acc, pb, pe, ne, idx[r.base + cb + lane], cb, one);
+        rows_chunk<XT, R, C, RUN0, RUNS>(acc, pb, pe, ne, idx[r.base + cb + lane], cb, one, lane8);
 }
 
 // Staging of one activation tile: global -> registers (issued a tile ahead), registers -> LDS.
@@ -1087,7 +1107,7 @@ __device__ __forceinline__ void regs_to_lds(const u32x4 (&pf)[PER], unsigned cha
 }
 
 // Scale, optional SiLU gate, and store of one workgroup's output tile.  Row of accumulator j of a lane:
-// fp16: rows {2l, 2l + 1} and {128 + 2l, 129 + 2l} of the row tile; fp32: rows l and 64 + l.
+// row R * l + j of the row tile.
 // A lane holds C neighbouring columns of R scattered rows, so storing from the accumulators would write
 // 2- or 4-byte pieces a row apart.  The tile therefore goes through LDS (the activation tile's space,
 // free by now): lanes write their C columns of a row side by side, then the workgroup stores whole
@@ -1126,7 +1146,7 @@ __device__ __forceinline__ void rows_store(const KernelArgs& a, int m0, int n_wg
             if (n >= a.N) continue;
 #pragma unroll
             for (int j = 0; j < R; ++j) {
-                const int m = m0 + (sizeof(XT) == 2 ? (j >> 1) * 128 + 2 * lane + (j & 1) : j * 64 + lane);
+                const int m = m0 + R * lane + j;
                 if (m < a.M) store_out(a.Y, a.y_f16, (long long)m * a.ldy + n, v[c][j]);
             }
         }
@@ -1135,7 +1155,7 @@ __device__ __forceinline__ void rows_store(const KernelArgs& a, int m0, int n_wg
     __syncthreads();  // every wave is done reading the activation tile
 #pragma unroll
     for (int j = 0; j < R; ++j) {
-        const int r = sizeof(XT) == 2 ? (j >> 1) * 128 + 2 * lane + (j & 1) : j * 64 + lane;
+        const int r = R * lane + j;
 #pragma unroll
         for (int g = 0; g < C; g += 4) {
             unsigned char* dst = smem + (size_t)r * stride + (size_t)(wave * C + g) * es;
@@ -1262,8 +1282,9 @@ __global__ __launch_bounds__(WAVES * 64) void tl_spmm_rows(KernelArgs a)
             if (wave_live) {
                 f0.advance(t, a.T);
                 if constexpr (GATED) f1.advance(t, a.T);
-                rows_consume<XT, R, C>(acc, f0.cur, a.w0.stream, lane, a.one);
-                if constexpr (GATED) rows_consume<XT, R, C>(acc2, f1.cur, a.w1.stream, lane, a.one);
+                constexpr int RUNS = (GATED ? 4 : 2) * C;  // runs of a wave per tile
+                rows_consume<XT, R, C, 0, RUNS>(acc, f0.cur, a.w0.stream, lane, a.one);
+                if constexpr (GATED) rows_consume<XT, R, C, 2 * C, RUNS>(acc2, f1.cur, a.w1.stream, lane, a.one);
             }
         }
 
