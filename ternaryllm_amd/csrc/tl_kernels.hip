@@ -167,6 +167,57 @@ __device__ __forceinline__ void gather_add_quad(float (&acc)[4], const XT* __res
     }
 }
 
+// The quad gather in two steps, so that a lane has the reads of several indices in flight at once (left to
+// the compiler, every read is waited for before the next is issued, and a wave spends most of its time on LDS
+// latency).  The reads are issued from assembly, which the compiler neither reorders nor tracks; the results
+// may be used only after quad_wait<N> has named them, N being the number of reads issued after them.
+template <typename XT>
+struct QuadRead {
+    typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+    typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+    using type = typename std::conditional<sizeof(XT) == 2, u32x2_t, u32x4_t>::type;  // four rows of a slot
+};
+
+template <int MT, typename XT>
+__device__ __forceinline__ void quad_issue(typename QuadRead<XT>::type (&v)[4], const XT* __restrict__ xq, uint32_t word)
+{
+    using lds_ptr = const __attribute__((address_space(3))) void*;
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+        const uint32_t r = (word >> (8 * b)) & 0xffu;
+        const uint32_t addr = (uint32_t)reinterpret_cast<uintptr_t>((lds_ptr)(xq + r * MT));
+        if constexpr (sizeof(XT) == 2) asm volatile("ds_read_b64 %0, %1" : "=v"(v[b]) : "v"(addr) : "memory");
+        else asm volatile("ds_read_b128 %0, %1" : "=v"(v[b]) : "v"(addr) : "memory");
+    }
+}
+
+template <int N, typename V>
+__device__ __forceinline__ void quad_wait(V (&v)[4])
+{
+    static_assert(N == 0 || N == 4, "reads are issued four at a time");
+    if constexpr (N == 0) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]) : : "memory");
+    else asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]) : : "memory");
+}
+
+template <typename XT>
+__device__ __forceinline__ void quad_accumulate(float (&acc)[4], const typename QuadRead<XT>::type (&v)[4], float sign)
+{
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+        if constexpr (sizeof(XT) == 4) {
+            acc[0] = fmaf(__uint_as_float(v[b].x), sign, acc[0]);
+            acc[1] = fmaf(__uint_as_float(v[b].y), sign, acc[1]);
+            acc[2] = fmaf(__uint_as_float(v[b].z), sign, acc[2]);
+            acc[3] = fmaf(__uint_as_float(v[b].w), sign, acc[3]);
+        } else {
+            acc[0] = fmaf(__half2float(__ushort_as_half((unsigned short)(v[b].x & 0xffffu))), sign, acc[0]);
+            acc[1] = fmaf(__half2float(__ushort_as_half((unsigned short)(v[b].x >> 16))), sign, acc[1]);
+            acc[2] = fmaf(__half2float(__ushort_as_half((unsigned short)(v[b].y & 0xffffu))), sign, acc[2]);
+            acc[3] = fmaf(__half2float(__ushort_as_half((unsigned short)(v[b].y >> 16))), sign, acc[3]);
+        }
+    }
+}
+
 constexpr int kBlockThreads = 512;            // workgroup of the small-M kernel
 // Staging of the activations by the small-M kernel:
 constexpr int kStageElements = 0;     // a thread owns slots and reads their MT values one by one (any layout)
@@ -572,21 +623,24 @@ __global__ __launch_bounds__(kBlockThreads) void tl_spmm_quad(KernelArgs a)
             const uint32_t* run = chunk + (d >> 16);
             const int pd = run_pos_dwords(d), tot = pd + run_neg_dwords(d);
             const XT* xq = reinterpret_cast<const XT*>(xs) + (size_t)tl * kTileSlots * MT + q * 4;
+            // two dwords a turn: the eight reads are in flight together, and those of the second dword land
+            // while the first is accumulated
+            typename QuadRead<XT>::type va[4], vb[4];
             int i = lw;
-            for (; i + 3 * LW < tot; i += 4 * LW) {
-                const uint32_t w0 = run[i], w1 = run[i + LW], w2 = run[i + 2 * LW], w3 = run[i + 3 * LW];
-                gather_add_quad<MT, XT>(acc, xq, w0, i < pd ? 1.0f : -1.0f);
-                gather_add_quad<MT, XT>(acc, xq, w1, i + LW < pd ? 1.0f : -1.0f);
-                gather_add_quad<MT, XT>(acc, xq, w2, i + 2 * LW < pd ? 1.0f : -1.0f);
-                gather_add_quad<MT, XT>(acc, xq, w3, i + 3 * LW < pd ? 1.0f : -1.0f);
-            }
-            if (i + LW < tot) {
+            for (; i + LW < tot; i += 2 * LW) {
                 const uint32_t w0 = run[i], w1 = run[i + LW];
-                gather_add_quad<MT, XT>(acc, xq, w0, i < pd ? 1.0f : -1.0f);
-                gather_add_quad<MT, XT>(acc, xq, w1, i + LW < pd ? 1.0f : -1.0f);
-                i += 2 * LW;
+                quad_issue<MT, XT>(va, xq, w0);
+                quad_issue<MT, XT>(vb, xq, w1);
+                quad_wait<4>(va);
+                quad_accumulate<XT>(acc, va, i < pd ? 1.0f : -1.0f);
+                quad_wait<0>(vb);
+                quad_accumulate<XT>(acc, vb, i + LW < pd ? 1.0f : -1.0f);
             }
-            if (i < tot) gather_add_quad<MT, XT>(acc, xq, run[i], i < pd ? 1.0f : -1.0f);
+            if (i < tot) {
+                quad_issue<MT, XT>(va, xq, run[i]);
+                quad_wait<0>(va);
+                quad_accumulate<XT>(acc, va, i < pd ? 1.0f : -1.0f);
+            }
         }
     }
     // fold the LPC partial sums of each (column, row quad) through LDS
