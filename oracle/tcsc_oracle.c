@@ -14,7 +14,10 @@
  *                         brute force on tiny W, round trip to dense.
  *   orc_tiled_csc      -- closed form (row % TILE_K, exclusive cumsum of the
  *                         per-(column, tile) counts), invariants, round trip.
- *   orc_tiled_mcsc     -- three hand-worked tiles, the p == n / even case that
+ *   orc_tiled_mcsc     -- six hand-worked cases (tests/golden/mcsc_hand_cases.json:
+ *                         odd pair counts on either side, padding with
+ *                         overwrite, the cursor overwrite across two tiles,
+ *                         padded arrays), the p == n / even case that
  *                         reduces to a plain interleave of orc_tiled_csc, the
  *                         alignment invariants of the offsets.  The reference
  *                         holds no fixture for it and its only other
@@ -30,8 +33,13 @@
  *                         one +-1 per column, all-ones column.
  *   orc_mcsc_product   -- what the reference kernels' loop structure sums from
  *                         merged arrays (with the tile offset applied to every
- *                         gather); checked against orc_dense_product on inputs
- *                         where the merged format is lossless.
+ *                         gather; without the same-sign part when `uniformed`).
+ *                         Pinned by the six hand cases: the terms of each sum
+ *                         are written out by hand in the fixture, for an x
+ *                         whose values (3^(k mod 11) + k) let no dropped term,
+ *                         wrong sign or missing tile offset go unnoticed, and
+ *                         the sums are asserted; also equals orc_dense_product
+ *                         on inputs where the merged format is lossless.
  */
 #include <stdint.h>
 #include <stdlib.h>
