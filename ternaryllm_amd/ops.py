@@ -81,9 +81,16 @@ def _x_geometry(x, K, x_layout):
 _workspaces = {}
 
 
+def release_workspaces():
+    """Drops every cached scratch buffer (one per (device, stream) that has run a product needing one; torch
+    reuses the memory in stream order).  Not while a captured HIP graph that contains such a product is still
+    to be replayed: the graph holds the buffer's address."""
+    _workspaces.clear()
+
+
 def _workspace(header, M, x_code, x_layout, device):
     """Scratch for one call: one buffer per (device, stream), kept and only replaced by a larger one
-    (work on one stream is ordered, so consecutive calls may share it)."""
+    (work on one stream is ordered, so consecutive calls may share it); release_workspaces() drops them."""
     need = ctypes.c_int64(0)
     _lib.check(_lib.lib().tl_spmm_workspace(ctypes.byref(header), M, x_code, x_layout, ctypes.byref(need)))
     if need.value == 0:
