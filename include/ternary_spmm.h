@@ -296,6 +296,19 @@ int tl_decode_attention(const void* q, const void* k_cache, const void* v_cache,
                         int64_t batch, int heads, int head_dim, int64_t max_seq,
                         const int64_t* pos_dev, void* out, int64_t out_kmajor_ld, void* stream);
 
+/* tl_decode_attention with the cache rows of every (batch row, head) shared out among `splits` workgroups
+ * (1 to 8), for steps with fewer (batch row, head) pairs than the GPU has compute units: one compute unit
+ * streams a head's cache rows at a fraction of what the chip can.  Each workgroup leaves a piece in
+ * `workspace`: fp32 [batch * heads][splits][head_dim + 4] -- head_dim unnormalised sums, then the piece's
+ * maximum and its sum of exponentials (16-byte aligned; TL_ERR_SIZE when the workspace is smaller) -- and a
+ * second small launch folds the pieces into `out`.  With out == NULL that launch is left out and the pieces
+ * are the result (any splits >= 1): tl_spmv_attn_combine folds them inside the output projection.
+ * splits == 1 with an `out` is tl_decode_attention (the workspace is not touched).  Same reference lines. */
+int tl_decode_attention_split(const void* q, const void* k_cache, const void* v_cache, int dtype,
+                              int64_t batch, int heads, int head_dim, int64_t max_seq,
+                              const int64_t* pos_dev, void* out, int64_t out_kmajor_ld,
+                              int splits, void* workspace, int64_t workspace_bytes, void* stream);
+
 /* Y[N] = (x * W) * scale for ONE activation row x that the call produces itself, so that a decode step
  * needs neither a launch nor a trip through memory for the producer (the reference leaves these steps to
  * separate torch operators, TernaryLLM/TernaryMLP.py:34 and the Hugging Face decoder layer it patches):
@@ -310,6 +323,17 @@ int tl_decode_attention(const void* q, const void* k_cache, const void* v_cache,
 int tl_spmv_fused(const tl_layout_header* header, const void* blob_dev, int producer,
                   const void* in, const void* in2, const void* norm_weight, float eps, void* sum_out, int x_dtype,
                   void* Y, int y_dtype, const void* scale, int scale_dtype, void* stream);
+
+/* Y[N] = (x * W) * scale for the single row x = the attention output that the pieces of
+ * tl_decode_attention_split (out == NULL) add up to, batch 1: the output projection of a decode step
+ * (o_proj over the eager softmax(QK^T)V, TernaryLLM/TernaryAttn.py:100-116) without a launch for the fold.
+ *   pieces    device fp32 [K / head_dim][splits][head_dim + 4], 16-byte aligned
+ *   x_dtype   the type x is rounded to before the product (the type a separate fold would write)
+ * Needs a blob whose tile height and K are whole 16-byte pieces of x_dtype (else TL_ERR_UNSUPPORTED) and
+ * head_dim a multiple of 16 bytes of it that divides K. */
+int tl_spmv_attn_combine(const tl_layout_header* header, const void* blob_dev, const void* pieces,
+                         int splits, int head_dim, int x_dtype, void* Y, int y_dtype,
+                         const void* scale, int scale_dtype, void* stream);
 
 /* x_out = x + y, h_out = RMSNorm(x_out) * weight, row by row ([rows][width], one dtype): the residual
  * add of a decoder layer fused with the normalisation that follows (the reference leaves both to the

@@ -67,7 +67,7 @@ template <typename T, int HD>
 __global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restrict__ q, const T* __restrict__ k_cache,
                                                                const T* __restrict__ v_cache, const long long* __restrict__ pos_p,
                                                                T* __restrict__ out, long long out_kld, int heads, long long max_seq,
-                                                               float scale)
+                                                               float scale, int splits, float* __restrict__ pieces)
 {
     constexpr int VE = 16 / (int)sizeof(T);   // values per 16-byte piece
     constexpr int CPR = HD / VE;              // lanes per cache row
@@ -81,6 +81,14 @@ __global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restri
     long long n = *pos_p + 1;  // valid rows
     if (n > max_seq) n = max_seq;
     if (n < 1) n = 1;
+    // With splits > 1 the rows of a (batch row, head) are shared out in contiguous pieces among gridDim.y
+    // workgroups; each leaves its unnormalised sums, maximum and sum of exponentials for tl_attn_combine.
+    long long lo = 0;
+    if (splits > 1) {
+        const long long piece = (n + splits - 1) / splits;
+        lo = (long long)blockIdx.y * piece;
+        n = lo + piece < n ? lo + piece : n;  // may leave this workgroup no rows (lo >= n)
+    }
     const T* kc = k_cache + (size_t)bh * max_seq * HD;
     const T* vc = v_cache + (size_t)bh * max_seq * HD;
     const int c = tid % CPR, rg = tid / CPR;
@@ -110,7 +118,7 @@ __global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restri
     float acc[VE];
 #pragma unroll
     for (int e = 0; e < VE; ++e) acc[e] = 0.f;
-    for (long long j0 = rg; j0 < n; j0 += (long long)RG * NB) {
+    for (long long j0 = lo + rg; j0 < n; j0 += (long long)RG * NB) {
         uint4 kk[NB], vv[NB];
 #pragma unroll
         for (int u = 0; u < NB; ++u) {
@@ -168,10 +176,41 @@ __global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restri
             norm = fmaf(group_sum[g], wgt, norm);
             o = fmaf(partial[g][tid], wgt, o);
         }
+        if (pieces) {
+            float* mine = pieces + ((size_t)bh * splits + blockIdx.y) * (HD + 4);
+            mine[tid] = o;  // 0 when the workgroup had no rows (top = -inf, norm = 0)
+            if (tid == 0) {
+                mine[HD] = top;
+                mine[HD + 1] = norm;
+            }
+            return;
+        }
         const long long b = bh / heads;
         const size_t col = (size_t)(bh % heads) * HD + tid;  // of the [batch][heads * head_dim] output
         out[out_kld ? col * out_kld + b : (size_t)b * heads * HD + col] = from_f<T>(o / norm);
     }
+}
+
+// Folds the pieces that a split tl_decode_attn left: one workgroup of HD threads per (batch row, head).
+template <typename T, int HD>
+__global__ __launch_bounds__(HD) void tl_attn_combine(const float* __restrict__ partial, int splits, T* __restrict__ out,
+                                                      long long out_kld, int heads)
+{
+    const long long bh = blockIdx.x;
+    const int tid = threadIdx.x;
+    const float* mine = partial + (size_t)bh * splits * (HD + 4);
+    float top = -INFINITY;
+    for (int s = 0; s < splits; ++s) top = fmaxf(top, mine[(size_t)s * (HD + 4) + HD]);
+    float norm = 0.f, o = 0.f;
+    for (int s = 0; s < splits; ++s) {
+        const float* piece = mine + (size_t)s * (HD + 4);
+        const float wgt = piece[HD] == -INFINITY ? 0.f : __expf(piece[HD] - top);
+        norm = fmaf(piece[HD + 1], wgt, norm);
+        o = fmaf(piece[tid], wgt, o);
+    }
+    const long long b = bh / heads;
+    const size_t col = (size_t)(bh % heads) * HD + tid;
+    out[out_kld ? col * out_kld + b : (size_t)b * heads * HD + col] = from_f<T>(o / norm);
 }
 
 // x_out = x + y (rounded to T), h_out = x_out / rms(x_out) * weight: the residual add and the RMSNorm that
@@ -313,22 +352,26 @@ int launched()
 
 template <typename T, int HD>
 int attn_launch(dim3 grid, size_t lds, hipStream_t st, const void* q, const void* k, const void* v, const long long* pos, void* out,
-                long long out_kld, int heads, long long max_seq, float scale)
+                long long out_kld, int heads, long long max_seq, float scale, int splits, float* partial)
 {
     auto kernel = tl_decode_attn<T, HD>;
-    hipLaunchKernelGGL(kernel, grid, dim3(kAttnThreads), lds, st, static_cast<const T*>(q), static_cast<const T*>(k),
-                       static_cast<const T*>(v), pos, static_cast<T*>(out), out_kld, heads, max_seq, scale);
+    hipLaunchKernelGGL(kernel, dim3(grid.x, (unsigned)splits), dim3(kAttnThreads), lds, st, static_cast<const T*>(q), static_cast<const T*>(k),
+                       static_cast<const T*>(v), pos, static_cast<T*>(out), out_kld, heads, max_seq, scale, splits, partial);
+    if (partial && out) {
+        auto combine = tl_attn_combine<T, HD>;
+        hipLaunchKernelGGL(combine, grid, dim3(HD), 0, st, partial, splits, static_cast<T*>(out), out_kld, heads);
+    }
     return TL_OK;
 }
 
 template <typename T>
 int attn_dispatch(int head_dim, dim3 grid, size_t lds, hipStream_t st, const void* q, const void* k, const void* v,
-                  const long long* pos, void* out, long long out_kld, int heads, long long max_seq, float scale)
+                  const long long* pos, void* out, long long out_kld, int heads, long long max_seq, float scale, int splits, float* partial)
 {
     switch (head_dim) {
-        case 64: return attn_launch<T, 64>(grid, lds, st, q, k, v, pos, out, out_kld, heads, max_seq, scale);
-        case 128: return attn_launch<T, 128>(grid, lds, st, q, k, v, pos, out, out_kld, heads, max_seq, scale);
-        case 256: return attn_launch<T, 256>(grid, lds, st, q, k, v, pos, out, out_kld, heads, max_seq, scale);
+        case 64: return attn_launch<T, 64>(grid, lds, st, q, k, v, pos, out, out_kld, heads, max_seq, scale, splits, partial);
+        case 128: return attn_launch<T, 128>(grid, lds, st, q, k, v, pos, out, out_kld, heads, max_seq, scale, splits, partial);
+        case 256: return attn_launch<T, 256>(grid, lds, st, q, k, v, pos, out, out_kld, heads, max_seq, scale, splits, partial);
         default: return fail(TL_ERR_UNSUPPORTED, "head_dim=%d (64, 128 or 256 supported)", head_dim);
     }
 }
@@ -358,25 +401,52 @@ extern "C" int tl_rope_cache_update(const void* qkv, int dtype, int64_t batch, i
     return launched();
 }
 
-extern "C" int tl_decode_attention(const void* q, const void* k_cache, const void* v_cache, int dtype, int64_t batch, int heads,
-                                   int head_dim, int64_t max_seq, const int64_t* pos_dev, void* out, int64_t out_kmajor_ld, void* stream)
+namespace {
+constexpr int kAttnMaxSplits = 8;
+
+int attention(const void* q, const void* k_cache, const void* v_cache, int dtype, int64_t batch, int heads, int head_dim, int64_t max_seq,
+              const int64_t* pos_dev, void* out, int64_t out_kmajor_ld, int splits, void* workspace, int64_t workspace_bytes, void* stream)
 {
     if (int rc = check_common(dtype, batch, heads, head_dim, max_seq, pos_dev)) return rc;
-    if (!q || !k_cache || !v_cache || !out) return fail(TL_ERR_ARG, "device pointer is null");
+    if (!q || !k_cache || !v_cache || (!out && !workspace)) return fail(TL_ERR_ARG, "device pointer is null");
     if (out_kmajor_ld && out_kmajor_ld < batch) return fail(TL_ERR_SHAPE, "out_kmajor_ld=%lld is less than the batch", (long long)out_kmajor_ld);
     const size_t lds = 0;
     if (reinterpret_cast<uintptr_t>(k_cache) % 16 || reinterpret_cast<uintptr_t>(v_cache) % 16 || reinterpret_cast<uintptr_t>(q) % 16)
         return fail(TL_ERR_ALIGN, "q and the caches must be 16-byte aligned");
+    if (splits < 1 || splits > kAttnMaxSplits) return fail(TL_ERR_ARG, "splits=%d (1 to %d expected)", splits, kAttnMaxSplits);
+    const bool leaves_pieces = splits > 1 || !out;
+    if (leaves_pieces) {
+        const int64_t need = batch * heads * splits * (int64_t)(head_dim + 4) * (int64_t)sizeof(float);
+        if (!workspace || workspace_bytes < need || reinterpret_cast<uintptr_t>(workspace) % 16)
+            return fail(TL_ERR_SIZE, "%d splits need a 16-byte aligned workspace of %lld bytes", splits, (long long)need);
+    }
     dim3 grid((unsigned)(batch * heads));
     hipStream_t st = static_cast<hipStream_t>(stream);
     const long long* pos = reinterpret_cast<const long long*>(pos_dev);
     const float scale = 1.0f / sqrtf((float)head_dim);
+    float* partial = leaves_pieces ? static_cast<float*>(workspace) : nullptr;
     int rc;
     if (dtype == TL_F16) rc = attn_dispatch<__half>(head_dim, grid, lds, st, q, k_cache, v_cache, pos, out, (long long)out_kmajor_ld, heads,
-                                                    (long long)max_seq, scale);
-    else rc = attn_dispatch<float>(head_dim, grid, lds, st, q, k_cache, v_cache, pos, out, (long long)out_kmajor_ld, heads, (long long)max_seq, scale);
+                                                    (long long)max_seq, scale, splits, partial);
+    else rc = attn_dispatch<float>(head_dim, grid, lds, st, q, k_cache, v_cache, pos, out, (long long)out_kmajor_ld, heads, (long long)max_seq,
+                                   scale, splits, partial);
     if (rc) return rc;
     return launched();
+}
+}  // namespace
+
+extern "C" int tl_decode_attention(const void* q, const void* k_cache, const void* v_cache, int dtype, int64_t batch, int heads,
+                                   int head_dim, int64_t max_seq, const int64_t* pos_dev, void* out, int64_t out_kmajor_ld, void* stream)
+{
+    return attention(q, k_cache, v_cache, dtype, batch, heads, head_dim, max_seq, pos_dev, out, out_kmajor_ld, 1, nullptr, 0, stream);
+}
+
+extern "C" int tl_decode_attention_split(const void* q, const void* k_cache, const void* v_cache, int dtype, int64_t batch, int heads,
+                                         int head_dim, int64_t max_seq, const int64_t* pos_dev, void* out, int64_t out_kmajor_ld,
+                                         int splits, void* workspace, int64_t workspace_bytes, void* stream)
+{
+    return attention(q, k_cache, v_cache, dtype, batch, heads, head_dim, max_seq, pos_dev, out, out_kmajor_ld, splits, workspace,
+                     workspace_bytes, stream);
 }
 
 extern "C" int tl_add_rmsnorm(const void* x, const void* y, const void* weight, int dtype, int64_t rows, int width, float eps,

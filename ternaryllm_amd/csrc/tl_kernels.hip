@@ -78,6 +78,8 @@ struct KernelArgs {
     const void* norm_w;   // RMSNorm weight [K]
     void* sum_out;        // where the first workgroup writes X + X2, or null
     float eps;
+    int pro_splits;       // attention-combine producer: pieces per head, and the head width
+    int pro_hd;
 };
 
 __device__ __forceinline__ float load_scale(const void* scale, int is_f16, int n)
@@ -683,9 +685,12 @@ __global__ __launch_bounds__(kBlockThreads) void tl_spmm_quad(KernelArgs a)
 //   kProSiluGate  x[k] = silu(in[k]) * in[K + k] for a side-by-side gate | up row `in` of 2K values;
 //   kProAddNorm   s = in + in2 (in2 may be null), x = s * rsqrt(mean(s^2) + eps) * norm_w; the first workgroup
 //                 also writes s to sum_out (the residual stream of a decoder layer).
-// Roundings are those of the separate kernels (tl_silu_mul, tl_add_rmsnorm): s, the SiLU and x are rounded to
-// the activation type.
-constexpr int kProNone = 0, kProSiluGate = 1, kProAddNorm = 2;
+//   kProAttnCombine  x = the attention output that tl_decode_attention_split's pieces add up to: per head h,
+//                 x[h * HD + d] = sum_s w_s * piece_s[d] with w_s = exp(top_s - top) / sum_s exp(top_s - top) * norm_s
+//                 (`in` = the pieces, fp32 [heads][splits][HD + 4]: HD sums, maximum, sum of exponentials).
+// Roundings are those of the separate kernels (tl_silu_mul, tl_add_rmsnorm, tl_attn_combine): s, the SiLU and x
+// are rounded to the activation type.
+constexpr int kProNone = 0, kProSiluGate = 1, kProAddNorm = 2, kProAttnCombine = 3;
 
 template <bool F16>
 __device__ __forceinline__ float round_to_x(float v)
@@ -715,6 +720,7 @@ __global__ __launch_bounds__(NT) void tl_spmv_direct(KernelArgs a)
     using global_ptr = const __attribute__((address_space(1))) void*;
     using lds_ptr = __attribute__((address_space(3))) void*;
     float inv_rms = 1.0f;  // kProAddNorm: rsqrt(mean(s^2) + eps), known before any tile is staged
+    const float* piece_w = nullptr;  // kProAttnCombine: [heads][splits] weights of the pieces, in LDS
 
     // the 16-byte piece of the row that starts at value k, as the producer makes it
     auto produce = [&](int k) -> u32x4 {
@@ -730,6 +736,26 @@ __global__ __launch_bounds__(NT) void tl_spmv_direct(KernelArgs a)
                 const float gf = (float)g[e];
                 o[e] = XT(round_to_x<XF16>(gf / (1.0f + __expf(-gf))) * (float)u[e]);
             }
+        } else if constexpr (PRO == kProAttnCombine) {
+            const int hd = a.pro_hd, sp = a.pro_splits;
+            const int h = k / hd, d = k - h * hd;  // a piece of VE values never straddles heads (HD is a multiple of VE)
+            const float* src = static_cast<const float*>(a.X) + (size_t)h * sp * (hd + 4) + d;
+            float f[VE];
+#pragma unroll
+            for (int e = 0; e < VE; ++e) f[e] = 0.f;
+            for (int sidx = 0; sidx < sp; ++sidx) {
+                const float w = piece_w[h * sp + sidx];
+#pragma unroll
+                for (int e4 = 0; e4 < VE; e4 += 4) {
+                    const float4 v = *reinterpret_cast<const float4*>(src + (size_t)sidx * (hd + 4) + e4);
+                    f[e4] = fmaf(v.x, w, f[e4]);
+                    f[e4 + 1] = fmaf(v.y, w, f[e4 + 1]);
+                    f[e4 + 2] = fmaf(v.z, w, f[e4 + 2]);
+                    f[e4 + 3] = fmaf(v.w, w, f[e4 + 3]);
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < VE; ++e) o[e] = XT(f[e]);
         } else {
             const u32x4 xv = *reinterpret_cast<const u32x4*>(Xb + (size_t)k * ES);
             const u32x4 wv = *reinterpret_cast<const u32x4*>(static_cast<const unsigned char*>(a.norm_w) + (size_t)k * ES);
@@ -813,6 +839,27 @@ __global__ __launch_bounds__(NT) void tl_spmv_direct(KernelArgs a)
 #pragma unroll
         for (int v = 0; v < NT / 64; ++v) total += red[v];
         inv_rms = rsqrtf(total / (float)a.K + a.eps);
+    }
+    if constexpr (PRO == kProAttnCombine) {
+        // the weight of every piece, while the chunks are on their way
+        float* wts = reinterpret_cast<float*>(cst + buffers * (TG + 1));  // [heads][splits]
+        const int hd = a.pro_hd, sp = a.pro_splits, heads = a.K / hd;
+        for (int h = tid; h < heads; h += NT) {
+            const float* stats = static_cast<const float*>(a.X) + (size_t)h * sp * (hd + 4) + hd;
+            float top = -INFINITY;
+            for (int sidx = 0; sidx < sp; ++sidx) top = fmaxf(top, stats[(size_t)sidx * (hd + 4)]);
+            float norm = 0.f;
+            for (int sidx = 0; sidx < sp; ++sidx) {
+                const float m = stats[(size_t)sidx * (hd + 4)];
+                norm = fmaf(stats[(size_t)sidx * (hd + 4) + 1], m == -INFINITY ? 0.f : __expf(m - top), norm);
+            }
+            for (int sidx = 0; sidx < sp; ++sidx) {
+                const float m = stats[(size_t)sidx * (hd + 4)];
+                wts[h * sp + sidx] = m == -INFINITY ? 0.f : __expf(m - top) / norm;
+            }
+        }
+        piece_w = wts;
+        __syncthreads();
     }
     stage_row(0, min(TG, a.T), 0);
     int which = 0;
@@ -1627,7 +1674,9 @@ int launch_spmv_direct_nt(KernelArgs a, const tl_layout_header* h, hipStream_t s
     a.xs_bytes = tg * tile_bytes;
     a.buf_bytes = (int)round_up((int64_t)tg * chunk_bytes, 16);
     const int buffers = tg < a.T ? 2 : 1;
-    const size_t lds = (size_t)buffers * ((size_t)a.xs_bytes + a.buf_bytes) + (size_t)buffers * (tg + 1) * 4 + (NT / 64) * 4;  // + the waves' partial mean squares
+    // + what a producer keeps: the waves' partial mean squares, or the weights of the attention pieces
+    const size_t pro_bytes = PRO == kProAttnCombine ? (size_t)(a.K / std::max(1, a.pro_hd)) * a.pro_splits * 4 : (size_t)(NT / 64) * 4;
+    const size_t lds = (size_t)buffers * ((size_t)a.xs_bytes + a.buf_bytes) + (size_t)buffers * (tg + 1) * 4 + pro_bytes;
     if (lds > 160 * 1024) return fail(TL_ERR_UNSUPPORTED, "one tile needs %zu bytes of LDS", lds);
     const int lpc = NT / TL_BLOCK_COLUMNS;
     const double mean_run = h->mean_run_dwords_x16 / 16.0;
@@ -2012,6 +2061,40 @@ extern "C" int tl_spmv_fused(const tl_layout_header* header, const void* blob_de
         rc = a.x_f16 ? launch_spmv_direct<true, kProSiluGate>(a, header, st) : launch_spmv_direct<false, kProSiluGate>(a, header, st);
     else
         rc = a.x_f16 ? launch_spmv_direct<true, kProAddNorm>(a, header, st) : launch_spmv_direct<false, kProAddNorm>(a, header, st);
+    if (rc) return rc;
+    return finish_launch();
+}
+
+extern "C" int tl_spmv_attn_combine(const tl_layout_header* header, const void* blob_dev, const void* pieces, int splits, int head_dim,
+                                    int x_dtype, void* Y, int y_dtype, const void* scale, int scale_dtype, void* stream)
+{
+    if (int rc = check_header(header)) return rc;
+    if (int rc = check_dtype(x_dtype, "x")) return rc;
+    if (int rc = check_dtype(y_dtype, "y")) return rc;
+    if (scale)
+        if (int rc = check_dtype(scale_dtype, "scale")) return rc;
+    if (!blob_dev || !pieces || !Y) return fail(TL_ERR_ARG, "device pointer is null");
+    if (reinterpret_cast<uintptr_t>(blob_dev) % 256) return fail(TL_ERR_ALIGN, "weight blob must be 256-byte aligned");
+    if (reinterpret_cast<uintptr_t>(pieces) % 16) return fail(TL_ERR_ALIGN, "pieces must be 16-byte aligned");
+    if (splits < 1 || splits > 8) return fail(TL_ERR_ARG, "splits=%d (1 to 8 expected)", splits);
+    const int es = x_dtype == TL_F16 ? 2 : 4, ve = 16 / es;
+    if (head_dim <= 0 || head_dim % ve || header->inners % (uint32_t)head_dim)
+        return fail(TL_ERR_SHAPE, "head_dim=%d must be a multiple of %d and divide K=%u", head_dim, ve, header->inners);
+    if (header->tile_rows % ve || header->inners % ve)
+        return fail(TL_ERR_UNSUPPORTED, "K=%u, tile height %u: the fused single-row kernel needs whole 16-byte pieces per tile", header->inners, header->tile_rows);
+    if ((int64_t)(header->inners / head_dim) * splits * 4 > 16 * 1024) return fail(TL_ERR_UNSUPPORTED, "too many heads x splits for the kernel's LDS table");
+    KernelArgs a;
+    std::memset(&a, 0, sizeof(a));
+    a.w0 = weight_ptrs(header, blob_dev, scale);
+    a.X = pieces; a.pro_splits = splits; a.pro_hd = head_dim;
+    a.Y = Y;
+    a.ldx = header->inners; a.ldy = header->columns;
+    a.M = 1; a.N = (int)header->columns; a.K = (int)header->inners; a.T = (int)header->n_tiles; a.tile_rows = (int)header->tile_rows;
+    a.NB = (int)header->n_blocks;
+    a.x_f16 = x_dtype == TL_F16; a.y_f16 = y_dtype == TL_F16; a.scale_f16 = scale_dtype == TL_F16;
+    a.one = 1.0f;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int rc = a.x_f16 ? launch_spmv_direct<true, kProAttnCombine>(a, header, st) : launch_spmv_direct<false, kProAttnCombine>(a, header, st);
     if (rc) return rc;
     return finish_launch();
 }

@@ -124,7 +124,7 @@ class TernaryLlamaDecoder(nn.Module):
         # single-row steps fold the norms and the SiLU gate into the products' kernels; that kernel wants rows and
         # tiles of whole 16-byte pieces
         self.fused_decode = all(m._header.tile_rows % 8 == 0 and m.in_features % 8 == 0
-                                for layer in self.layers for m in (layer.qkv_proj, layer.gate_up_proj, layer.down_proj)) and \
+                                for layer in self.layers for m in (layer.qkv_proj, layer.o_proj, layer.gate_up_proj, layer.down_proj)) and \
             self.lm_head._header.tile_rows % 8 == 0 and H % 8 == 0
         self._layer_index = {id(layer): i for i, layer in enumerate(self.layers)}
 
@@ -231,15 +231,17 @@ class TernaryLlamaDecoder(nn.Module):
     def _decode_step_fused(self, x, pos, q):
         """One row: the residual add + RMSNorm in front of the q|k|v and gate|up products and the SiLU gate in
         front of the down projection are computed inside those products' kernels (tl_spmv_fused), six launches
-        per layer instead of nine."""
+        per layer instead of nine.  The attention shares the cache rows of a head out among several workgroups
+        (32 heads alone would leave seven compute units in eight idle) and leaves its result in pieces that the
+        output projection folds while it stages its row (tl_spmv_attn_combine)."""
         eps = self.config.rms_norm_eps
         y = None   # what the previous block still has to add to the residual stream
         for layer in self.layers:
             qkv, x = ops.spmv_fused(layer.qkv_proj.device_weight(), "add_rmsnorm", x, y, layer.input_layernorm.weight, eps,
                                     layer.qkv_proj.w_scale, want_sum=True)
             ops.rope_cache_update(qkv, self.rope_cos, self.rope_sin, pos, q, self._cache_of(layer, 0), self._cache_of(layer, 1))
-            a = ops.decode_attention(q, self._cache_of(layer, 0), self._cache_of(layer, 1), pos)
-            o = layer.o_proj(a)
+            pieces = ops.decode_attention_pieces(q, self._cache_of(layer, 0), self._cache_of(layer, 1), pos)
+            o = ops.spmv_attn_combine(layer.o_proj.device_weight(), pieces, self.config.head_dim, x.dtype, layer.o_proj.w_scale)
             gu, x = ops.spmv_fused(layer.gate_up_proj.device_weight(), "add_rmsnorm", x, o, layer.post_attention_layernorm.weight, eps,
                                    layer.gate_up_proj.w_scale, want_sum=True)
             y = ops.spmv_fused(layer.down_proj.device_weight(), "silu_gate", gu, scale=layer.down_proj.w_scale)

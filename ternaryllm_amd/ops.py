@@ -86,6 +86,7 @@ def release_workspaces():
     reuses the memory in stream order).  Not while a captured HIP graph that contains such a product is still
     to be replayed: the graph holds the buffer's address."""
     _workspaces.clear()
+    _attn_workspaces.clear()
 
 
 def _workspace(header, M, x_code, x_layout, device):
@@ -197,6 +198,28 @@ def spmv_fused(weight, producer, inp, inp2=None, norm_weight=None, eps=0.0, scal
     return (y, s_out) if want_sum else y
 
 
+def spmv_attn_combine(weight, pieces, head_dim, x_dtype, scale=None, out_dtype=None):
+    """y[1, N] = (a @ W) * scale where a is the attention output (rounded to x_dtype) that `pieces` -- what
+    decode_attention_pieces returned for batch 1 -- add up to: the output projection with the fold of the
+    pieces inside (tl_spmv_attn_combine).  Raises RuntimeError (TL_ERR_UNSUPPORTED) where the fused kernel
+    does not apply."""
+    K, N = weight.inners, weight.columns
+    if pieces.dtype != torch.float32 or pieces.dim() != 3 or not pieces.is_contiguous() or pieces.device != weight.device:
+        raise ValueError("pieces must be a contiguous float32 [heads, splits, head_dim + 4] tensor on the weight's device")
+    heads, splits, width = pieces.shape
+    if width != head_dim + 4 or heads * head_dim != K:
+        raise ValueError(f"pieces of shape {tuple(pieces.shape)} do not make a row of K={K} with head_dim={head_dim}")
+    out_dtype = out_dtype or x_dtype
+    y = torch.empty((1, N), dtype=out_dtype, device=pieces.device)
+    scale, s_code = _scale_args(scale, N, pieces.device)
+    with torch.cuda.device(pieces.device):
+        rc = _lib.lib().tl_spmv_attn_combine(ctypes.byref(weight.header), weight.blob.data_ptr(), pieces.data_ptr(), splits, head_dim,
+                                             _code(x_dtype, "x_dtype"), y.data_ptr(), _code(out_dtype, "out_dtype"),
+                                             scale.data_ptr() if scale is not None else None, s_code, _stream_ptr(pieces.device))
+    _lib.check(rc)
+    return y
+
+
 def spmm_time(weight, x, iters, scale=None, out_dtype=None, x_layout=_lib.TL_X_ROW_MAJOR):
     """Mean milliseconds per tl_spmm call over `iters` back-to-back calls, timed with HIP events
     recorded on the stream the kernels run on.  Returns (ms, y)."""
@@ -247,10 +270,23 @@ def _kmajor_image(rows, width, like):
     return torch.empty((width, ld), dtype=like.dtype, device=like.device), ld
 
 
-def decode_attention(q, k_cache, v_cache, pos, out=None, kmajor=False):
+_attn_workspaces = {}
+_ATTN_MAX_SPLITS = 8
+
+
+def _attention_splits(B, heads, device):
+    """Workgroups per (batch row, head): as many as keep half the compute units busy (more pieces cost the
+    fold more than they save the pass over the cache), at most 8."""
+    units = torch.cuda.get_device_properties(device).multi_processor_count
+    return max(1, min(_ATTN_MAX_SPLITS, units // max(1, 2 * B * heads)))
+
+
+def decode_attention(q, k_cache, v_cache, pos, out=None, kmajor=False, splits=None):
     """Attention of one query per (batch row, head) over cache rows [0, pos].  q: [B, heads, head_dim];
     caches: [B, heads, max_seq, head_dim]; pos: one-element int64 device tensor.  Returns [B, heads * head_dim],
-    or with kmajor its transpose [heads * head_dim, B] as a view of a K-major image (for spmm's x_layout=1)."""
+    or with kmajor its transpose [heads * head_dim, B] as a view of a K-major image (for spmm's x_layout=1).
+    splits: workgroups that share the cache rows of a (batch row, head) (1 to 8; default: by the size of
+    the step, see _attention_splits)."""
     B, heads, max_seq, hd = k_cache.shape
     ld = 0
     if kmajor:
@@ -267,11 +303,47 @@ def decode_attention(q, k_cache, v_cache, pos, out=None, kmajor=False):
         raise ValueError("shapes of q, out and the caches do not agree")
     if pos.dtype != torch.int64 or pos.numel() != 1 or pos.device != q.device:
         raise ValueError("pos must be a one-element int64 tensor on the same device")
+    if splits is None:
+        splits = _attention_splits(B, heads, q.device)
+    ws_ptr, ws_bytes = None, 0
+    if splits > 1:
+        # scratch for the pieces: one buffer per (device, stream), like the products' (work on a stream is ordered)
+        key = (q.device.index, torch.cuda.current_stream(q.device).cuda_stream)
+        need = B * heads * _ATTN_MAX_SPLITS * (hd + 4) * 4
+        ws = _attn_workspaces.get(key)
+        if ws is None or ws.numel() < need:
+            ws = torch.empty(need, dtype=torch.uint8, device=q.device)
+            _attn_workspaces[key] = ws
+        ws_ptr, ws_bytes = ws.data_ptr(), ws.numel()
     with torch.cuda.device(q.device):
-        rc = _lib.lib().tl_decode_attention(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), _code(q.dtype, "q"), B, heads, hd,
-                                            max_seq, pos.data_ptr(), out.data_ptr(), ld, _stream_ptr(q.device))
+        rc = _lib.lib().tl_decode_attention_split(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), _code(q.dtype, "q"), B, heads, hd,
+                                                  max_seq, pos.data_ptr(), out.data_ptr(), ld, splits, ws_ptr, ws_bytes,
+                                                  _stream_ptr(q.device))
     _lib.check(rc)
     return out[:, :B] if kmajor else out
+
+
+def decode_attention_pieces(q, k_cache, v_cache, pos, splits=None):
+    """The attention of decode_attention left unfolded: float32 [B * heads, splits, head_dim + 4], per piece
+    head_dim unnormalised sums, the piece's maximum and its sum of exponentials (two unused floats behind them).
+    spmv_attn_combine folds them inside the output projection (batch 1)."""
+    B, heads, max_seq, hd = k_cache.shape
+    for t in (q, k_cache, v_cache):
+        if not t.is_contiguous() or t.dtype != q.dtype or t.device != q.device:
+            raise ValueError("tensors must be contiguous, of one dtype, on one device")
+    if q.numel() != B * heads * hd or v_cache.shape != k_cache.shape:
+        raise ValueError("shapes of q and the caches do not agree")
+    if pos.dtype != torch.int64 or pos.numel() != 1 or pos.device != q.device:
+        raise ValueError("pos must be a one-element int64 tensor on the same device")
+    if splits is None:
+        splits = _attention_splits(B, heads, q.device)
+    pieces = torch.empty((B * heads, splits, hd + 4), dtype=torch.float32, device=q.device)
+    with torch.cuda.device(q.device):
+        rc = _lib.lib().tl_decode_attention_split(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), _code(q.dtype, "q"), B, heads, hd,
+                                                  max_seq, pos.data_ptr(), None, 0, splits, pieces.data_ptr(), pieces.numel() * 4,
+                                                  _stream_ptr(q.device))
+    _lib.check(rc)
+    return pieces
 
 
 def add_rmsnorm(x, y, weight, eps, kmajor=False):

@@ -215,6 +215,57 @@ def test_decode_attention_over_a_long_cache(cuda):
         assert (out.double() - ref).abs().max().item() <= 3e-3 * max(1.0, ref.abs().max().item()), pos
 
 
+def test_split_attention_and_its_fold_inside_the_output_projection(cuda, oracle):
+    """tl_decode_attention_split: the cache rows of a head shared out among 1-8 workgroups, folded by the second
+    launch, against the single-pass kernel and a float64 restatement (few rows, pieces without rows, a position
+    past the end); and the pieces folded inside the output projection (tl_spmv_attn_combine) against the
+    separate fold followed by the plain product."""
+    from tests.util import max_rel_err, ternary_weight
+    from ternaryllm_amd import ops
+    from ternaryllm_amd.packing import PackedWeight
+    g = torch.Generator().manual_seed(23)
+    for dtype, tol in ((torch.float16, 3e-3), (torch.float32, 2e-5)):
+        for B, H, hd, S in ((1, 32, 128, 700), (2, 3, 64, 90)):
+            q = torch.randn((B, H, hd), generator=g).to(dtype).to(cuda)
+            kc = torch.randn((B, H, S, hd), generator=g).to(dtype).to(cuda)
+            vc = torch.randn((B, H, S, hd), generator=g).to(dtype).to(cuda)
+            for pos in (0, 2, 6, S // 2, S - 1, S + 3):
+                n = min(pos, S - 1) + 1
+                p = torch.tensor([pos], dtype=torch.long, device=cuda)
+                sc = (q.double()[:, :, None, :] * kc.double()[:, :, :n]).sum(-1) / hd ** 0.5
+                ref = (sc.softmax(-1)[..., None] * vc.double()[:, :, :n]).sum(2).reshape(B, H * hd)
+                single = ops.decode_attention(q, kc, vc, p, splits=1)
+                for splits in (2, 3, 8):
+                    out = ops.decode_attention(q, kc, vc, p, splits=splits)
+                    assert (out.double() - ref).abs().max().item() <= tol * max(1.0, ref.abs().max().item()), (pos, splits)
+                    assert (out.double() - single.double()).abs().max().item() <= tol * max(1.0, ref.abs().max().item())
+                    outk = ops.decode_attention(q, kc, vc, p, kmajor=True, splits=splits)
+                    assert torch.equal(outk.t(), out)
+        # the output projection with the fold inside, batch 1
+        H, hd, S, N = 32, 128, 700, 272
+        K = H * hd
+        w = ternary_weight(K, N, 0.7, 77)
+        dw = ops.DeviceWeight(PackedWeight.from_dense(w), cuda)
+        scale = (0.5 + torch.rand(N, generator=g)).to(dtype).to(cuda)
+        q = torch.randn((1, H, hd), generator=g).to(dtype).to(cuda)
+        kc = torch.randn((1, H, S, hd), generator=g).to(dtype).to(cuda)
+        vc = torch.randn((1, H, S, hd), generator=g).to(dtype).to(cuda)
+        for pos in (1, 333, S - 1):
+            p = torch.tensor([pos], dtype=torch.long, device=cuda)
+            for splits in (1, 4, 8):
+                pieces = ops.decode_attention_pieces(q, kc, vc, p, splits=splits)
+                assert pieces.shape == (H, splits, hd + 4)
+                out = ops.spmv_attn_combine(dw, pieces, hd, dtype, scale)
+                a = ops.decode_attention(q, kc, vc, p, splits=splits)
+                unfused = ops.spmm(dw, a, scale)
+                # the folded row may differ from the separately folded one in its last bit (fp32 sums in another order)
+                assert max_rel_err(out.double().cpu().numpy(), unfused.double().cpu().numpy(), a.double().cpu().numpy(), w) <= tol
+    with pytest.raises(ValueError):
+        ops.spmv_attn_combine(dw, torch.zeros((H, 2, hd + 3), device=cuda), hd, torch.float16)
+    with pytest.raises(ValueError, match="splits"):
+        ops.decode_attention(q, kc, vc, p, splits=9)
+
+
 def test_add_rmsnorm_and_silu_mul(cuda):
     from ternaryllm_amd import ops
     g = torch.Generator().manual_seed(10)
