@@ -670,6 +670,149 @@ __global__ __launch_bounds__(kBlockThreads) void tl_spmm_quad(KernelArgs a)
 }
 
 // ---------------------------------------------------------------------------
+// 16 fp16 rows, eight per lane, two column blocks per workgroup.
+// ---------------------------------------------------------------------------
+// tl_spmm_quad<16, true> with the work cut differently: a lane owns EIGHT rows of one column (one 16-byte LDS
+// read and eight accumulates per index, so each index is decoded by two lanes instead of four), and the 64 lanes
+// of a wave cover 32 columns -- two neighbouring blocks, which share the staged activation image.  Per non-zero
+// that is five vector ops fewer in the loop, and half as many lanes go through a run's set-up and tail; per block
+// the image is staged half as often.  The launcher uses it where it still leaves every compute unit workgroups
+// enough (wide outputs).
+__global__ __launch_bounds__(kBlockThreads) void tl_spmm_octet(KernelArgs a)
+{
+    extern __shared__ __align__(16) unsigned char lds[];
+    using XT = __half;
+    constexpr int NT = kBlockThreads;
+    constexpr int MT = 16, ES = 2, VPS = MT * ES / 16, BS = 2, COLS = TL_BLOCK_COLUMNS * BS;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int TG = a.tiles_per_group;
+    const int nb0 = blockIdx.x * BS, m0 = blockIdx.y * MT;
+    const int bs = min(BS, a.NB - nb0);  // blocks this workgroup really has
+    const int stage_bytes = a.xs_bytes + a.buf_bytes;
+    const int block_buf_bytes = a.buf_bytes / BS;  // chunk copies of one block and group (a multiple of 16)
+    uint32_t* cst = reinterpret_cast<uint32_t*>(lds + 2 * stage_bytes);  // [2][BS][TG + 1] chunk starts inside a block's chunk copies
+    const_u32_ptr cs = as_const(a.w0.chunkstart) + (size_t)nb0 * a.T;
+    const unsigned char* Xb = static_cast<const unsigned char*>(a.X) + (size_t)m0 * ES;
+    const size_t row_bytes = (size_t)a.ldx * ES;
+    using global_ptr = const __attribute__((address_space(1))) void*;
+    using lds_ptr = __attribute__((address_space(3))) void*;
+
+    auto issue = [&](int t, int nt, int which) {
+        unsigned char* xs = lds + which * stage_bytes;
+        unsigned char* buf = xs + a.xs_bytes;
+        const int pieces = nt * kTileSlots * VPS;  // a multiple of 64: whole waves
+        for (int first = wave * 64; first < pieces; first += NT) {
+            const int p = first + lane, slot = p / VPS, v = p % VPS;
+            const int r = slot & (kTileSlots - 1), k = (t + (slot >> 8)) * a.tile_rows + r;
+            if (r < a.tile_rows && k < a.K)
+                __builtin_amdgcn_global_load_lds((global_ptr)(Xb + (size_t)k * row_bytes + v * 16), (lds_ptr)(xs + (size_t)first * 16), 16, 0, 0);
+            else
+                *reinterpret_cast<u32x4*>(xs + (size_t)p * 16) = u32x4{0u, 0u, 0u, 0u};
+        }
+        for (int j = 0; j < bs; ++j) {
+            const_u32_ptr csj = cs + (size_t)j * a.T;
+            const uint32_t lo = csj[t];
+            const int vectors = (int)((csj[t + nt] - lo) / 4);
+            unsigned char* bufj = buf + (size_t)j * block_buf_bytes;
+            for (int first = wave * 64; first < vectors; first += NT)
+                if (first + lane < vectors)
+                    __builtin_amdgcn_global_load_lds((global_ptr)(a.w0.stream + lo + (size_t)(first + lane) * 4), (lds_ptr)(bufj + (size_t)first * 16), 16, 0, 0);
+            if (tid <= nt) cst[(which * BS + j) * (TG + 1) + tid] = csj[t + tid] - lo;
+        }
+    };
+
+    const int lw_shift = a.lw_shift;
+    const int LPC = 1 << a.lpc_shift, LW = 1 << lw_shift, TP = LPC >> lw_shift;
+    // a wave is one lane group: lanes 2c, 2c + 1 hold rows 0-7 and 8-15 of column c of the workgroup's 32
+    const int q = tid & 1, col = (tid >> 1) & (COLS - 1), lig = tid / (2 * COLS);
+    const int blk = col / TL_BLOCK_COLUMNS, c16 = col % TL_BLOCK_COLUMNS;
+    const int tp = lig >> lw_shift, lw = lig & (LW - 1);
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+    auto issue4 = [](u32x4 (&v)[4], const XT* xq, uint32_t word) {
+        using lds_cptr = const __attribute__((address_space(3))) void*;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const uint32_t r = (word >> (8 * b)) & 0xffu;
+            const uint32_t addr = (uint32_t)reinterpret_cast<uintptr_t>((lds_cptr)(xq + r * MT));
+            asm volatile("ds_read_b128 %0, %1" : "=v"(v[b]) : "v"(addr) : "memory");
+        }
+    };
+    auto add4 = [&](const u32x4 (&v)[4], float sign) {
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                acc[2 * e] = fmaf(__half2float(__ushort_as_half((unsigned short)(v[b][e] & 0xffffu))), sign, acc[2 * e]);
+                acc[2 * e + 1] = fmaf(__half2float(__ushort_as_half((unsigned short)(v[b][e] >> 16))), sign, acc[2 * e + 1]);
+            }
+    };
+
+    issue(0, min(TG, a.T), 0);
+    int which = 0;
+    for (int t = 0; t < a.T; t += TG, which ^= 1) {
+        const int nt = min(TG, a.T - t);
+        // this wave's loads have landed; after the barrier everybody's have, and the other buffer is free
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (t + TG < a.T) issue(t + TG, min(TG, a.T - t - TG), which ^ 1);
+        const unsigned char* xs = lds + which * stage_bytes;
+        const uint32_t* buf = reinterpret_cast<const uint32_t*>(xs + a.xs_bytes + (size_t)blk * block_buf_bytes);
+        const uint32_t* my_cst = cst + (which * BS + blk) * (TG + 1);
+        if (blk < bs) {
+            for (int tl = tp; tl < nt; tl += TP) {
+                const uint32_t* chunk = buf + my_cst[tl];
+                const uint32_t d = chunk[c16];
+                const uint32_t* run = chunk + (d >> 16);
+                const int pd = run_pos_dwords(d), tot = pd + run_neg_dwords(d);
+                const XT* xq = reinterpret_cast<const XT*>(xs) + (size_t)tl * kTileSlots * MT + q * 8;
+                u32x4 va[4], vb[4];
+                int i = lw;
+                for (; i + LW < tot; i += 2 * LW) {
+                    const uint32_t w0 = run[i], w1 = run[i + LW];
+                    issue4(va, xq, w0);
+                    issue4(vb, xq, w1);
+                    quad_wait<4>(va);
+                    add4(va, i < pd ? 1.0f : -1.0f);
+                    quad_wait<0>(vb);
+                    add4(vb, i + LW < pd ? 1.0f : -1.0f);
+                }
+                if (i < tot) {
+                    issue4(va, xq, run[i]);
+                    quad_wait<0>(va);
+                    add4(va, i < pd ? 1.0f : -1.0f);
+                }
+            }
+        }
+    }
+    // fold the LPC partial sums of each (column, row octet) through LDS
+    __syncthreads();
+    float4* red = reinterpret_cast<float4*>(lds);  // [lane group][2][64 lanes]
+    red[(size_t)lig * 128 + lane] = make_float4(acc[0], acc[1], acc[2], acc[3]);
+    red[(size_t)lig * 128 + 64 + lane] = make_float4(acc[4], acc[5], acc[6], acc[7]);
+    __syncthreads();
+    if (tid < 64) {
+        float4 s0 = red[tid], s1 = red[64 + tid];
+#pragma unroll 4
+        for (int l = 1; l < LPC; ++l) {
+            const float4 o0 = red[(size_t)l * 128 + tid], o1 = red[(size_t)l * 128 + 64 + tid];
+            s0.x += o0.x; s0.y += o0.y; s0.z += o0.z; s0.w += o0.w;
+            s1.x += o1.x; s1.y += o1.y; s1.z += o1.z; s1.w += o1.w;
+        }
+        const int n = (nb0 + blk) * TL_BLOCK_COLUMNS + c16;
+        if (blk < bs && n < a.N) {
+            const float sc = load_scale(a.w0.scale, a.scale_f16, n);
+            const float out[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                if (m0 + q * 8 + j < a.M) store_out(a.Y, a.y_f16, (long long)(m0 + q * 8 + j) * a.ldy + n, out[j] * sc);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
 // One activation row (decode), staged by direct global -> LDS loads.
 // ---------------------------------------------------------------------------
 // As tl_spmm_quad, for M = 1 and a contiguous, 16-byte aligned activation row whose tiles are whole
@@ -1474,9 +1617,9 @@ inline int rows_mtile(int x_dtype) { return x_dtype == TL_F16 ? 256 : 128; }
 // Tuning knobs (environment variables of the same names).  They are read once, at the first launch of the
 // process; tl_reload_options() reads them again.  A knob that is not set leaves the launcher's own choice.
 enum Knob { TL_SMALL_LDS, TL_TILE_GROUP, TL_QUAD_SHARE, TL_LW, TL_SPMV_SHARE, TL_SPMV_WIDE, TL_SMALL_MT, TL_SPMV_DIRECT,
-            TL_BLOCK_SET, TL_ROWS_SPLIT, kKnobCount };
+            TL_BLOCK_SET, TL_ROWS_SPLIT, TL_OCTET, kKnobCount };
 const char* const kKnobNames[kKnobCount] = {"TL_SMALL_LDS", "TL_TILE_GROUP", "TL_QUAD_SHARE", "TL_LW", "TL_SPMV_SHARE", "TL_SPMV_WIDE",
-                                            "TL_SMALL_MT", "TL_SPMV_DIRECT", "TL_BLOCK_SET", "TL_ROWS_SPLIT"};
+                                            "TL_SMALL_MT", "TL_SPMV_DIRECT", "TL_BLOCK_SET", "TL_ROWS_SPLIT", "TL_OCTET"};
 struct Knobs {
     bool set[kKnobCount];
     int value[kKnobCount];
@@ -1656,6 +1799,41 @@ int launch_quad_kernel(KernelArgs a, const tl_layout_header* h, hipStream_t st)
     return TL_OK;
 }
 
+// tl_spmm_octet: two blocks per workgroup, LDS sized for up to three workgroups per compute unit.
+int launch_octet_kernel(KernelArgs a, const tl_layout_header* h, hipStream_t st)
+{
+    constexpr int groups = kBlockThreads / 64;  // lane groups: one per wave
+    const int tile_bytes = kTileSlots * 16 * 2;
+    const int chunk_bytes = (int)h->max_chunk_dwords * 4;
+    const unsigned gx = (unsigned)ceil_div(a.NB, 2), gy = (unsigned)ceil_div(a.M, 16);
+    const int share = std::max(1, std::min(knob(TL_QUAD_SHARE, 3), (int)ceil_div((int64_t)gx * gy, compute_units())));
+    const int budget = 160 * 1024 / share - 1024;
+    const int per_tile = tile_bytes + 2 * chunk_bytes;
+    int tg = std::max(1, std::min(a.T, (budget - 256) / (2 * per_tile)));
+    tg = std::max(1, std::min(tg, knob(TL_TILE_GROUP, tg)));
+    tg = (int)ceil_div(a.T, ceil_div(a.T, tg));  // same number of groups, evened out
+    a.tiles_per_group = tg;
+    a.xs_bytes = tg * tile_bytes;
+    a.buf_bytes = 2 * (int)round_up((int64_t)tg * chunk_bytes, 16);
+    const size_t lds = std::max<size_t>(2 * ((size_t)a.xs_bytes + a.buf_bytes) + 2 * 2 * (size_t)(tg + 1) * 4, (size_t)kBlockThreads * 32);
+    if (lds > 160 * 1024) return fail(TL_ERR_UNSUPPORTED, "two tiles of 16 rows and two blocks need %zu bytes of LDS", lds);
+    const double mean_run = h->mean_run_dwords_x16 / 16.0;
+    int lw = 2;
+    while (lw < groups && lw * 8 < mean_run) lw *= 2;
+    while (groups / lw > tg) lw *= 2;
+    lw = std::min(knob(TL_LW, lw), groups);
+    if (lw < 1 || (lw & (lw - 1))) return fail(TL_ERR_ARG, "TL_LW=%d (a power of two expected)", lw);
+    a.lpc_shift = log2_exact(groups);
+    a.lw_shift = log2_exact(lw);
+    static bool raised = false;  // a repeated or racing call is harmless
+    if (!raised) {
+        if (int rc = raise_lds_limit(tl_spmm_octet, 160 * 1024)) return rc;
+        raised = true;
+    }
+    hipLaunchKernelGGL(tl_spmm_octet, dim3(gx, gy), dim3(kBlockThreads), lds, st, a);
+    return TL_OK;
+}
+
 // The direct-load kernel for one activation row.  All of K in one group when `share` workgroups of that
 // size fit a compute unit, else two alternating buffers of TG tiles.
 template <bool XF16, int NT, int PRO = kProNone>
@@ -1748,6 +1926,9 @@ int launch_small(KernelArgs a, const tl_layout_header* h, int x_dtype, void* wor
     }
     if (mt >= 8) {
         if (mt == 8) return a.x_f16 ? launch_quad_kernel<8, true>(a, h, st) : launch_quad_kernel<8, false>(a, h, st);
+        // fp16, 16 rows: eight rows per lane and two blocks per workgroup where the workgroups still fill the chip
+        const bool octet = a.x_f16 && knob(TL_OCTET, ceil_div(a.NB, 2) * ceil_div(a.M, 16) >= 2 * (int64_t)compute_units() ? 1 : 0) != 0;
+        if (octet) return launch_octet_kernel(a, h, st);
         return a.x_f16 ? launch_quad_kernel<16, true>(a, h, st) : launch_quad_kernel<16, false>(a, h, st);
     }
     // one contiguous aligned row whose tiles are whole 16-byte pieces: straight copies into LDS
