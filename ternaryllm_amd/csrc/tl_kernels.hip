@@ -558,12 +558,11 @@ void tl_spmm_block(KernelArgs a)
 // columns next to each other, so one gather instruction reads 16 slots (one per column) as whole
 // contiguous pieces.  The P lane groups of a column share its runs: TP tiles side by side, LW groups
 // per run, up to four dwords (16 independent gathers) per turn.  The P partial sums are folded through LDS.
-template <int MT, bool XF16>
-__global__ __launch_bounds__(kBlockThreads) void tl_spmm_quad(KernelArgs a)
+template <int MT, bool XF16, int NT = kBlockThreads>
+__global__ __launch_bounds__(NT) void tl_spmm_quad(KernelArgs a)
 {
     extern __shared__ __align__(16) unsigned char lds[];
     using XT = typename std::conditional<XF16, __half, float>::type;
-    constexpr int NT = kBlockThreads;
     constexpr int ES = (int)sizeof(XT);
     constexpr int SLOT = MT * ES;      // bytes of a slot
     constexpr int VPS = SLOT / 16;     // 16-byte pieces per slot
@@ -1617,9 +1616,9 @@ inline int rows_mtile(int x_dtype) { return x_dtype == TL_F16 ? 256 : 128; }
 // Tuning knobs (environment variables of the same names).  They are read once, at the first launch of the
 // process; tl_reload_options() reads them again.  A knob that is not set leaves the launcher's own choice.
 enum Knob { TL_SMALL_LDS, TL_TILE_GROUP, TL_QUAD_SHARE, TL_LW, TL_SPMV_SHARE, TL_SPMV_WIDE, TL_SMALL_MT, TL_SPMV_DIRECT,
-            TL_BLOCK_SET, TL_ROWS_SPLIT, TL_OCTET, kKnobCount };
+            TL_BLOCK_SET, TL_ROWS_SPLIT, TL_OCTET, TL_QUAD_WIDE, kKnobCount };
 const char* const kKnobNames[kKnobCount] = {"TL_SMALL_LDS", "TL_TILE_GROUP", "TL_QUAD_SHARE", "TL_LW", "TL_SPMV_SHARE", "TL_SPMV_WIDE",
-                                            "TL_SMALL_MT", "TL_SPMV_DIRECT", "TL_BLOCK_SET", "TL_ROWS_SPLIT", "TL_OCTET"};
+                                            "TL_SMALL_MT", "TL_SPMV_DIRECT", "TL_BLOCK_SET", "TL_ROWS_SPLIT", "TL_OCTET", "TL_QUAD_WIDE"};
 struct Knobs {
     bool set[kKnobCount];
     int value[kKnobCount];
@@ -1761,11 +1760,11 @@ inline int log2_exact(int v)
 // The direct-load kernel for 8- and 16-row slots.  Its LDS holds two buffers of TG tiles (activation image +
 // chunk copies); TG is sized so that `share` workgroups fit a compute unit, as many as the launch can
 // give each compute unit, up to four.
-template <int MT, bool XF16>
+template <int MT, bool XF16, int NT = kBlockThreads>
 int launch_quad_kernel(KernelArgs a, const tl_layout_header* h, hipStream_t st)
 {
     constexpr int es = XF16 ? 2 : 4;
-    constexpr int groups = kBlockThreads / (TL_BLOCK_COLUMNS * (MT / 4));  // lane groups per column
+    constexpr int groups = NT / (TL_BLOCK_COLUMNS * (MT / 4));  // lane groups per column
     const int tile_bytes = kTileSlots * MT * es;
     const int chunk_bytes = (int)h->max_chunk_dwords * 4;
     const unsigned gx = (unsigned)a.NB, gy = (unsigned)ceil_div(a.M, MT);
@@ -1777,25 +1776,25 @@ int launch_quad_kernel(KernelArgs a, const tl_layout_header* h, hipStream_t st)
     a.tiles_per_group = tg;
     a.xs_bytes = tg * tile_bytes;
     a.buf_bytes = (int)round_up((int64_t)tg * chunk_bytes, 16);
-    const size_t lds = std::max<size_t>(2 * ((size_t)a.xs_bytes + a.buf_bytes) + 2 * (size_t)(tg + 1) * 4, (size_t)kBlockThreads * 16);
+    const size_t lds = std::max<size_t>(2 * ((size_t)a.xs_bytes + a.buf_bytes) + 2 * (size_t)(tg + 1) * 4, (size_t)NT * 16);
     if (lds > 160 * 1024) return fail(TL_ERR_UNSUPPORTED, "two tiles of %d rows need %zu bytes of LDS", MT, lds);
     // lane groups per run: a run's dwords go round the LW groups, four per group and turn; no more
     // tiles side by side than a group of tiles has
     const double mean_run = h->mean_run_dwords_x16 / 16.0;
     int lw = 2;
-    while (lw < groups && lw * 8 < mean_run) lw *= 2;
+    while (lw < groups && lw * (NT > kBlockThreads ? 16 : 8) < mean_run) lw *= 2;  // the wide workgroup has tiles enough side by side
     while (groups / lw > tg) lw *= 2;
     lw = std::min(knob(TL_LW, lw), groups);
     if (lw < 1 || (lw & (lw - 1))) return fail(TL_ERR_ARG, "TL_LW=%d (a power of two expected)", lw);
     a.lpc_shift = log2_exact(groups);
     a.lw_shift = log2_exact(lw);
-    auto kernel = tl_spmm_quad<MT, XF16>;
+    auto kernel = tl_spmm_quad<MT, XF16, NT>;
     static bool raised = false;  // per instantiation; a repeated or racing call is harmless
     if (!raised) {
         if (int rc = raise_lds_limit(kernel, 160 * 1024)) return rc;
         raised = true;
     }
-    hipLaunchKernelGGL(kernel, dim3(gx, gy), dim3(kBlockThreads), lds, st, a);
+    hipLaunchKernelGGL(kernel, dim3(gx, gy), dim3(NT), lds, st, a);
     return TL_OK;
 }
 
@@ -1895,7 +1894,11 @@ int launch_small(KernelArgs a, const tl_layout_header* h, int x_dtype, void* wor
     while (mt < a.M && mt < 16) mt *= 2;
     // 16-row slots with no more workgroups than compute units: 8-row slots give twice the workgroups,
     // each with half the LDS image, so that two share a compute unit and hide each other's waits.
-    if (mt == 16 && (int64_t)a.NB * ceil_div(a.M, 16) <= compute_units()) mt = 8;
+    const bool alone = (int64_t)a.NB * ceil_div(a.M, 16) <= compute_units();  // a workgroup of 16-row slots would have its compute unit to itself
+    // ... then it takes 1024 threads (16 lane groups: the index of a non-zero is decoded once for all 16 rows, and
+    // the runs are shared out among fewer lanes each); TL_QUAD_WIDE=0 runs two 8-row halves of 512 threads instead
+    const bool wide = mt == 16 && alone && knob(TL_QUAD_WIDE, 1) != 0;
+    if (mt == 16 && alone && !wide) mt = 8;
     mt = knob(TL_SMALL_MT, mt);
     if (mt != 1 && mt != 2 && mt != 4 && mt != 8 && mt != 16) return fail(TL_ERR_ARG, "TL_SMALL_MT=%d (1, 2, 4, 8 or 16 expected)", mt);
     const int es = x_dtype == TL_F16 ? 2 : 4;
@@ -1929,6 +1932,7 @@ int launch_small(KernelArgs a, const tl_layout_header* h, int x_dtype, void* wor
         // fp16, 16 rows: eight rows per lane and two blocks per workgroup where the workgroups still fill the chip
         const bool octet = a.x_f16 && knob(TL_OCTET, ceil_div(a.NB, 2) * ceil_div(a.M, 16) >= 2 * (int64_t)compute_units() ? 1 : 0) != 0;
         if (octet) return launch_octet_kernel(a, h, st);
+        if (wide) return a.x_f16 ? launch_quad_kernel<16, true, 1024>(a, h, st) : launch_quad_kernel<16, false, 1024>(a, h, st);
         return a.x_f16 ? launch_quad_kernel<16, true>(a, h, st) : launch_quad_kernel<16, false>(a, h, st);
     }
     // one contiguous aligned row whose tiles are whole 16-byte pieces: straight copies into LDS
