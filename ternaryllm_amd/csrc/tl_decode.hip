@@ -8,6 +8,9 @@
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
+#include <atomic>
+
 #include "tl_common.h"
 
 using namespace tl;
@@ -241,7 +244,9 @@ __global__ __launch_bounds__(256) void tl_add_rmsnorm_k(const T* __restrict__ x,
 }
 
 // The same for rows that are whole 16-byte vectors and at most 4 vectors per thread of a 512-thread
-// workgroup: every value is read once, all loads of a thread are in flight together.
+// workgroup: every value is read once, all loads of a thread are in flight together.  With few rows the
+// launch has gridDim.y workgroups per row: each reads the whole row (the sum of squares needs it) and writes
+// its share of the columns -- the K-major image is written value by value, a row apart, and that is the slow part.
 template <typename T>
 __global__ __launch_bounds__(512) void tl_add_rmsnorm_vec(const T* __restrict__ x, const T* __restrict__ y, const T* __restrict__ weight,
                                                           T* __restrict__ x_out, T* __restrict__ h_out, long long h_kld, int width, float eps)
@@ -273,7 +278,8 @@ __global__ __launch_bounds__(512) void tl_add_rmsnorm_vec(const T* __restrict__ 
             val[k][e] = v;
             if (live) ss = fmaf(v, v, ss);
         }
-        if (live && x_out) {
+        const bool mine = (((int)threadIdx.x + k * 512) * (int)gridDim.y) / nvec == (int)blockIdx.y;  // this workgroup's share of the columns
+        if (live && mine && x_out) {
             uint4 o;
             T* oe = reinterpret_cast<T*>(&o);
 #pragma unroll
@@ -291,7 +297,7 @@ __global__ __launch_bounds__(512) void tl_add_rmsnorm_vec(const T* __restrict__ 
     const float inv = rsqrtf(total / (float)width + eps);
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
-        if ((int)threadIdx.x + k * 512 < nvec) {
+        if ((int)threadIdx.x + k * 512 < nvec && (((int)threadIdx.x + k * 512) * (int)gridDim.y) / nvec == (int)blockIdx.y) {
             const T* we = reinterpret_cast<const T*>(&wv[k]);
             uint4 o;
             T* oe = reinterpret_cast<T*>(&o);
@@ -341,6 +347,20 @@ int check_common(int dtype, int64_t batch, int heads, int head_dim, int64_t max_
     if (head_dim <= 0 || head_dim % 2) return fail(TL_ERR_SHAPE, "head_dim=%d must be positive and even", head_dim);
     if (!pos_dev) return fail(TL_ERR_ARG, "position pointer is null");
     return TL_OK;
+}
+
+// Compute units of the current device, read once per device.
+int device_units()
+{
+    static std::atomic<int> cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 64;
+    int units = cached[dev].load(std::memory_order_relaxed);
+    if (units == 0) {
+        if (hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || units <= 0) units = 64;
+        cached[dev].store(units, std::memory_order_relaxed);
+    }
+    return units;
 }
 
 int launched()
@@ -462,12 +482,15 @@ extern "C" int tl_add_rmsnorm(const void* x, const void* y, const void* weight, 
     const int ve = dtype == TL_F16 ? 8 : 4;
     auto aligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
     if (width % ve == 0 && width / ve <= 4 * 512 && aligned(x) && aligned(y) && aligned(weight) && aligned(x_out) && aligned(h_out)) {
+        // workgroups per row: as many as spread a small launch over the chip, at most 8
+        const int units = device_units();
+        const unsigned parts = (unsigned)std::max<int64_t>(1, std::min<int64_t>(8, units / (4 * rows)));
         if (dtype == TL_F16)
-            hipLaunchKernelGGL(tl_add_rmsnorm_vec<__half>, dim3((unsigned)rows), dim3(512), 0, st, static_cast<const __half*>(x),
+            hipLaunchKernelGGL(tl_add_rmsnorm_vec<__half>, dim3((unsigned)rows, parts), dim3(512), 0, st, static_cast<const __half*>(x),
                                static_cast<const __half*>(y), static_cast<const __half*>(weight), static_cast<__half*>(x_out),
                                static_cast<__half*>(h_out), kld, width, eps);
         else
-            hipLaunchKernelGGL(tl_add_rmsnorm_vec<float>, dim3((unsigned)rows), dim3(512), 0, st, static_cast<const float*>(x),
+            hipLaunchKernelGGL(tl_add_rmsnorm_vec<float>, dim3((unsigned)rows, parts), dim3(512), 0, st, static_cast<const float*>(x),
                                static_cast<const float*>(y), static_cast<const float*>(weight), static_cast<float*>(x_out),
                                static_cast<float*>(h_out), kld, width, eps);
         return launched();
