@@ -1049,6 +1049,123 @@ __global__ __launch_bounds__(NT) void tl_spmv_direct(KernelArgs a)
 }
 
 // ---------------------------------------------------------------------------
+// One activation row, a tile per wave.
+// ---------------------------------------------------------------------------
+// tl_spmv_direct with the work cut the other way: a wave owns whole TILES of the workgroup's block (tiles w,
+// w + W, ... of W waves), all 16 columns of them, four lanes to a run.  What a wave gathers from -- its tiles' chunks
+// and their pieces of the activation row -- it loads itself, so no wave waits for another until the column sums
+// are folded at the very end: a wave starts on a tile when that tile's loads have landed (its own vmcnt, no
+// barrier), while the loads of later tiles and of the other waves are still in flight.  The kernel's length is
+// then about the time the block's bytes take to arrive plus one tile's gather, where tl_spmv_direct, which splits
+// a tile's columns over the waves and so needs every wave's loads behind a barrier, adds the whole gather to it.
+// Only the plain product runs here: with a producer, whose operands must arrive and be worked on before the
+// first gather, tl_spmv_direct is the faster of the two.
+
+// Waits until at most `later` of this wave's vector-memory instructions are outstanding (they complete in
+// order): everything issued before the last `later` has then arrived.  Counts above 13 wait for a few more.
+__device__ __forceinline__ void tiles_wait_vm(int later)
+{
+    switch (later) {
+        case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+        case 1: asm volatile("s_waitcnt vmcnt(1)" ::: "memory"); break;
+        case 2: asm volatile("s_waitcnt vmcnt(2)" ::: "memory"); break;
+        case 3: asm volatile("s_waitcnt vmcnt(3)" ::: "memory"); break;
+        case 4: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
+        case 5: asm volatile("s_waitcnt vmcnt(5)" ::: "memory"); break;
+        case 6: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
+        case 7: asm volatile("s_waitcnt vmcnt(7)" ::: "memory"); break;
+        case 8: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+        case 9: asm volatile("s_waitcnt vmcnt(9)" ::: "memory"); break;
+        case 10: asm volatile("s_waitcnt vmcnt(10)" ::: "memory"); break;
+        case 11: asm volatile("s_waitcnt vmcnt(11)" ::: "memory"); break;
+        case 12: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
+        default: asm volatile("s_waitcnt vmcnt(13)" ::: "memory"); break;
+    }
+}
+
+constexpr int kTilesMaxOwn = 8;  // tiles a wave of tl_spmv_tiles may own
+
+template <bool XF16, int NT>
+__global__ __launch_bounds__(NT) void tl_spmv_tiles(KernelArgs a)
+{
+    extern __shared__ __align__(16) unsigned char lds[];
+    using XT = typename std::conditional<XF16, __half, float>::type;
+    constexpr int ES = (int)sizeof(XT);
+    constexpr int VE = 16 / ES;                  // values per 16-byte piece
+    constexpr int PITCH = kTileSlots + kSpmvImageSkew / ES;  // slots from one tile image to the next
+    constexpr int W = NT / 64;                   // waves
+    constexpr int kMaxOwn = kTilesMaxOwn;        // tiles a wave may own (the launcher holds T to W * kMaxOwn)
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nb = blockIdx.x;
+    const_u32_ptr cs = as_const(a.w0.chunkstart) + (size_t)nb * a.T;
+    const unsigned char* Xb = static_cast<const unsigned char*>(a.X);
+    unsigned char* xs = lds;                     // [T] tile images
+    unsigned char* buf = lds + a.xs_bytes;       // the block's chunks, as they lie in the stream
+    float* red = reinterpret_cast<float*>(lds + a.xs_bytes + a.buf_bytes);  // [W][16] column sums of the waves
+    using global_ptr = const __attribute__((address_space(1))) void*;
+    using lds_ptr = __attribute__((address_space(3))) void*;
+    const uint32_t base = cs[0];
+
+    // every load of this wave, tile after tile; loads[j] = vector-memory instructions of its j-th tile
+    int loads[kMaxOwn];
+#pragma unroll
+    for (int j = 0; j < kMaxOwn; ++j) {
+        loads[j] = 0;
+        const int t = wave + j * W;
+        if (t < a.T) {
+            const uint32_t lo = cs[t];
+            const int vectors = (int)((cs[t + 1] - lo) / 4);
+            unsigned char* dst = buf + (size_t)(lo - base) * 4;
+            for (int first = 0; first < vectors; first += 64) {
+                if (first + lane < vectors)
+                    __builtin_amdgcn_global_load_lds((global_ptr)(a.w0.stream + lo + (size_t)(first + lane) * 4), (lds_ptr)(dst + (size_t)first * 16), 16, 0, 0);
+                ++loads[j];
+            }
+            // the tile's piece of the row: pieces of rows that exist are copied, the rest of the 256 slots (the zero
+            // slot among them) is zeroed
+            const int rows_here = min(a.tile_rows, a.K - t * a.tile_rows);
+            unsigned char* image = xs + (size_t)t * PITCH * ES;
+            if (lane * VE < rows_here)
+                __builtin_amdgcn_global_load_lds((global_ptr)(Xb + ((size_t)t * a.tile_rows + (size_t)lane * VE) * ES), (lds_ptr)image, 16, 0, 0);
+            else if (lane * VE < kTileSlots)
+                *reinterpret_cast<u32x4*>(image + (size_t)lane * 16) = u32x4{0u, 0u, 0u, 0u};
+            ++loads[j];
+        }
+    }
+
+    const int c16 = lane >> 2, lw = lane & 3;
+    float acc[1] = {0.f};
+#pragma unroll
+    for (int j = 0; j < kMaxOwn; ++j) {
+        const int t = wave + j * W;
+        if (t < a.T) {
+            int later = 0;  // loads issued after this tile's
+#pragma unroll
+            for (int q = j + 1; q < kMaxOwn; ++q) later += loads[q];
+            tiles_wait_vm(later);
+            const uint32_t* chunk = reinterpret_cast<const uint32_t*>(buf) + (cs[t] - base);
+            const uint32_t d = chunk[c16];
+            const uint32_t* run = chunk + (d >> 16);
+            const int pd = run_pos_dwords(d), tot = pd + run_neg_dwords(d);
+            const XT* xt = reinterpret_cast<const XT*>(xs) + (size_t)t * PITCH;
+            for (int i = lw; i < tot; i += 4) gather_add<1, XT>(acc, xt, run[i], i < pd ? 1.0f : -1.0f);
+        }
+    }
+    acc[0] += __shfl_xor(acc[0], 1, 64);
+    acc[0] += __shfl_xor(acc[0], 2, 64);
+    if (lw == 0) red[wave * TL_BLOCK_COLUMNS + c16] = acc[0];
+    __syncthreads();
+    if (tid < TL_BLOCK_COLUMNS) {
+        float sum = 0.f;
+#pragma unroll
+        for (int w = 0; w < W; ++w) sum += red[w * TL_BLOCK_COLUMNS + tid];
+        const int n = nb * TL_BLOCK_COLUMNS + tid;
+        if (n < a.N) store_out(a.Y, a.y_f16, n, sum * load_scale(a.w0.scale, a.scale_f16, n));
+    }
+}
+
+// ---------------------------------------------------------------------------
 // Activation re-layout for the row-parallel kernel: XT[k][m] (m contiguous, padded
 // with zeros to ldm columns) from row-major X[m][k] or K-major X[k][m].
 // ---------------------------------------------------------------------------
@@ -1616,9 +1733,9 @@ inline int rows_mtile(int x_dtype) { return x_dtype == TL_F16 ? 256 : 128; }
 // Tuning knobs (environment variables of the same names).  They are read once, at the first launch of the
 // process; tl_reload_options() reads them again.  A knob that is not set leaves the launcher's own choice.
 enum Knob { TL_SMALL_LDS, TL_TILE_GROUP, TL_QUAD_SHARE, TL_LW, TL_SPMV_SHARE, TL_SPMV_WIDE, TL_SMALL_MT, TL_SPMV_DIRECT,
-            TL_BLOCK_SET, TL_ROWS_SPLIT, TL_OCTET, TL_QUAD_WIDE, kKnobCount };
+            TL_BLOCK_SET, TL_ROWS_SPLIT, TL_OCTET, TL_QUAD_WIDE, TL_SPMV_TILES, kKnobCount };
 const char* const kKnobNames[kKnobCount] = {"TL_SMALL_LDS", "TL_TILE_GROUP", "TL_QUAD_SHARE", "TL_LW", "TL_SPMV_SHARE", "TL_SPMV_WIDE",
-                                            "TL_SMALL_MT", "TL_SPMV_DIRECT", "TL_BLOCK_SET", "TL_ROWS_SPLIT", "TL_OCTET", "TL_QUAD_WIDE"};
+                                            "TL_SMALL_MT", "TL_SPMV_DIRECT", "TL_BLOCK_SET", "TL_ROWS_SPLIT", "TL_OCTET", "TL_QUAD_WIDE", "TL_SPMV_TILES"};
 struct Knobs {
     bool set[kKnobCount];
     int value[kKnobCount];
@@ -1873,12 +1990,43 @@ int launch_spmv_direct_nt(KernelArgs a, const tl_layout_header* h, hipStream_t s
     return TL_OK;
 }
 
+// tl_spmv_tiles: every tile of the block resident (a wave loads its own and waits for nobody else's).
+// Returns TL_ERR_UNSUPPORTED when that does not fit; the caller then takes tl_spmv_direct.
+template <bool XF16, int NT>
+int launch_spmv_tiles_nt(KernelArgs a, const tl_layout_header* h, hipStream_t st)
+{
+    constexpr int es = XF16 ? 2 : 4;
+    const int tile_bytes = kTileSlots * es + kSpmvImageSkew;
+    const int chunk_bytes = (int)h->max_chunk_dwords * 4;
+    if (a.T > (NT / 64) * kTilesMaxOwn) return TL_ERR_UNSUPPORTED;
+    a.xs_bytes = a.T * tile_bytes;
+    a.buf_bytes = (int)round_up((int64_t)a.T * chunk_bytes, 16);
+    const size_t lds = (size_t)a.xs_bytes + a.buf_bytes + (size_t)(NT / 64) * TL_BLOCK_COLUMNS * 4;
+    const int share = std::max(1, std::min(knob(TL_SPMV_SHARE, 4), (int)ceil_div(a.NB, compute_units())));
+    if (lds > (size_t)(160 * 1024 / share - 1024)) return TL_ERR_UNSUPPORTED;
+    auto kernel = tl_spmv_tiles<XF16, NT>;
+    static bool raised = false;  // per instantiation; a repeated or racing call is harmless
+    if (!raised) {
+        if (int rc = raise_lds_limit(kernel, 160 * 1024)) return rc;
+        raised = true;
+    }
+    hipLaunchKernelGGL(kernel, dim3((unsigned)a.NB), dim3(NT), lds, st, a);
+    return TL_OK;
+}
+
 // With no more blocks than compute units a workgroup has its compute unit to itself: 1024 threads
 // (64 lanes per column) then keep more gathers in flight than 512 do.
 template <bool XF16, int PRO = kProNone>
 int launch_spmv_direct(const KernelArgs& a, const tl_layout_header* h, hipStream_t st)
 {
     const bool wide = knob(TL_SPMV_WIDE, a.NB <= compute_units() ? 1 : 0) != 0;
+    if constexpr (PRO == kProNone) {
+        // the tile-per-wave kernel where the block fits it; with a producer it is the slower of the two
+        if (knob(TL_SPMV_TILES, 1) != 0) {
+            const int rc = wide ? launch_spmv_tiles_nt<XF16, 1024>(a, h, st) : launch_spmv_tiles_nt<XF16, kBlockThreads>(a, h, st);
+            if (rc != TL_ERR_UNSUPPORTED) return rc;
+        }
+    }
     return wide ? launch_spmv_direct_nt<XF16, 1024, PRO>(a, h, st) : launch_spmv_direct_nt<XF16, kBlockThreads, PRO>(a, h, st);
 }
 

@@ -210,7 +210,8 @@ def test_small_m_kernels_in_every_mode(cuda, oracle, dtype):
     for M in (1, 6, 16, 37):
         x = activations(M, K, 72 + M, dtype, integer=True)
         ref = oracle.fast_product(x.double().numpy(), w)
-        extra = [{"TL_SPMV_DIRECT": "0"}, {"TL_SPMV_WIDE": "0"}, {"TL_SPMV_WIDE": "1"}, {"TL_SPMV_WIDE": "1", "TL_TILE_GROUP": "2"}] if M == 1 else [{"TL_SMALL_MT": "8"}, {"TL_SMALL_MT": "16"}, {"TL_SMALL_MT": "16", "TL_TILE_GROUP": "2"},
+        extra = [{"TL_SPMV_DIRECT": "0"}, {"TL_SPMV_WIDE": "0"}, {"TL_SPMV_WIDE": "1"}, {"TL_SPMV_WIDE": "1", "TL_TILE_GROUP": "2"},
+                 {"TL_SPMV_TILES": "1"}, {"TL_SPMV_TILES": "1", "TL_SPMV_WIDE": "0"}, {"TL_SPMV_TILES": "0"}] if M == 1 else [{"TL_SMALL_MT": "8"}, {"TL_SMALL_MT": "16"}, {"TL_SMALL_MT": "16", "TL_TILE_GROUP": "2"},
                                    {"TL_SMALL_MT": "16", "TL_OCTET": "1"}, {"TL_SMALL_MT": "16", "TL_OCTET": "1", "TL_TILE_GROUP": "1"},
                                    {"TL_SMALL_MT": "16", "TL_OCTET": "1", "TL_LW": "1", "TL_TILE_GROUP": "8"},
                                    {"TL_QUAD_WIDE": "0"}, {"TL_QUAD_WIDE": "1", "TL_LW": "2"}, {"TL_QUAD_WIDE": "1", "TL_TILE_GROUP": "1"}]
