@@ -309,6 +309,19 @@ int tl_decode_attention_split(const void* q, const void* k_cache, const void* v_
                               const int64_t* pos_dev, void* out, int64_t out_kmajor_ld,
                               int splits, void* workspace, int64_t workspace_bytes, void* stream);
 
+/* tl_rope_cache_update and tl_decode_attention_split as ONE launch: the attention kernel rotates q on the way
+ * in, lets the token's rotated key and its value stand in for cache row *pos_dev (which the cache does not
+ * hold yet), and the workgroup whose rows include that row writes them into the caches for the steps to come
+ * (TernaryLLM/TernaryAttn.py:93-113).  qkv, cos_table, sin_table as in tl_rope_cache_update; the rest as in
+ * tl_decode_attention_split (workspace may be NULL when splits == 1 and out is given).  Values are rounded to
+ * `dtype` where the two separate calls store them: out, the pieces and the caches equal theirs bit for bit.
+ * A position outside [0, max_seq) writes nothing; the attention then covers the rows the cache has. */
+int tl_decode_attention_rope(const void* qkv, const void* cos_table, const void* sin_table,
+                             void* k_cache, void* v_cache, int dtype,
+                             int64_t batch, int heads, int head_dim, int64_t max_seq,
+                             const int64_t* pos_dev, void* out, int64_t out_kmajor_ld,
+                             int splits, void* workspace, int64_t workspace_bytes, void* stream);
+
 /* Y[N] = (x * W) * scale for ONE activation row x that the call produces itself, so that a decode step
  * needs neither a launch nor a trip through memory for the producer (the reference leaves these steps to
  * separate torch operators, TernaryLLM/TernaryMLP.py:34 and the Hugging Face decoder layer it patches):

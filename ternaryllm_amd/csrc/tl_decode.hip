@@ -24,6 +24,17 @@ template <typename T> __device__ __forceinline__ T from_f(float v);
 template <> __device__ __forceinline__ float from_f<float>(float v) { return v; }
 template <> __device__ __forceinline__ __half from_f<__half>(float v) { return __float2half(v); }
 
+// One value of the rotate-half rotary embedding: x at dimension d, xp its partner half a head away, sgn = -1
+// below the middle and +1 above.  One explicit fma whose fp32 result is kept apart from the conversion that
+// follows it, so that every kernel rounds the same way: left to the compiler, some uses become an fma that
+// rounds straight to fp16 (v_fma_mixlo_f16) and others an fp32 fma plus a conversion, which differ on near-ties.
+__device__ __forceinline__ float rope_value(float x, float xp, float c, float s, float sgn)
+{
+    float r = fmaf(sgn * xp, s, x * c);
+    asm volatile("" : "+v"(r));
+    return r;
+}
+
 // qkv: [batch][3][heads][head_dim] (q, k, v of one token per batch row, as the fused projection
 // writes them).  Rotate-half form: out[d] = x[d] * cos[d] - x[d + h/2] * sin[d] for d < h/2,
 // out[d] = x[d] * cos[d] + x[d - h/2] * sin[d] above.  q goes to q_out [batch][heads][head_dim];
@@ -47,8 +58,8 @@ __global__ __launch_bounds__(256) void tl_rope_cache(const T* __restrict__ qkv, 
     const float c = to_f(cos_t[(size_t)pos * head_dim + d]), s = to_f(sin_t[(size_t)pos * head_dim + d]);
     const int partner = d < half ? d + half : d - half;
     const float sgn = d < half ? -1.0f : 1.0f;
-    const float q = to_f(base[d]) * c + sgn * to_f(base[partner]) * s;
-    const float k = to_f(base[plane + d]) * c + sgn * to_f(base[plane + partner]) * s;
+    const float q = rope_value(to_f(base[d]), to_f(base[partner]), c, s, sgn);
+    const float k = rope_value(to_f(base[plane + d]), to_f(base[plane + partner]), c, s, sgn);
     q_out[i] = from_f<T>(q);
     const size_t row = ((size_t)bh * max_seq + pos) * head_dim + d;
     k_cache[row] = from_f<T>(k);
@@ -66,11 +77,26 @@ __global__ __launch_bounds__(256) void tl_rope_cache(const T* __restrict__ qkv, 
 constexpr int kAttnThreads = 1024;
 constexpr int kAttnBatch = 4;  // rows of a row group whose loads are in flight together
 
+//
+// With `fresh` (q|k|v of the token as the projection wrote them, [batch][3][heads][HD], plus the rotary tables)
+// the kernel is also what tl_rope_cache does: q is rotated on the way in; the rotated key and the value of the
+// token stand in for cache row `pos`, which does not exist yet, and the workgroup whose rows include `pos` writes
+// them there for the steps to come.  Values are rounded to T where the separate kernels would store them, so
+// the result is theirs bit for bit.
+template <typename T>
+struct FreshToken {
+    const T* qkv;    // null: q and the cache are complete already
+    const T* cos_t;
+    const T* sin_t;
+    T* k_cache;      // the caches again, to write row `pos` through
+    T* v_cache;
+};
+
 template <typename T, int HD>
 __global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restrict__ q, const T* __restrict__ k_cache,
                                                                const T* __restrict__ v_cache, const long long* __restrict__ pos_p,
                                                                T* __restrict__ out, long long out_kld, int heads, long long max_seq,
-                                                               float scale, int splits, float* __restrict__ pieces)
+                                                               float scale, int splits, float* __restrict__ pieces, FreshToken<T> fresh)
 {
     constexpr int VE = 16 / (int)sizeof(T);   // values per 16-byte piece
     constexpr int CPR = HD / VE;              // lanes per cache row
@@ -81,7 +107,9 @@ __global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restri
     __shared__ float group_max[RG], group_sum[RG];
     const int tid = threadIdx.x;
     const long long bh = blockIdx.x;
-    long long n = *pos_p + 1;  // valid rows
+    const long long pos = *pos_p;
+    const bool has_fresh = fresh.qkv != nullptr && pos >= 0 && pos < max_seq;  // row `pos` comes from fresh.qkv
+    long long n = pos + 1;  // valid rows
     if (n > max_seq) n = max_seq;
     if (n < 1) n = 1;
     // With splits > 1 the rows of a (batch row, head) are shared out in contiguous pieces among gridDim.y
@@ -110,8 +138,47 @@ __global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restri
         }
     };
 
+    // A row group's rows come NB at a time; the first batch is asked for before q is ready.  (Asking for the next
+    // batch before the current one is worked on, two register sets alternating, was slower: 128 registers.)
+    auto load_batch = [&](long long j0, uint4 (&kk)[NB], uint4 (&vv)[NB]) {
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            const long long j = j0 + (long long)u * RG;
+            kk[u] = vv[u] = make_uint4(0u, 0u, 0u, 0u);
+            if (j < n && !(has_fresh && j == pos)) {  // rows past the end are not fetched, nor the row the token will take
+                kk[u] = *reinterpret_cast<const uint4*>(kc + (size_t)j * HD + c * VE);
+                vv[u] = *reinterpret_cast<const uint4*>(vc + (size_t)j * HD + c * VE);
+            }
+        }
+    };
+    uint4 ka[NB], va[NB];
+    const long long step = (long long)RG * NB;
+    long long j0 = lo + rg;
+    if (j0 < n) load_batch(j0, ka, va);
+
     float qv[VE];
-    {
+    uint4 k_new = make_uint4(0u, 0u, 0u, 0u), v_new = make_uint4(0u, 0u, 0u, 0u);  // this lane's piece of the token's key and value
+    if (fresh.qkv) {
+        static_assert((HD / 2) % VE == 0, "a 16-byte piece lies in one half of the head");
+        const T* base = fresh.qkv + ((size_t)(bh / heads) * 3 * heads + (size_t)(bh % heads)) * HD;
+        const size_t plane = (size_t)heads * HD;
+        const int d0 = c * VE, p0 = d0 < HD / 2 ? d0 + HD / 2 : d0 - HD / 2;
+        const float sgn = d0 < HD / 2 ? -1.0f : 1.0f;
+        const long long table_row = pos < 0 ? 0 : pos < max_seq ? pos : max_seq - 1;
+        float cs[VE], sn[VE], x[VE], xp[VE];
+        unpack(*reinterpret_cast<const uint4*>(fresh.cos_t + (size_t)table_row * HD + d0), cs);
+        unpack(*reinterpret_cast<const uint4*>(fresh.sin_t + (size_t)table_row * HD + d0), sn);
+        unpack(*reinterpret_cast<const uint4*>(base + d0), x);
+        unpack(*reinterpret_cast<const uint4*>(base + p0), xp);
+#pragma unroll
+        for (int e = 0; e < VE; ++e) qv[e] = to_f(from_f<T>(rope_value(x[e], xp[e], cs[e], sn[e], sgn))) * scale;
+        unpack(*reinterpret_cast<const uint4*>(base + plane + d0), x);
+        unpack(*reinterpret_cast<const uint4*>(base + plane + p0), xp);
+        T* kt = reinterpret_cast<T*>(&k_new);
+#pragma unroll
+        for (int e = 0; e < VE; ++e) kt[e] = from_f<T>(rope_value(x[e], xp[e], cs[e], sn[e], sgn));
+        v_new = *reinterpret_cast<const uint4*>(base + 2 * plane + d0);
+    } else {
         float f[VE];
         unpack(*reinterpret_cast<const uint4*>(q + (size_t)bh * HD + c * VE), f);
 #pragma unroll
@@ -121,29 +188,37 @@ __global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restri
     float acc[VE];
 #pragma unroll
     for (int e = 0; e < VE; ++e) acc[e] = 0.f;
-    for (long long j0 = lo + rg; j0 < n; j0 += (long long)RG * NB) {
-        uint4 kk[NB], vv[NB];
+    auto work = [&](long long j0, uint4 (&kk)[NB], uint4 (&vv)[NB]) {
+        if (has_fresh) {
 #pragma unroll
-        for (int u = 0; u < NB; ++u) {
-            const long long j = j0 + (long long)u * RG;
-            kk[u] = vv[u] = make_uint4(0u, 0u, 0u, 0u);
-            if (j < n) {  // rows past the end are not fetched
-                kk[u] = *reinterpret_cast<const uint4*>(kc + (size_t)j * HD + c * VE);
-                vv[u] = *reinterpret_cast<const uint4*>(vc + (size_t)j * HD + c * VE);
-            }
+            for (int u = 0; u < NB; ++u)
+                if (j0 + (long long)u * RG == pos && pos < n) {  // the token itself: not in the cache yet
+                    kk[u] = k_new;
+                    vv[u] = v_new;
+                }
         }
         float sc[NB];
-        float top = m;
 #pragma unroll
         for (int u = 0; u < NB; ++u) {
             float f[VE];
             unpack(kk[u], f);
-            float dot = 0.f;
+            sc[u] = 0.f;
 #pragma unroll
-            for (int e = 0; e < VE; ++e) dot = fmaf(f[e], qv[e], dot);
+            for (int e = 0; e < VE; ++e) sc[u] = fmaf(f[e], qv[e], sc[u]);
+        }
+        // the CPR lanes of a row add up their shares, the NB rows side by side: their exchanges do not wait for each other
 #pragma unroll
-            for (int off = CPR / 2; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
-            sc[u] = j0 + (long long)u * RG < n ? dot : -INFINITY;
+        for (int off = CPR / 2; off > 0; off >>= 1) {
+            float other[NB];
+#pragma unroll
+            for (int u = 0; u < NB; ++u) other[u] = __shfl_xor(sc[u], off, 64);
+#pragma unroll
+            for (int u = 0; u < NB; ++u) sc[u] += other[u];
+        }
+        float top = m;
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            if (j0 + (long long)u * RG >= n) sc[u] = -INFINITY;
             top = fmaxf(top, sc[u]);
         }
         const float keep = __expf(m - top);  // m == -inf on the first turn: exp(-inf) = 0, and l, acc are 0
@@ -160,6 +235,17 @@ __global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restri
             for (int e = 0; e < VE; ++e) acc[e] = fmaf(p, f[e], acc[e]);
         }
         m = top;
+    };
+    if (j0 < n) {
+        work(j0, ka, va);
+        for (j0 += step; j0 < n; j0 += step) {
+            load_batch(j0, ka, va);
+            work(j0, ka, va);
+        }
+    }
+    if (has_fresh && rg == 0 && pos >= lo && pos < n) {  // one workgroup per (batch row, head) has row `pos` among its rows
+        *reinterpret_cast<uint4*>(fresh.k_cache + ((size_t)bh * max_seq + pos) * HD + c * VE) = k_new;
+        *reinterpret_cast<uint4*>(fresh.v_cache + ((size_t)bh * max_seq + pos) * HD + c * VE) = v_new;
     }
 #pragma unroll
     for (int e = 0; e < VE; ++e) partial[rg][c * VE + e] = acc[e];
@@ -370,13 +456,22 @@ int launched()
     return TL_OK;
 }
 
+// q|k|v of the token and the rotary tables for the fused form of the attention (all null otherwise)
+struct FreshArgs {
+    const void* qkv;
+    const void* cos_table;
+    const void* sin_table;
+};
+
 template <typename T, int HD>
 int attn_launch(dim3 grid, size_t lds, hipStream_t st, const void* q, const void* k, const void* v, const long long* pos, void* out,
-                long long out_kld, int heads, long long max_seq, float scale, int splits, float* partial)
+                long long out_kld, int heads, long long max_seq, float scale, int splits, float* partial, const FreshArgs& f)
 {
     auto kernel = tl_decode_attn<T, HD>;
+    FreshToken<T> fresh{static_cast<const T*>(f.qkv), static_cast<const T*>(f.cos_table), static_cast<const T*>(f.sin_table),
+                        f.qkv ? static_cast<T*>(const_cast<void*>(k)) : nullptr, f.qkv ? static_cast<T*>(const_cast<void*>(v)) : nullptr};
     hipLaunchKernelGGL(kernel, dim3(grid.x, (unsigned)splits), dim3(kAttnThreads), lds, st, static_cast<const T*>(q), static_cast<const T*>(k),
-                       static_cast<const T*>(v), pos, static_cast<T*>(out), out_kld, heads, max_seq, scale, splits, partial);
+                       static_cast<const T*>(v), pos, static_cast<T*>(out), out_kld, heads, max_seq, scale, splits, partial, fresh);
     if (partial && out) {
         auto combine = tl_attn_combine<T, HD>;
         hipLaunchKernelGGL(combine, grid, dim3(HD), 0, st, partial, splits, static_cast<T*>(out), out_kld, heads);
@@ -386,12 +481,13 @@ int attn_launch(dim3 grid, size_t lds, hipStream_t st, const void* q, const void
 
 template <typename T>
 int attn_dispatch(int head_dim, dim3 grid, size_t lds, hipStream_t st, const void* q, const void* k, const void* v,
-                  const long long* pos, void* out, long long out_kld, int heads, long long max_seq, float scale, int splits, float* partial)
+                  const long long* pos, void* out, long long out_kld, int heads, long long max_seq, float scale, int splits, float* partial,
+                  const FreshArgs& f)
 {
     switch (head_dim) {
-        case 64: return attn_launch<T, 64>(grid, lds, st, q, k, v, pos, out, out_kld, heads, max_seq, scale, splits, partial);
-        case 128: return attn_launch<T, 128>(grid, lds, st, q, k, v, pos, out, out_kld, heads, max_seq, scale, splits, partial);
-        case 256: return attn_launch<T, 256>(grid, lds, st, q, k, v, pos, out, out_kld, heads, max_seq, scale, splits, partial);
+        case 64: return attn_launch<T, 64>(grid, lds, st, q, k, v, pos, out, out_kld, heads, max_seq, scale, splits, partial, f);
+        case 128: return attn_launch<T, 128>(grid, lds, st, q, k, v, pos, out, out_kld, heads, max_seq, scale, splits, partial, f);
+        case 256: return attn_launch<T, 256>(grid, lds, st, q, k, v, pos, out, out_kld, heads, max_seq, scale, splits, partial, f);
         default: return fail(TL_ERR_UNSUPPORTED, "head_dim=%d (64, 128 or 256 supported)", head_dim);
     }
 }
@@ -424,15 +520,19 @@ extern "C" int tl_rope_cache_update(const void* qkv, int dtype, int64_t batch, i
 namespace {
 constexpr int kAttnMaxSplits = 8;
 
-int attention(const void* q, const void* k_cache, const void* v_cache, int dtype, int64_t batch, int heads, int head_dim, int64_t max_seq,
-              const int64_t* pos_dev, void* out, int64_t out_kmajor_ld, int splits, void* workspace, int64_t workspace_bytes, void* stream)
+int attention(const void* q, const FreshArgs& fresh, const void* k_cache, const void* v_cache, int dtype, int64_t batch, int heads, int head_dim,
+              int64_t max_seq, const int64_t* pos_dev, void* out, int64_t out_kmajor_ld, int splits, void* workspace, int64_t workspace_bytes,
+              void* stream)
 {
     if (int rc = check_common(dtype, batch, heads, head_dim, max_seq, pos_dev)) return rc;
-    if (!q || !k_cache || !v_cache || (!out && !workspace)) return fail(TL_ERR_ARG, "device pointer is null");
+    if (!(q || fresh.qkv) || !k_cache || !v_cache || (!out && !workspace)) return fail(TL_ERR_ARG, "device pointer is null");
+    if (fresh.qkv && (!fresh.cos_table || !fresh.sin_table)) return fail(TL_ERR_ARG, "rotary table pointer is null");
     if (out_kmajor_ld && out_kmajor_ld < batch) return fail(TL_ERR_SHAPE, "out_kmajor_ld=%lld is less than the batch", (long long)out_kmajor_ld);
     const size_t lds = 0;
     if (reinterpret_cast<uintptr_t>(k_cache) % 16 || reinterpret_cast<uintptr_t>(v_cache) % 16 || reinterpret_cast<uintptr_t>(q) % 16)
         return fail(TL_ERR_ALIGN, "q and the caches must be 16-byte aligned");
+    if (reinterpret_cast<uintptr_t>(fresh.qkv) % 16 || reinterpret_cast<uintptr_t>(fresh.cos_table) % 16 || reinterpret_cast<uintptr_t>(fresh.sin_table) % 16)
+        return fail(TL_ERR_ALIGN, "qkv and the rotary tables must be 16-byte aligned");
     if (splits < 1 || splits > kAttnMaxSplits) return fail(TL_ERR_ARG, "splits=%d (1 to %d expected)", splits, kAttnMaxSplits);
     const bool leaves_pieces = splits > 1 || !out;
     if (leaves_pieces) {
@@ -447,9 +547,9 @@ int attention(const void* q, const void* k_cache, const void* v_cache, int dtype
     float* partial = leaves_pieces ? static_cast<float*>(workspace) : nullptr;
     int rc;
     if (dtype == TL_F16) rc = attn_dispatch<__half>(head_dim, grid, lds, st, q, k_cache, v_cache, pos, out, (long long)out_kmajor_ld, heads,
-                                                    (long long)max_seq, scale, splits, partial);
+                                                    (long long)max_seq, scale, splits, partial, fresh);
     else rc = attn_dispatch<float>(head_dim, grid, lds, st, q, k_cache, v_cache, pos, out, (long long)out_kmajor_ld, heads, (long long)max_seq,
-                                   scale, splits, partial);
+                                   scale, splits, partial, fresh);
     if (rc) return rc;
     return launched();
 }
@@ -458,15 +558,25 @@ int attention(const void* q, const void* k_cache, const void* v_cache, int dtype
 extern "C" int tl_decode_attention(const void* q, const void* k_cache, const void* v_cache, int dtype, int64_t batch, int heads,
                                    int head_dim, int64_t max_seq, const int64_t* pos_dev, void* out, int64_t out_kmajor_ld, void* stream)
 {
-    return attention(q, k_cache, v_cache, dtype, batch, heads, head_dim, max_seq, pos_dev, out, out_kmajor_ld, 1, nullptr, 0, stream);
+    return attention(q, FreshArgs{nullptr, nullptr, nullptr}, k_cache, v_cache, dtype, batch, heads, head_dim, max_seq, pos_dev, out, out_kmajor_ld,
+                     1, nullptr, 0, stream);
 }
 
 extern "C" int tl_decode_attention_split(const void* q, const void* k_cache, const void* v_cache, int dtype, int64_t batch, int heads,
                                          int head_dim, int64_t max_seq, const int64_t* pos_dev, void* out, int64_t out_kmajor_ld,
                                          int splits, void* workspace, int64_t workspace_bytes, void* stream)
 {
-    return attention(q, k_cache, v_cache, dtype, batch, heads, head_dim, max_seq, pos_dev, out, out_kmajor_ld, splits, workspace,
-                     workspace_bytes, stream);
+    return attention(q, FreshArgs{nullptr, nullptr, nullptr}, k_cache, v_cache, dtype, batch, heads, head_dim, max_seq, pos_dev, out, out_kmajor_ld,
+                     splits, workspace, workspace_bytes, stream);
+}
+
+extern "C" int tl_decode_attention_rope(const void* qkv, const void* cos_table, const void* sin_table, void* k_cache, void* v_cache, int dtype,
+                                        int64_t batch, int heads, int head_dim, int64_t max_seq, const int64_t* pos_dev, void* out,
+                                        int64_t out_kmajor_ld, int splits, void* workspace, int64_t workspace_bytes, void* stream)
+{
+    if (!qkv) return fail(TL_ERR_ARG, "device pointer is null");
+    return attention(nullptr, FreshArgs{qkv, cos_table, sin_table}, k_cache, v_cache, dtype, batch, heads, head_dim, max_seq, pos_dev, out,
+                     out_kmajor_ld, splits, workspace, workspace_bytes, stream);
 }
 
 extern "C" int tl_add_rmsnorm(const void* x, const void* y, const void* weight, int dtype, int64_t rows, int width, float eps,

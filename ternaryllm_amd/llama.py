@@ -126,6 +126,8 @@ class TernaryLlamaDecoder(nn.Module):
         self.fused_decode = all(m._header.tile_rows % 8 == 0 and m.in_features % 8 == 0
                                 for layer in self.layers for m in (layer.qkv_proj, layer.o_proj, layer.gate_up_proj, layer.down_proj)) and \
             self.lm_head._header.tile_rows % 8 == 0 and H % 8 == 0
+        # the attention kernel rotates q and k and writes the token's cache row itself; False runs the separate kernel first
+        self.fused_rope = True
         self._layer_index = {id(layer): i for i, layer in enumerate(self.layers)}
 
     # -- pieces ------------------------------------------------------------------------------
@@ -205,33 +207,31 @@ class TernaryLlamaDecoder(nn.Module):
         return self.lm_head(self.norm(x[:, 0]))
 
     def _decode_step_native(self, token, pos):
-        """The decode step with rotary embedding + cache update and the attention over the cache as one
-        library kernel each (activations stay [B, hidden] throughout)."""
+        """The decode step with rotary embedding, cache update and the attention over the cache as one
+        library kernel (activations stay [B, hidden] throughout)."""
         c = self.config
         x = self.embed_tokens[token]
         B = x.shape[0]
-        q = torch.empty((B, c.num_attention_heads, c.head_dim), dtype=x.dtype, device=x.device)
         eps = c.rms_norm_eps
         # 5 to 48 rows: the products read a K-major image, so whatever feeds one writes it in that layout
         # (its transpose as a view) and no re-layout pass runs in front of the products
         if B == 1 and self.fused_decode:
-            return self._decode_step_fused(x, pos, q)
+            return self._decode_step_fused(x, pos)
         km = 5 <= B <= 48 and c.hidden_size != B and c.intermediate_size != B
         _, h = ops.add_rmsnorm(x, None, self.layers[0].input_layernorm.weight, eps, kmajor=km)
         for li, layer in enumerate(self.layers):
             qkv = layer.qkv_proj(h)
-            ops.rope_cache_update(qkv, self.rope_cos, self.rope_sin, pos, q, self._cache[li, 0], self._cache[li, 1])
-            a = ops.decode_attention(q, self._cache[li, 0], self._cache[li, 1], pos, kmajor=km)
+            a = self._attend(qkv, self._cache[li, 0], self._cache[li, 1], pos, km)
             x, h = ops.add_rmsnorm(x, layer.o_proj(a), layer.post_attention_layernorm.weight, eps, kmajor=km)
             y = layer.down_proj(ops.silu_mul(layer.gate_up_proj(h), kmajor=km))
             nxt = self.layers[li + 1].input_layernorm.weight if li + 1 < len(self.layers) else self.norm.weight
             x, h = ops.add_rmsnorm(x, y, nxt, eps, kmajor=km)  # the residual add, and the norm the next layer (or the head) starts with
         return self.lm_head(h)
 
-    def _decode_step_fused(self, x, pos, q):
+    def _decode_step_fused(self, x, pos):
         """One row: the residual add + RMSNorm in front of the q|k|v and gate|up products and the SiLU gate in
-        front of the down projection are computed inside those products' kernels (tl_spmv_fused), six launches
-        per layer instead of nine.  The attention shares the cache rows of a head out among several workgroups
+        front of the down projection are computed inside those products' kernels (tl_spmv_fused), and the
+        rotary embedding and the cache update inside the attention's: five launches per layer instead of nine.  The attention shares the cache rows of a head out among several workgroups
         (32 heads alone would leave seven compute units in eight idle) and leaves its result in pieces that the
         output projection folds while it stages its row (tl_spmv_attn_combine)."""
         eps = self.config.rms_norm_eps
@@ -239,13 +239,25 @@ class TernaryLlamaDecoder(nn.Module):
         for layer in self.layers:
             qkv, x = ops.spmv_fused(layer.qkv_proj.device_weight(), "add_rmsnorm", x, y, layer.input_layernorm.weight, eps,
                                     layer.qkv_proj.w_scale, want_sum=True)
-            ops.rope_cache_update(qkv, self.rope_cos, self.rope_sin, pos, q, self._cache_of(layer, 0), self._cache_of(layer, 1))
-            pieces = ops.decode_attention_pieces(q, self._cache_of(layer, 0), self._cache_of(layer, 1), pos)
+            pieces = self._attend(qkv, self._cache_of(layer, 0), self._cache_of(layer, 1), pos, False, pieces=True)
             o = ops.spmv_attn_combine(layer.o_proj.device_weight(), pieces, self.config.head_dim, x.dtype, layer.o_proj.w_scale)
             gu, x = ops.spmv_fused(layer.gate_up_proj.device_weight(), "add_rmsnorm", x, o, layer.post_attention_layernorm.weight, eps,
                                    layer.gate_up_proj.w_scale, want_sum=True)
             y = ops.spmv_fused(layer.down_proj.device_weight(), "silu_gate", gu, scale=layer.down_proj.w_scale)
         return ops.spmv_fused(self.lm_head.device_weight(), "add_rmsnorm", x, y, self.norm.weight, eps, self.lm_head.w_scale)
+
+    def _attend(self, qkv, k_cache, v_cache, pos, kmajor, pieces=False):
+        """Rotary embedding, cache update and attention for the token whose q | k | v the projection just wrote: one
+        launch, or (fused_rope False) the rotary + cache kernel followed by the attention."""
+        q, fresh = None, (qkv, self.rope_cos, self.rope_sin)
+        if not self.fused_rope:
+            c = self.config
+            q = torch.empty((qkv.shape[0], c.num_attention_heads, c.head_dim), dtype=qkv.dtype, device=qkv.device)
+            ops.rope_cache_update(qkv, self.rope_cos, self.rope_sin, pos, q, k_cache, v_cache)
+            fresh = None
+        if pieces:
+            return ops.decode_attention_pieces(q, k_cache, v_cache, pos, fresh=fresh)
+        return ops.decode_attention(q, k_cache, v_cache, pos, kmajor=kmajor, fresh=fresh)
 
     def _cache_of(self, layer, which):
         return self._cache[self._layer_index[id(layer)], which]

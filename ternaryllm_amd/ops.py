@@ -281,13 +281,49 @@ def _attention_splits(B, heads, device):
     return max(1, min(_ATTN_MAX_SPLITS, units // max(1, 2 * B * heads)))
 
 
-def decode_attention(q, k_cache, v_cache, pos, out=None, kmajor=False, splits=None):
+def _check_fresh(fresh, k_cache):
+    """fresh = (qkv, cos_table, sin_table) of rope_cache_update, for the attention calls that do its work too."""
+    B, heads, max_seq, hd = k_cache.shape
+    qkv, cos_table, sin_table = fresh
+    for t in (qkv, cos_table, sin_table):
+        if not t.is_contiguous() or t.dtype != k_cache.dtype or t.device != k_cache.device:
+            raise ValueError("tensors must be contiguous, of one dtype, on one device")
+    if qkv.numel() != B * 3 * heads * hd:
+        raise ValueError("qkv must hold q | k | v of one token per batch row")
+    if cos_table.shape != (max_seq, hd) or sin_table.shape != (max_seq, hd):
+        raise ValueError("rotary tables must be [max_seq, head_dim]")
+    return qkv, cos_table, sin_table
+
+
+def _attention_call(q, fresh, k_cache, v_cache, pos, out_ptr, ld, splits, ws_ptr, ws_bytes):
+    B, heads, max_seq, hd = k_cache.shape
+    L = _lib.lib()
+    with torch.cuda.device(k_cache.device):
+        if fresh is None:
+            rc = L.tl_decode_attention_split(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), _code(q.dtype, "q"), B, heads, hd,
+                                             max_seq, pos.data_ptr(), out_ptr, ld, splits, ws_ptr, ws_bytes, _stream_ptr(q.device))
+        else:
+            qkv, cos_table, sin_table = fresh
+            rc = L.tl_decode_attention_rope(qkv.data_ptr(), cos_table.data_ptr(), sin_table.data_ptr(), k_cache.data_ptr(),
+                                            v_cache.data_ptr(), _code(qkv.dtype, "qkv"), B, heads, hd, max_seq, pos.data_ptr(), out_ptr, ld,
+                                            splits, ws_ptr, ws_bytes, _stream_ptr(qkv.device))
+    _lib.check(rc)
+
+
+def decode_attention(q, k_cache, v_cache, pos, out=None, kmajor=False, splits=None, fresh=None):
     """Attention of one query per (batch row, head) over cache rows [0, pos].  q: [B, heads, head_dim];
     caches: [B, heads, max_seq, head_dim]; pos: one-element int64 device tensor.  Returns [B, heads * head_dim],
     or with kmajor its transpose [heads * head_dim, B] as a view of a K-major image (for spmm's x_layout=1).
     splits: workgroups that share the cache rows of a (batch row, head) (1 to 8; default: by the size of
-    the step, see _attention_splits)."""
+    the step, see _attention_splits).
+    fresh=(qkv, cos_table, sin_table) with q=None: the same kernel also does what rope_cache_update does --
+    rotates q and k of the token and writes its k, v into cache row `pos` -- in the one launch."""
     B, heads, max_seq, hd = k_cache.shape
+    if (q is None) == (fresh is None):
+        raise ValueError("give q, or fresh=(qkv, cos_table, sin_table) with q=None")
+    if fresh is not None:
+        fresh = _check_fresh(fresh, k_cache)
+        q = fresh[0]   # stands for dtype, device and the element count below
     ld = 0
     if kmajor:
         if out is not None:
@@ -299,7 +335,7 @@ def decode_attention(q, k_cache, v_cache, pos, out=None, kmajor=False, splits=No
     for t in (q, k_cache, v_cache, out):
         if not t.is_contiguous() or t.dtype != q.dtype or t.device != q.device:
             raise ValueError("tensors must be contiguous, of one dtype, on one device")
-    if q.numel() != B * heads * hd or out.numel() != max(B, ld) * heads * hd or v_cache.shape != k_cache.shape:
+    if q.numel() != B * heads * hd * (3 if fresh is not None else 1) or out.numel() != max(B, ld) * heads * hd or v_cache.shape != k_cache.shape:
         raise ValueError("shapes of q, out and the caches do not agree")
     if pos.dtype != torch.int64 or pos.numel() != 1 or pos.device != q.device:
         raise ValueError("pos must be a one-element int64 tensor on the same device")
@@ -315,34 +351,31 @@ def decode_attention(q, k_cache, v_cache, pos, out=None, kmajor=False, splits=No
             ws = torch.empty(need, dtype=torch.uint8, device=q.device)
             _attn_workspaces[key] = ws
         ws_ptr, ws_bytes = ws.data_ptr(), ws.numel()
-    with torch.cuda.device(q.device):
-        rc = _lib.lib().tl_decode_attention_split(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), _code(q.dtype, "q"), B, heads, hd,
-                                                  max_seq, pos.data_ptr(), out.data_ptr(), ld, splits, ws_ptr, ws_bytes,
-                                                  _stream_ptr(q.device))
-    _lib.check(rc)
+    _attention_call(None if fresh is not None else q, fresh, k_cache, v_cache, pos, out.data_ptr(), ld, splits, ws_ptr, ws_bytes)
     return out[:, :B] if kmajor else out
 
 
-def decode_attention_pieces(q, k_cache, v_cache, pos, splits=None):
+def decode_attention_pieces(q, k_cache, v_cache, pos, splits=None, fresh=None):
     """The attention of decode_attention left unfolded: float32 [B * heads, splits, head_dim + 4], per piece
     head_dim unnormalised sums, the piece's maximum and its sum of exponentials (two unused floats behind them).
-    spmv_attn_combine folds them inside the output projection (batch 1)."""
+    spmv_attn_combine folds them inside the output projection (batch 1).  fresh: as in decode_attention."""
     B, heads, max_seq, hd = k_cache.shape
+    if (q is None) == (fresh is None):
+        raise ValueError("give q, or fresh=(qkv, cos_table, sin_table) with q=None")
+    if fresh is not None:
+        fresh = _check_fresh(fresh, k_cache)
+        q = fresh[0]
     for t in (q, k_cache, v_cache):
         if not t.is_contiguous() or t.dtype != q.dtype or t.device != q.device:
             raise ValueError("tensors must be contiguous, of one dtype, on one device")
-    if q.numel() != B * heads * hd or v_cache.shape != k_cache.shape:
+    if q.numel() != B * heads * hd * (3 if fresh is not None else 1) or v_cache.shape != k_cache.shape:
         raise ValueError("shapes of q and the caches do not agree")
     if pos.dtype != torch.int64 or pos.numel() != 1 or pos.device != q.device:
         raise ValueError("pos must be a one-element int64 tensor on the same device")
     if splits is None:
         splits = _attention_splits(B, heads, q.device)
     pieces = torch.empty((B * heads, splits, hd + 4), dtype=torch.float32, device=q.device)
-    with torch.cuda.device(q.device):
-        rc = _lib.lib().tl_decode_attention_split(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), _code(q.dtype, "q"), B, heads, hd,
-                                                  max_seq, pos.data_ptr(), None, 0, splits, pieces.data_ptr(), pieces.numel() * 4,
-                                                  _stream_ptr(q.device))
-    _lib.check(rc)
+    _attention_call(None if fresh is not None else q, fresh, k_cache, v_cache, pos, None, 0, splits, pieces.data_ptr(), pieces.numel() * 4)
     return pieces
 
 

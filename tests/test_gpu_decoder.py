@@ -266,6 +266,52 @@ def test_split_attention_and_its_fold_inside_the_output_projection(cuda, oracle)
         ops.decode_attention(q, kc, vc, p, splits=9)
 
 
+def test_attention_that_rotates_and_updates_the_cache_itself(cuda):
+    """tl_decode_attention_rope against tl_rope_cache_update followed by tl_decode_attention_split: the output (row-major,
+    K-major, and left in pieces) and both caches bit for bit -- first, middle and last cache row, one and several
+    workgroups per head, and a position past the cache, which writes nothing."""
+    from ternaryllm_amd import ops
+    g = torch.Generator().manual_seed(29)
+    for dtype in (torch.float16, torch.float32):
+        for B, H, hd, S in ((1, 32, 128, 300), (3, 5, 64, 150), (2, 2, 256, 70)):
+            inv = 1.0 / (10000 ** (torch.arange(0, hd, 2).double() / hd))
+            ang = torch.arange(S).double()[:, None] * inv[None, :]
+            cos = torch.cat([ang.cos(), ang.cos()], 1).to(dtype).to(cuda)
+            sin = torch.cat([ang.sin(), ang.sin()], 1).to(dtype).to(cuda)
+            kc0 = torch.randn((B, H, S, hd), generator=g).to(dtype).to(cuda)
+            vc0 = torch.randn((B, H, S, hd), generator=g).to(dtype).to(cuda)
+            for pos in (0, 1, S // 2, S - 1, S):
+                qkv = torch.randn((B, 3 * H * hd), generator=g).to(dtype).to(cuda)
+                p = torch.tensor([pos], dtype=torch.long, device=cuda)
+                for splits in (1, 3, 8):
+                    kc1, vc1, kc2, vc2 = kc0.clone(), vc0.clone(), kc0.clone(), vc0.clone()
+                    if pos < S:
+                        # the row the token will take holds something else: it must not be read
+                        kc1[:, :, pos], kc2[:, :, pos] = 7.0, 7.0
+                        vc1[:, :, pos], vc2[:, :, pos] = -3.0, -3.0
+                    q = torch.zeros((B, H, hd), dtype=dtype, device=cuda)
+                    ops.rope_cache_update(qkv, cos, sin, p, q, kc1, vc1)
+                    fused = ops.decode_attention(None, kc2, vc2, p, splits=splits, fresh=(qkv, cos, sin))
+                    assert torch.equal(kc1, kc2) and torch.equal(vc1, vc2), (dtype, pos, splits)
+                    if pos < S:
+                        assert torch.equal(fused, ops.decode_attention(q, kc1, vc1, p, splits=splits)), (dtype, B, pos, splits)
+                        assert not torch.equal(kc2[:, :, pos], kc0[:, :, pos])
+                    else:
+                        assert torch.equal(kc2, kc0) and torch.isfinite(fused).all()
+                    kc3, vc3 = kc0.clone(), vc0.clone()
+                    assert torch.equal(ops.decode_attention(None, kc3, vc3, p, kmajor=True, splits=splits, fresh=(qkv, cos, sin)).t(), fused)
+                    assert torch.equal(kc3, kc2)
+                    if pos < S:
+                        kc4, vc4 = kc0.clone(), vc0.clone()
+                        pieces = ops.decode_attention_pieces(None, kc4, vc4, p, splits=splits, fresh=(qkv, cos, sin))
+                        assert torch.equal(pieces[..., :hd + 2], ops.decode_attention_pieces(q, kc1, vc1, p, splits=splits)[..., :hd + 2])
+                        assert torch.equal(kc4, kc2) and torch.equal(vc4, vc2)
+    with pytest.raises(ValueError, match="q, or fresh"):
+        ops.decode_attention(q, kc1, vc1, p, fresh=(qkv, cos, sin))
+    with pytest.raises(ValueError, match="rotary tables"):
+        ops.decode_attention(None, kc1, vc1, p, fresh=(qkv, cos[:-1], sin))
+
+
 def test_add_rmsnorm_and_silu_mul(cuda):
     from ternaryllm_amd import ops
     g = torch.Generator().manual_seed(10)
