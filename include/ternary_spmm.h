@@ -337,6 +337,12 @@ int tl_spmv_fused(const tl_layout_header* header, const void* blob_dev, int prod
                   const void* in, const void* in2, const void* norm_weight, float eps, void* sum_out, int x_dtype,
                   void* Y, int y_dtype, const void* scale, int scale_dtype, void* stream);
 
+/* tl_spmv_fused with the epilogue of tl_spmm_gated: the weight's columns are (gate, up) pairs and Y holds the N / 2
+ * values silu(y[2j]) * y[2j + 1].  Same arguments otherwise. */
+int tl_spmv_fused_gated(const tl_layout_header* header, const void* blob_dev, int producer,
+                        const void* in, const void* in2, const void* norm_weight, float eps, void* sum_out, int x_dtype,
+                        void* Y, int y_dtype, const void* scale, int scale_dtype, void* stream);
+
 /* Y[N] = (x * W) * scale for the single row x = the attention output that the pieces of
  * tl_decode_attention_split (out == NULL) add up to, batch 1: the output projection of a decode step
  * (o_proj over the eager softmax(QK^T)V, TernaryLLM/TernaryAttn.py:100-116) without a launch for the fold.
@@ -359,6 +365,26 @@ int tl_add_rmsnorm(const void* x, const void* y, const void* weight, int dtype, 
  * gate of LlamaTernaryMLP (TernaryLLM/TernaryMLP.py:33-35) on a side-by-side gate | up product.
  * out_kmajor_ld: 0, or the leading dimension (>= rows) of a K-major out [width][ld]. */
 int tl_silu_mul(const void* gate_up, int dtype, int64_t rows, int width, void* out, int64_t out_kmajor_ld, void* stream);
+
+/* tl_silu_mul for a gate | up product whose columns are PAIRS -- column 2j the gate and column 2j + 1 the up
+ * projection of output j (a weight packed that way lets a product's kernel finish both halves of a pair in one
+ * workgroup, see tl_spmm_gated): out[r][j] = silu(gate_up[r][2j]) * gate_up[r][2j + 1].  Same reference lines. */
+int tl_silu_mul_pairs(const void* gate_up, int dtype, int64_t rows, int width, void* out, int64_t out_kmajor_ld, void* stream);
+
+/* tl_spmm with the SiLU gate of LlamaTernaryMLP (TernaryLLM/TernaryMLP.py:33-35) in the epilogue, for a weight
+ * whose columns are (gate, up) pairs as above: Y[m][j] = silu(y[m][2j]) * y[m][2j + 1] with y = (X * W) * scale,
+ * N / 2 outputs per row -- what tl_spmm followed by tl_silu_mul_pairs computes, bit for bit (y and the SiLU are
+ * rounded to y_dtype where those would store them), without the launch and the trip through memory.
+ *   y_layout   TL_X_ROW_MAJOR: Y [M][ldy], ldy >= N / 2;  TL_X_K_MAJOR: Y [N / 2][ldy], ldy >= M, rows M..ldy-1
+ *              zeroed -- the image tl_spmm multiplies 5 to 48 rows from (9 to 16 rows only)
+ * The kernels with this epilogue are those of M = 1 (a contiguous aligned row) and of 9 to 16 fp16 rows with
+ * N >= 64 * compute units; any other call returns TL_ERR_UNSUPPORTED and the two separate calls do the work
+ * (for more than 48 rows and separate gate and up weights there is tl_mlp_gate_up). */
+int tl_spmm_gated(const tl_layout_header* header, const void* blob_dev,
+                  const void* X, int x_dtype, int x_layout, int64_t ldx, int64_t M,
+                  void* Y, int y_dtype, int64_t ldy, int y_layout,
+                  const void* scale, int scale_dtype,
+                  void* workspace, int64_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

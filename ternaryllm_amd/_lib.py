@@ -16,6 +16,7 @@ TL_X_ROW_MAJOR, TL_X_K_MAJOR = 0, 1
 TL_ACT_SILU_GATE = 1
 TL_PRODUCER_SILU_GATE, TL_PRODUCER_ADD_RMSNORM = 1, 2
 TL_LAYOUT_MAGIC = 0x35474C54
+TL_ERR_UNSUPPORTED = -5
 
 ERROR_NAMES = {
     -1: "TL_ERR_ARG", -2: "TL_ERR_SHAPE", -3: "TL_ERR_DTYPE", -4: "TL_ERR_ALIGN", -5: "TL_ERR_UNSUPPORTED",
@@ -69,6 +70,8 @@ SIGNATURES = {
     "tl_spmm": (_INT, [_HDRP, _VP, _VP, _INT, _INT, _I64, _I64, _VP, _INT, _I64, _VP, _INT, _VP, _I64, _VP]),
     "tl_spmm_noalloc": (_INT, [_HDRP, _VP, _VP, _INT, _INT, _I64, _I64, _VP, _INT, _I64, _VP, _INT, _VP]),
     "tl_spmv_fused": (_INT, [_HDRP, _VP, _INT, _VP, _VP, _VP, ctypes.c_float, _VP, _INT, _VP, _INT, _VP, _INT, _VP]),
+    "tl_spmv_fused_gated": (_INT, [_HDRP, _VP, _INT, _VP, _VP, _VP, ctypes.c_float, _VP, _INT, _VP, _INT, _VP, _INT, _VP]),
+    "tl_spmm_gated": (_INT, [_HDRP, _VP, _VP, _INT, _INT, _I64, _I64, _VP, _INT, _I64, _INT, _VP, _INT, _VP, _I64, _VP]),
     "tl_mlp_gate_up": (_INT, [_HDRP, _VP, _HDRP, _VP, _VP, _INT, _INT, _I64, _I64, _VP, _INT, _I64, _VP, _VP, _INT, _INT,
                               _VP, _I64, _VP]),
     "tl_spmm_time": (_INT, [_HDRP, _VP, _VP, _INT, _INT, _I64, _I64, _VP, _INT, _I64, _VP, _INT, _VP, _I64, _VP, _INT,
@@ -80,6 +83,7 @@ SIGNATURES = {
     "tl_spmv_attn_combine": (_INT, [_HDRP, _VP, _VP, _INT, _INT, _INT, _VP, _INT, _VP, _INT, _VP]),
     "tl_add_rmsnorm": (_INT, [_VP, _VP, _VP, _INT, _I64, _INT, ctypes.c_float, _VP, _VP, _I64, _VP]),
     "tl_silu_mul": (_INT, [_VP, _INT, _I64, _INT, _VP, _I64, _VP]),
+    "tl_silu_mul_pairs": (_INT, [_VP, _INT, _I64, _INT, _VP, _I64, _VP]),
 }
 
 _lib = None

@@ -404,7 +404,8 @@ __global__ __launch_bounds__(512) void tl_add_rmsnorm_vec(const T* __restrict__ 
 // With out_kld the result goes to a K-major image [width][out_kld]; threads then walk the image in its
 // own order (rows of one column side by side, stores contiguous), and the columns past `rows` are zeroed.
 template <typename T>
-__global__ __launch_bounds__(256) void tl_silu_mul_k(const T* __restrict__ gu, T* __restrict__ out, long long out_kld, long long rows, int width)
+__global__ __launch_bounds__(256) void tl_silu_mul_k(const T* __restrict__ gu, T* __restrict__ out, long long out_kld, long long rows, int width,
+                                                     int pairs)
 {
     const long long i = blockIdx.x * 256ll + threadIdx.x;
     long long r;
@@ -422,7 +423,9 @@ __global__ __launch_bounds__(256) void tl_silu_mul_k(const T* __restrict__ gu, T
         r = i / width;
         c = (int)(i - r * width);
     }
-    const float g = to_f(gu[(size_t)r * 2 * width + c]), u = to_f(gu[(size_t)r * 2 * width + width + c]);
+    // gate and up of column c: side by side halves of the row, or (pairs) neighbours 2c, 2c + 1
+    const T* row = gu + (size_t)r * 2 * width;
+    const float g = to_f(pairs ? row[2 * c] : row[c]), u = to_f(pairs ? row[2 * c + 1] : row[width + c]);
     out[i] = from_f<T>(to_f(from_f<T>(g / (1.0f + __expf(-g)))) * u);  // the SiLU is rounded to T before the product, as two separate operators would
 }
 
@@ -616,7 +619,8 @@ extern "C" int tl_add_rmsnorm(const void* x, const void* y, const void* weight, 
     return launched();
 }
 
-extern "C" int tl_silu_mul(const void* gate_up, int dtype, int64_t rows, int width, void* out, int64_t out_kmajor_ld, void* stream)
+namespace {
+int silu_mul_call(const void* gate_up, int dtype, int64_t rows, int width, void* out, int64_t out_kmajor_ld, void* stream, int pairs)
 {
     if (dtype != TL_F16 && dtype != TL_F32) return fail(TL_ERR_DTYPE, "dtype code %d unknown", dtype);
     if (!gate_up || !out) return fail(TL_ERR_ARG, "device pointer is null");
@@ -626,9 +630,20 @@ extern "C" int tl_silu_mul(const void* gate_up, int dtype, int64_t rows, int wid
     const unsigned blocks = (unsigned)ceil_div((out_kmajor_ld ? out_kmajor_ld : rows) * width, 256);
     if (dtype == TL_F16)
         hipLaunchKernelGGL(tl_silu_mul_k<__half>, dim3(blocks), dim3(256), 0, st, static_cast<const __half*>(gate_up), static_cast<__half*>(out),
-                           (long long)out_kmajor_ld, (long long)rows, width);
+                           (long long)out_kmajor_ld, (long long)rows, width, pairs);
     else
         hipLaunchKernelGGL(tl_silu_mul_k<float>, dim3(blocks), dim3(256), 0, st, static_cast<const float*>(gate_up), static_cast<float*>(out),
-                           (long long)out_kmajor_ld, (long long)rows, width);
+                           (long long)out_kmajor_ld, (long long)rows, width, pairs);
     return launched();
+}
+}  // namespace
+
+extern "C" int tl_silu_mul(const void* gate_up, int dtype, int64_t rows, int width, void* out, int64_t out_kmajor_ld, void* stream)
+{
+    return silu_mul_call(gate_up, dtype, rows, width, out, out_kmajor_ld, stream, 0);
+}
+
+extern "C" int tl_silu_mul_pairs(const void* gate_up, int dtype, int64_t rows, int width, void* out, int64_t out_kmajor_ld, void* stream)
+{
+    return silu_mul_call(gate_up, dtype, rows, width, out, out_kmajor_ld, stream, 1);
 }

@@ -80,6 +80,9 @@ struct KernelArgs {
     float eps;
     int pro_splits;       // attention-combine producer: pieces per head, and the head width
     int pro_hd;
+    // gated epilogue: columns 2j, 2j + 1 of the weight are gate and up column j; Y[j] = silu(y[2j]) * y[2j + 1] (N / 2 outputs)
+    int gated;
+    long long y_kld;      // gated epilogue of the 16-row kernel: 0, or the leading dimension of a K-major output [N / 2][y_kld]
 };
 
 __device__ __forceinline__ float load_scale(const void* scale, int is_f16, int n)
@@ -88,13 +91,30 @@ __device__ __forceinline__ float load_scale(const void* scale, int is_f16, int n
     return is_f16 ? __half2float(static_cast<const __half*>(scale)[n]) : static_cast<const float*>(scale)[n];
 }
 
+// An fp32 value on its way to an fp16 result is kept apart from the conversion: left to the compiler, a product
+// that feeds the conversion becomes one instruction that rounds the exact product straight to fp16
+// (v_fma_mixlo_f16) in one kernel and a multiply plus a conversion in another, and the two differ on near-ties.
+// Every kernel of this file converts the rounded fp32 value.
+__device__ __forceinline__ float settled(float v)
+{
+    asm volatile("" : "+v"(v));
+    return v;
+}
+
 __device__ __forceinline__ void store_out(void* Y, int is_f16, long long off, float v)
 {
-    if (is_f16) static_cast<__half*>(Y)[off] = __float2half(v);
+    if (is_f16) static_cast<__half*>(Y)[off] = __float2half(settled(v));
     else static_cast<float*>(Y)[off] = v;
 }
 
 __device__ __forceinline__ float silu(float g) { return g / (1.0f + __expf(-g)); }
+
+// v as a stored output of the call's type would read back
+__device__ __forceinline__ float as_output(float v, int is_f16) { return is_f16 ? __half2float(__float2half(settled(v))) : v; }
+
+// silu(g) * u for a product's outputs g, u (already rounded to the output type), with the roundings of the separate
+// operator: the SiLU is rounded to the type before the product.
+__device__ __forceinline__ float gate_pair(float g, float u, int is_f16) { return as_output(g / (1.0f + __expf(-g)), is_f16) * u; }
 
 __device__ __forceinline__ int run_pos_dwords(uint32_t d) { return (int)(((d & 0xffu) + 3u) >> 2); }
 __device__ __forceinline__ int run_neg_dwords(uint32_t d) { return (int)((((d >> 8) & 0xffu) + 3u) >> 2); }
@@ -801,9 +821,24 @@ __global__ __launch_bounds__(kBlockThreads) void tl_spmm_octet(KernelArgs a)
             s1.x += o1.x; s1.y += o1.y; s1.z += o1.z; s1.w += o1.w;
         }
         const int n = (nb0 + blk) * TL_BLOCK_COLUMNS + c16;
-        if (blk < bs && n < a.N) {
-            const float sc = load_scale(a.w0.scale, a.scale_f16, n);
-            const float out[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+        const bool real = blk < bs && n < a.N;
+        const float sc = real ? load_scale(a.w0.scale, a.scale_f16, n) : 0.f;
+        const float out[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+        if (a.gated) {
+            // gate and up column of a pair sit two lanes apart (same rows): the even column's lane writes the eight products
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float y = real ? as_output(out[j] * sc, a.y_f16) : 0.f;
+                const float up = __shfl_xor(y, 2, 64);
+                const int m = m0 + q * 8 + j;
+                if (!(c16 & 1) && real && n + 1 < a.N) {
+                    if (m < a.M) store_out(a.Y, a.y_f16, a.y_kld ? (long long)(n / 2) * a.y_kld + m : (long long)m * a.ldy + n / 2, gate_pair(y, up, a.y_f16));
+                    else if (m < a.y_kld) store_out(a.Y, a.y_f16, (long long)(n / 2) * a.y_kld + m, 0.f);  // the image's padding rows
+                }
+            }
+            return;
+        }
+        if (real) {
 #pragma unroll
             for (int j = 0; j < 8; ++j)
                 if (m0 + q * 8 + j < a.M) store_out(a.Y, a.y_f16, (long long)(m0 + q * 8 + j) * a.ldy + n, out[j] * sc);
@@ -1045,6 +1080,16 @@ __global__ __launch_bounds__(NT) void tl_spmv_direct(KernelArgs a)
     for (int off = 32; off > 0; off >>= 1)
         if (off < LPC) acc[0] += __shfl_xor(acc[0], off, 64);
     const int n = nb * TL_BLOCK_COLUMNS + c16;
+    if (a.gated) {
+        // the 16 column sums of the block meet in LDS (no wave may still be gathering from it), eight products go out
+        __syncthreads();
+        float* sums = reinterpret_cast<float*>(lds);
+        if (lig == 0) sums[c16] = n < a.N ? as_output(acc[0] * load_scale(a.w0.scale, a.scale_f16, n), a.y_f16) : 0.f;
+        __syncthreads();
+        if (tid < TL_BLOCK_COLUMNS / 2 && nb * TL_BLOCK_COLUMNS + 2 * tid + 1 < a.N)
+            store_out(a.Y, a.y_f16, nb * (TL_BLOCK_COLUMNS / 2) + tid, gate_pair(sums[2 * tid], sums[2 * tid + 1], a.y_f16));
+        return;
+    }
     if (lig == 0 && n < a.N) store_out(a.Y, a.y_f16, n, acc[0] * load_scale(a.w0.scale, a.scale_f16, n));
 }
 
@@ -1161,6 +1206,12 @@ __global__ __launch_bounds__(NT) void tl_spmv_tiles(KernelArgs a)
 #pragma unroll
         for (int w = 0; w < W; ++w) sum += red[w * TL_BLOCK_COLUMNS + tid];
         const int n = nb * TL_BLOCK_COLUMNS + tid;
+        if (a.gated) {
+            const float y = n < a.N ? as_output(sum * load_scale(a.w0.scale, a.scale_f16, n), a.y_f16) : 0.f;
+            const float up = __shfl_xor(y, 1, 64);  // the odd neighbour's
+            if (!(tid & 1) && n + 1 < a.N) store_out(a.Y, a.y_f16, n / 2, gate_pair(y, up, a.y_f16));
+            return;
+        }
         if (n < a.N) store_out(a.Y, a.y_f16, n, sum * load_scale(a.w0.scale, a.scale_f16, n));
     }
 }
@@ -2076,9 +2127,10 @@ int launch_small(KernelArgs a, const tl_layout_header* h, int x_dtype, void* wor
         aligned = true;
     }
     if (mt >= 8) {
-        if (mt == 8) return a.x_f16 ? launch_quad_kernel<8, true>(a, h, st) : launch_quad_kernel<8, false>(a, h, st);
         // fp16, 16 rows: eight rows per lane and two blocks per workgroup where the workgroups still fill the chip
-        const bool octet = a.x_f16 && knob(TL_OCTET, ceil_div(a.NB, 2) * ceil_div(a.M, 16) >= 2 * (int64_t)compute_units() ? 1 : 0) != 0;
+        const bool octet = mt == 16 && a.x_f16 && knob(TL_OCTET, ceil_div(a.NB, 2) * ceil_div(a.M, 16) >= 2 * (int64_t)compute_units() ? 1 : 0) != 0;
+        if (a.gated && !octet) return fail(TL_ERR_UNSUPPORTED, "no gated epilogue in the kernel for M=%d, N=%d (tl_spmm, then tl_silu_mul_pairs)", a.M, a.N);
+        if (mt == 8) return a.x_f16 ? launch_quad_kernel<8, true>(a, h, st) : launch_quad_kernel<8, false>(a, h, st);
         if (octet) return launch_octet_kernel(a, h, st);
         if (wide) return a.x_f16 ? launch_quad_kernel<16, true, 1024>(a, h, st) : launch_quad_kernel<16, false, 1024>(a, h, st);
         return a.x_f16 ? launch_quad_kernel<16, true>(a, h, st) : launch_quad_kernel<16, false>(a, h, st);
@@ -2087,6 +2139,7 @@ int launch_small(KernelArgs a, const tl_layout_header* h, int x_dtype, void* wor
     if (mt == 1 && a.x_sk == 1 && reinterpret_cast<uintptr_t>(a.X) % 16 == 0 && h->tile_rows % (16 / es) == 0 && a.K % (16 / es) == 0 &&
         knob(TL_SPMV_DIRECT, 1))
         return a.x_f16 ? launch_spmv_direct<true>(a, h, st) : launch_spmv_direct<false>(a, h, st);
+    if (a.gated) return fail(TL_ERR_UNSUPPORTED, "no gated epilogue in the kernel for M=%d and this activation layout (tl_spmm, then tl_silu_mul_pairs)", a.M);
     // Column blocks per workgroup.  A compute unit works through ceil(workgroups / 256) workgroups of
     // `set` blocks each: the narrowest set that keeps that product smallest.
     int set = 1;
@@ -2287,16 +2340,28 @@ extern "C" int tl_spmm_workspace(const tl_layout_header* header, int64_t M, int 
     return TL_OK;
 }
 
-extern "C" int tl_spmm(const tl_layout_header* header, const void* blob_dev,
-                       const void* X, int x_dtype, int x_layout, int64_t ldx, int64_t M,
-                       void* Y, int y_dtype, int64_t ldy,
-                       const void* scale, int scale_dtype,
-                       void* workspace, int64_t workspace_bytes, void* stream)
+namespace {
+// tl_spmm, or (y_layout >= 0) tl_spmm_gated with that output layout
+int spmm_call(const tl_layout_header* header, const void* blob_dev, const void* X, int x_dtype, int x_layout, int64_t ldx, int64_t M,
+              void* Y, int y_dtype, int64_t ldy, int y_layout, const void* scale, int scale_dtype, void* workspace, int64_t workspace_bytes,
+              void* stream)
 {
     if (int rc = check_header(header)) return rc;
-    if (int rc = check_io(blob_dev, X, Y, x_dtype, x_layout, ldx, M, y_dtype, ldy, scale, scale_dtype, header)) return rc;
+    const bool gated = y_layout >= 0;
+    // the checks of tl_spmm, with the width of the gated output where ldy is compared
+    if (int rc = check_io(blob_dev, X, Y, x_dtype, x_layout, ldx, M, y_dtype, gated ? (int64_t)header->columns : ldy, scale, scale_dtype, header)) return rc;
+    if (gated) {
+        if (y_layout != TL_X_ROW_MAJOR && y_layout != TL_X_K_MAJOR) return fail(TL_ERR_ARG, "y_layout=%d unknown", y_layout);
+        if (header->columns % 2) return fail(TL_ERR_SHAPE, "N=%u: gate and up columns come in pairs", header->columns);
+        const int64_t min_ldy = y_layout == TL_X_K_MAJOR ? M : (int64_t)header->columns / 2;
+        if (ldy < min_ldy) return fail(TL_ERR_SHAPE, "ldy=%lld smaller than %lld", (long long)ldy, (long long)min_ldy);
+        if (M > kSmallMaxM) return fail(TL_ERR_UNSUPPORTED, "no gated epilogue for M=%lld (tl_spmm, then tl_silu_mul_pairs; or tl_mlp_gate_up)", (long long)M);
+        if (y_layout == TL_X_K_MAJOR && (M <= 8 || M > 16)) return fail(TL_ERR_UNSUPPORTED, "a K-major gated output is written for 9 to 16 rows");
+    }
     KernelArgs a;
     std::memset(&a, 0, sizeof(a));
+    a.gated = gated;
+    if (gated && y_layout == TL_X_K_MAJOR) a.y_kld = ldy;
     a.w0 = weight_ptrs(header, blob_dev, scale);
     a.X = X; a.Y = Y;
     a.ldx = ldx; a.ldy = ldy;
@@ -2309,6 +2374,25 @@ extern "C" int tl_spmm(const tl_layout_header* header, const void* blob_dev,
                                : launch_rows(a, x_dtype, workspace, workspace_bytes, false, st);
     if (rc) return rc;
     return finish_launch();
+}
+}  // namespace
+
+extern "C" int tl_spmm(const tl_layout_header* header, const void* blob_dev,
+                       const void* X, int x_dtype, int x_layout, int64_t ldx, int64_t M,
+                       void* Y, int y_dtype, int64_t ldy,
+                       const void* scale, int scale_dtype,
+                       void* workspace, int64_t workspace_bytes, void* stream)
+{
+    return spmm_call(header, blob_dev, X, x_dtype, x_layout, ldx, M, Y, y_dtype, ldy, -1, scale, scale_dtype, workspace, workspace_bytes, stream);
+}
+
+extern "C" int tl_spmm_gated(const tl_layout_header* header, const void* blob_dev,
+                             const void* X, int x_dtype, int x_layout, int64_t ldx, int64_t M,
+                             void* Y, int y_dtype, int64_t ldy, int y_layout,
+                             const void* scale, int scale_dtype,
+                             void* workspace, int64_t workspace_bytes, void* stream)
+{
+    return spmm_call(header, blob_dev, X, x_dtype, x_layout, ldx, M, Y, y_dtype, ldy, y_layout, scale, scale_dtype, workspace, workspace_bytes, stream);
 }
 
 // Scratch of tl_spmm_noalloc: device memory that belongs to the library's code object, one copy per GPU,
@@ -2357,11 +2441,13 @@ extern "C" int tl_spmm_noalloc(const tl_layout_header* header, const void* blob_
     return tl_spmm(header, blob_dev, X, x_dtype, x_layout, ldx, M, Y, y_dtype, ldy, scale, scale_dtype, ws, need, stream);
 }
 
-extern "C" int tl_spmv_fused(const tl_layout_header* header, const void* blob_dev, int producer,
-                             const void* in, const void* in2, const void* norm_weight, float eps, void* sum_out, int x_dtype,
-                             void* Y, int y_dtype, const void* scale, int scale_dtype, void* stream)
+namespace {
+int spmv_fused_call(const tl_layout_header* header, const void* blob_dev, int producer,
+                    const void* in, const void* in2, const void* norm_weight, float eps, void* sum_out, int x_dtype,
+                    void* Y, int y_dtype, const void* scale, int scale_dtype, void* stream, bool gated)
 {
     if (int rc = check_header(header)) return rc;
+    if (gated && header->columns % 2) return fail(TL_ERR_SHAPE, "N=%u: gate and up columns come in pairs", header->columns);
     if (int rc = check_dtype(x_dtype, "x")) return rc;
     if (int rc = check_dtype(y_dtype, "y")) return rc;
     if (scale)
@@ -2388,6 +2474,7 @@ extern "C" int tl_spmv_fused(const tl_layout_header* header, const void* blob_de
     a.NB = (int)header->n_blocks;
     a.x_f16 = x_dtype == TL_F16; a.y_f16 = y_dtype == TL_F16; a.scale_f16 = scale_dtype == TL_F16;
     a.one = 1.0f;
+    a.gated = gated;
     hipStream_t st = static_cast<hipStream_t>(stream);
     int rc;
     if (producer == TL_PRODUCER_SILU_GATE)
@@ -2396,6 +2483,21 @@ extern "C" int tl_spmv_fused(const tl_layout_header* header, const void* blob_de
         rc = a.x_f16 ? launch_spmv_direct<true, kProAddNorm>(a, header, st) : launch_spmv_direct<false, kProAddNorm>(a, header, st);
     if (rc) return rc;
     return finish_launch();
+}
+}  // namespace
+
+extern "C" int tl_spmv_fused(const tl_layout_header* header, const void* blob_dev, int producer,
+                             const void* in, const void* in2, const void* norm_weight, float eps, void* sum_out, int x_dtype,
+                             void* Y, int y_dtype, const void* scale, int scale_dtype, void* stream)
+{
+    return spmv_fused_call(header, blob_dev, producer, in, in2, norm_weight, eps, sum_out, x_dtype, Y, y_dtype, scale, scale_dtype, stream, false);
+}
+
+extern "C" int tl_spmv_fused_gated(const tl_layout_header* header, const void* blob_dev, int producer,
+                                   const void* in, const void* in2, const void* norm_weight, float eps, void* sum_out, int x_dtype,
+                                   void* Y, int y_dtype, const void* scale, int scale_dtype, void* stream)
+{
+    return spmv_fused_call(header, blob_dev, producer, in, in2, norm_weight, eps, sum_out, x_dtype, Y, y_dtype, scale, scale_dtype, stream, true);
 }
 
 extern "C" int tl_spmv_attn_combine(const tl_layout_header* header, const void* blob_dev, const void* pieces, int splits, int head_dim,

@@ -20,7 +20,7 @@ import numpy as np
 import torch
 from torch import nn
 
-from . import ops, packing
+from . import _lib, ops, packing
 from .linear import TernaryLinear
 
 
@@ -138,9 +138,8 @@ class TernaryLlamaDecoder(nn.Module):
         return x * cos + rot * sin
 
     def _mlp(self, layer, x2):
-        gu = layer.gate_up_proj(x2)
-        inter = self.config.intermediate_size
-        return layer.down_proj(torch.nn.functional.silu(gu[:, :inter]) * gu[:, inter:])
+        gu = layer.gate_up_proj(x2)   # columns 2j, 2j + 1: gate and up of output j
+        return layer.down_proj(torch.nn.functional.silu(gu[:, 0::2]) * gu[:, 1::2])
 
     def allocate_cache(self, batch):
         c = self.config
@@ -223,7 +222,10 @@ class TernaryLlamaDecoder(nn.Module):
             qkv = layer.qkv_proj(h)
             a = self._attend(qkv, self._cache[li, 0], self._cache[li, 1], pos, km)
             x, h = ops.add_rmsnorm(x, layer.o_proj(a), layer.post_attention_layernorm.weight, eps, kmajor=km)
-            y = layer.down_proj(ops.silu_mul(layer.gate_up_proj(h), kmajor=km))
+            # the SiLU gate in the epilogue of the gate | up product where its kernel has one (else a launch of its own)
+            gated = ops.spmm_gated(layer.gate_up_proj.device_weight(), h, layer.gate_up_proj.w_scale,
+                                   x_layout=_lib.TL_X_K_MAJOR if km else _lib.TL_X_ROW_MAJOR, kmajor=km)
+            y = layer.down_proj(gated)
             nxt = self.layers[li + 1].input_layernorm.weight if li + 1 < len(self.layers) else self.norm.weight
             x, h = ops.add_rmsnorm(x, y, nxt, eps, kmajor=km)  # the residual add, and the norm the next layer (or the head) starts with
         return self.lm_head(h)
@@ -241,9 +243,9 @@ class TernaryLlamaDecoder(nn.Module):
                                     layer.qkv_proj.w_scale, want_sum=True)
             pieces = self._attend(qkv, self._cache_of(layer, 0), self._cache_of(layer, 1), pos, False, pieces=True)
             o = ops.spmv_attn_combine(layer.o_proj.device_weight(), pieces, self.config.head_dim, x.dtype, layer.o_proj.w_scale)
-            gu, x = ops.spmv_fused(layer.gate_up_proj.device_weight(), "add_rmsnorm", x, o, layer.post_attention_layernorm.weight, eps,
-                                   layer.gate_up_proj.w_scale, want_sum=True)
-            y = ops.spmv_fused(layer.down_proj.device_weight(), "silu_gate", gu, scale=layer.down_proj.w_scale)
+            gated, x = ops.spmv_fused(layer.gate_up_proj.device_weight(), "add_rmsnorm", x, o, layer.post_attention_layernorm.weight, eps,
+                                      layer.gate_up_proj.w_scale, want_sum=True, gated=True)
+            y = ops.spmm(layer.down_proj.device_weight(), gated, layer.down_proj.w_scale)
         return ops.spmv_fused(self.lm_head.device_weight(), "add_rmsnorm", x, y, self.norm.weight, eps, self.lm_head.w_scale)
 
     def _attend(self, qkv, k_cache, v_cache, pos, kmajor, pieces=False):

@@ -140,6 +140,37 @@ def spmm(weight, x, scale=None, out_dtype=None, x_layout=_lib.TL_X_ROW_MAJOR, ou
     return y
 
 
+def spmm_gated(weight, x, scale=None, x_layout=_lib.TL_X_ROW_MAJOR, kmajor=False):
+    """h[M, N / 2] with h[:, j] = silu(y[:, 2j]) * y[:, 2j + 1], y = (x @ W) * scale, for a gate | up weight whose
+    columns are (gate, up) pairs.  One launch (tl_spmm_gated) where the shape's kernel has the epilogue -- one
+    aligned row, or 9 to 16 fp16 rows and a wide N -- else the product followed by silu_mul(pairs=True); the result
+    is the same bit for bit.  With kmajor the transpose [N / 2, M] is returned, a view of a K-major image."""
+    if x.device != weight.device:
+        raise RuntimeError(f"x is on {x.device}, the weight on {weight.device}")
+    if weight.columns % 2:
+        raise ValueError("gate and up columns come in pairs: N must be even")
+    x_code = _code(x.dtype, "x")
+    xg, M, ldx = _x_geometry(x, weight.inners, x_layout)
+    half = weight.columns // 2
+    fused = M == 1 or (9 <= M <= 16 and x.dtype == torch.float16)
+    if fused and not (kmajor and M == 1):
+        if kmajor:
+            out, ld = _kmajor_image(M, half, x)
+        else:
+            out, ld = torch.empty((M, half), dtype=x.dtype, device=x.device), half
+        sc, s_code = _scale_args(scale, weight.columns, x.device)
+        ws, ws_bytes = _workspace(weight.header, M, x_code, x_layout, x.device)
+        with torch.cuda.device(x.device):
+            rc = _lib.lib().tl_spmm_gated(ctypes.byref(weight.header), weight.blob.data_ptr(), xg.data_ptr(), x_code, x_layout, ldx, M,
+                                          out.data_ptr(), x_code, ld, _lib.TL_X_K_MAJOR if kmajor else _lib.TL_X_ROW_MAJOR,
+                                          sc.data_ptr() if sc is not None else None, s_code,
+                                          ws.data_ptr() if ws is not None else None, ws_bytes, _stream_ptr(x.device))
+        if rc != _lib.TL_ERR_UNSUPPORTED:
+            _lib.check(rc)
+            return out[:, :M] if kmajor else out
+    return silu_mul(spmm(weight, x, scale, x_layout=x_layout), kmajor=kmajor, pairs=True)
+
+
 def mlp_gate_up(gate, up, x, gate_scale=None, up_scale=None, out_dtype=None):
     """h[M, N] = silu((x @ Wg) * sg) * ((x @ Wu) * su) in one pass over x (M > 48), else two products."""
     if gate.columns != up.columns or gate.inners != up.inners:
@@ -168,13 +199,17 @@ def mlp_gate_up(gate, up, x, gate_scale=None, up_scale=None, out_dtype=None):
     return h
 
 
-def spmv_fused(weight, producer, inp, inp2=None, norm_weight=None, eps=0.0, scale=None, out_dtype=None, want_sum=False):
+def spmv_fused(weight, producer, inp, inp2=None, norm_weight=None, eps=0.0, scale=None, out_dtype=None, want_sum=False, gated=False):
     """y[1, N] = (x @ W) * scale for one activation row x that the call produces itself (tl_spmv_fused):
     producer "silu_gate": x = silu(inp[:K]) * inp[K:] for a gate | up row inp of 2K values;
     producer "add_rmsnorm": s = inp + inp2 (inp2 may be None), x = rmsnorm(s) * norm_weight; with want_sum the
     call also returns s (a new tensor).  Returns y, or (y, s).  Raises RuntimeError (TL_ERR_UNSUPPORTED) where the
-    fused kernel does not apply (K or the tile height not whole 16-byte pieces); callers then use the separate operators."""
+    fused kernel does not apply (K or the tile height not whole 16-byte pieces); callers then use the separate operators.
+    gated: the weight's columns are (gate, up) pairs and y is [1, N / 2] with y[j] = silu(y'[2j]) * y'[2j + 1]
+    (tl_spmv_fused_gated)."""
     K, N = weight.inners, weight.columns
+    if gated and N % 2:
+        raise ValueError("gate and up columns come in pairs: N must be even")
     code = {"silu_gate": _lib.TL_PRODUCER_SILU_GATE, "add_rmsnorm": _lib.TL_PRODUCER_ADD_RMSNORM}[producer]
     x_code = _code(inp.dtype, "inp")
     need = 2 * K if producer == "silu_gate" else K
@@ -185,11 +220,12 @@ def spmv_fused(weight, producer, inp, inp2=None, norm_weight=None, eps=0.0, scal
     if producer == "add_rmsnorm" and norm_weight is None:
         raise ValueError("add_rmsnorm needs norm_weight")
     out_dtype = out_dtype or inp.dtype
-    y = torch.empty((1, N), dtype=out_dtype, device=inp.device)
+    y = torch.empty((1, N // 2 if gated else N), dtype=out_dtype, device=inp.device)
     s_out = torch.empty(K, dtype=inp.dtype, device=inp.device).view(inp.shape) if (want_sum and producer == "add_rmsnorm") else None
     scale, s_code = _scale_args(scale, N, inp.device)
+    call = _lib.lib().tl_spmv_fused_gated if gated else _lib.lib().tl_spmv_fused
     with torch.cuda.device(inp.device):
-        rc = _lib.lib().tl_spmv_fused(ctypes.byref(weight.header), weight.blob.data_ptr(), code, inp.data_ptr(),
+        rc = call(ctypes.byref(weight.header), weight.blob.data_ptr(), code, inp.data_ptr(),
                                       inp2.data_ptr() if inp2 is not None else None,
                                       norm_weight.data_ptr() if norm_weight is not None else None, float(eps),
                                       s_out.data_ptr() if s_out is not None else None, x_code, y.data_ptr(), _code(out_dtype, "out_dtype"),
@@ -399,14 +435,16 @@ def add_rmsnorm(x, y, weight, eps, kmajor=False):
     return x_out, (h[:, :x.shape[0]] if kmajor else h)
 
 
-def silu_mul(gate_up, kmajor=False):
+def silu_mul(gate_up, kmajor=False, pairs=False):
     """silu(gate_up[:, :w]) * gate_up[:, w:] for a contiguous [rows, 2 * w] tensor; with kmajor the transpose
-    [w, rows] of that, a view of a K-major image (for spmm's x_layout=1)."""
+    [w, rows] of that, a view of a K-major image (for spmm's x_layout=1).  pairs: gate and up of output j are
+    columns 2j and 2j + 1 instead of j and w + j."""
     if gate_up.dim() != 2 or not gate_up.is_contiguous() or gate_up.shape[1] % 2:
         raise ValueError("gate_up must be a contiguous [rows, 2 * width] tensor")
     rows, w = gate_up.shape[0], gate_up.shape[1] // 2
     out, ld = _kmajor_image(rows, w, gate_up) if kmajor else (torch.empty((rows, w), dtype=gate_up.dtype, device=gate_up.device), 0)
     with torch.cuda.device(gate_up.device):
-        rc = _lib.lib().tl_silu_mul(gate_up.data_ptr(), _code(gate_up.dtype, "gate_up"), rows, w, out.data_ptr(), ld, _stream_ptr(gate_up.device))
+        call = _lib.lib().tl_silu_mul_pairs if pairs else _lib.lib().tl_silu_mul
+        rc = call(gate_up.data_ptr(), _code(gate_up.dtype, "gate_up"), rows, w, out.data_ptr(), ld, _stream_ptr(gate_up.device))
     _lib.check(rc)
     return out[:, :rows] if kmajor else out

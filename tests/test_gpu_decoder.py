@@ -45,9 +45,8 @@ def _reference_logits(model, tokens):
         a = (att @ v).transpose(1, 2).reshape(B, S, H)
         x = x + lin(layer.o_proj, a)
         h = norm(layer.post_attention_layernorm, x)
-        gu = lin(layer.gate_up_proj, h)
-        inter = c.intermediate_size
-        x = x + lin(layer.down_proj, torch.nn.functional.silu(gu[..., :inter]) * gu[..., inter:])
+        gu = lin(layer.gate_up_proj, h)   # columns 2j, 2j + 1: gate and up of output j
+        x = x + lin(layer.down_proj, torch.nn.functional.silu(gu[..., 0::2]) * gu[..., 1::2])
     return lin(model.lm_head, norm(model.norm, x))
 
 
@@ -375,6 +374,80 @@ def test_fused_producers_of_the_single_row_product(cuda, oracle, dtype, tol):
     with pytest.raises(RuntimeError, match="UNSUPPORTED"):   # a tile height that is not whole 16-byte pieces: the separate kernels are the way then
         odd = ops.DeviceWeight(PackedWeight.from_dense(ternary_weight(1000, 40, 0.7, 3), tile_rows=250), cuda)
         ops.spmv_fused(odd, "silu_gate", torch.zeros(2000, dtype=dtype, device=cuda))
+
+
+def test_silu_gate_in_the_epilogue_of_the_gate_up_product(cuda):
+    """tl_spmm_gated / tl_spmv_fused_gated on a weight whose columns are (gate, up) pairs against the product followed
+    by tl_silu_mul_pairs: bit for bit -- one row (both single-row kernels, with and without a producer), 9 to 16 fp16
+    rows on a wide output (row-major and as a K-major image with zeroed padding rows), and the shapes without the
+    epilogue, which take the two launches."""
+    import ctypes
+    from tests.util import knobs, ternary_weight
+    from ternaryllm_amd import _lib, ops
+    from ternaryllm_amd.packing import PackedWeight
+    g = torch.Generator().manual_seed(31)
+    L = _lib.lib()
+
+    def fused_rc(dw, x, M, layout=0):
+        """status of the one-launch call by itself (ops.spmm_gated falls back silently)"""
+        out = torch.empty((M, dw.columns // 2), dtype=x.dtype, device=cuda)
+        ws = torch.empty(1 << 22, dtype=torch.uint8, device=cuda)
+        return L.tl_spmm_gated(ctypes.byref(dw.header), dw.blob.data_ptr(), x.data_ptr(), ops._code(x.dtype, "x"), 0, dw.inners, M,
+                               out.data_ptr(), ops._code(x.dtype, "x"), dw.columns // 2 if layout == 0 else 16, layout, None, 0,
+                               ws.data_ptr(), ws.numel(), None)
+
+    # the separate operator on pairs
+    gu = torch.randn((5, 600), generator=g).half().to(cuda)
+    ref = (torch.nn.functional.silu(gu[:, 0::2].float()).half().float() * gu[:, 1::2].float()).half()
+    assert torch.equal(ops.silu_mul(gu, pairs=True), ref)
+    assert torch.equal(ops.silu_mul(gu, kmajor=True, pairs=True).t(), ref)
+    for dtype in (torch.float16, torch.float32):
+        for K, N in ((4096, 544), (11008, 96), (1000, 40)):   # the tile-per-wave kernel; a block too tall for it at 512 threads; ragged
+            w = ternary_weight(K, N, 0.7, K + N)
+            dw = ops.DeviceWeight(PackedWeight.from_dense(w), cuda)
+            sc = (0.5 + torch.rand(N, generator=g)).to(dtype).to(cuda)
+            x = torch.randn((1, K), generator=g).to(dtype).to(cuda)
+            want = ops.silu_mul(ops.spmm(dw, x, sc), pairs=True)
+            assert fused_rc(dw, x, 1) == 0
+            for setting in ({}, {"TL_SPMV_TILES": "0"}):
+                with knobs(**setting):
+                    assert torch.equal(ops.spmm_gated(dw, x, sc), ops.silu_mul(ops.spmm(dw, x, sc), pairs=True)), (dtype, K, N, setting)
+            # with the residual add + RMSNorm in front
+            y = torch.randn(K, generator=g).to(dtype).to(cuda)
+            nw = (1 + 0.1 * torch.randn(K, generator=g)).to(dtype).to(cuda)
+            plain, s1 = ops.spmv_fused(dw, "add_rmsnorm", x[0], y, nw, 1e-5, sc, want_sum=True)
+            gated, s2 = ops.spmv_fused(dw, "add_rmsnorm", x[0], y, nw, 1e-5, sc, want_sum=True, gated=True)
+            assert torch.equal(s1, s2) and gated.shape == (1, N // 2)
+            assert torch.equal(gated, ops.silu_mul(plain, pairs=True))
+    # 9 to 16 fp16 rows, an output wide enough for the eight-rows-per-lane kernel
+    units = torch.cuda.get_device_properties(cuda).multi_processor_count
+    K, N = 520, 64 * units + 48
+    w = ternary_weight(K, N, 0.8, 5)
+    dw = ops.DeviceWeight(PackedWeight.from_dense(w), cuda)
+    sc = (0.5 + torch.rand(N, generator=g)).half().to(cuda)
+    for M in (16, 9, 13):
+        x = torch.randn((M, K), generator=g).half().to(cuda)
+        want = ops.silu_mul(ops.spmm(dw, x, sc), pairs=True)
+        assert fused_rc(dw, x, M) == 0 and fused_rc(dw, x, M, layout=1) == 0
+        assert torch.equal(ops.spmm_gated(dw, x, sc), want), M
+        image = ops.spmm_gated(dw, x, sc, kmajor=True)
+        assert torch.equal(image.t(), want)
+        assert image.stride(0) == 16 and not image.as_strided((N // 2, 16), (16, 1))[:, M:].any()   # the padding rows of the image
+        xk, _ = ops._kmajor_image(M, K, x)
+        xk[:, :M] = x.t()
+        assert torch.equal(ops.spmm_gated(dw, xk[:, :M], sc, x_layout=1), want)
+    # shapes whose kernels have no such epilogue: same result from two launches
+    x32 = torch.randn((16, K), generator=g).to(cuda)
+    assert fused_rc(dw, x32, 16) == _lib.TL_ERR_UNSUPPORTED
+    for x in (torch.randn((5, K), generator=g).half().to(cuda), torch.randn((3, K), generator=g).half().to(cuda),
+              torch.randn((60, K), generator=g).half().to(cuda), x32):
+        assert fused_rc(dw, x, x.shape[0]) == _lib.TL_ERR_UNSUPPORTED
+        assert torch.equal(ops.spmm_gated(dw, x, sc.to(x.dtype)), ops.silu_mul(ops.spmm(dw, x, sc.to(x.dtype)), pairs=True))
+    narrow = ops.DeviceWeight(PackedWeight.from_dense(ternary_weight(K, 96, 0.8, 6)), cuda)
+    assert fused_rc(narrow, torch.zeros((16, K), dtype=torch.float16, device=cuda), 16) == _lib.TL_ERR_UNSUPPORTED
+    odd = ops.DeviceWeight(PackedWeight.from_dense(ternary_weight(K, 33, 0.8, 7)), cuda)
+    with pytest.raises(ValueError, match="pairs"):
+        ops.spmm_gated(odd, torch.zeros((1, K), dtype=torch.float16, device=cuda))
 
 
 def test_fused_single_row_step_equals_the_unfused_one(tiny, cuda):
