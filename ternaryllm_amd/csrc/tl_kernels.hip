@@ -826,14 +826,28 @@ __global__ __launch_bounds__(kBlockThreads) void tl_spmm_octet(KernelArgs a)
         const float out[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
         if (a.gated) {
             // gate and up column of a pair sit two lanes apart (same rows): the even column's lane writes the eight products
+            float h[8];
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const float y = real ? as_output(out[j] * sc, a.y_f16) : 0.f;
                 const float up = __shfl_xor(y, 2, 64);
-                const int m = m0 + q * 8 + j;
-                if (!(c16 & 1) && real && n + 1 < a.N) {
-                    if (m < a.M) store_out(a.Y, a.y_f16, a.y_kld ? (long long)(n / 2) * a.y_kld + m : (long long)m * a.ldy + n / 2, gate_pair(y, up, a.y_f16));
-                    else if (m < a.y_kld) store_out(a.Y, a.y_f16, (long long)(n / 2) * a.y_kld + m, 0.f);  // the image's padding rows
+                h[j] = m0 + q * 8 + j < a.M ? gate_pair(y, up, a.y_f16) : 0.f;  // zeros in the padding rows of a K-major image
+            }
+            if (!(c16 & 1) && real && n + 1 < a.N) {
+                const int m = m0 + q * 8;
+                if (a.y_kld && a.y_f16 && a.y_kld % 8 == 0 && m + 8 <= a.y_kld && reinterpret_cast<uintptr_t>(a.Y) % 16 == 0) {
+                    // eight neighbouring rows of one column of the image: one 16-byte store
+                    u32x4 packed;
+                    __half* p = reinterpret_cast<__half*>(&packed);
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) p[j] = __float2half(settled(h[j]));
+                    *reinterpret_cast<u32x4*>(static_cast<__half*>(a.Y) + (long long)(n / 2) * a.y_kld + m) = packed;
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        if (m + j < a.M) store_out(a.Y, a.y_f16, a.y_kld ? (long long)(n / 2) * a.y_kld + m + j : (long long)(m + j) * a.ldy + n / 2, h[j]);
+                        else if (m + j < a.y_kld) store_out(a.Y, a.y_f16, (long long)(n / 2) * a.y_kld + m + j, 0.f);
+                    }
                 }
             }
             return;
