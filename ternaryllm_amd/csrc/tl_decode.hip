@@ -165,19 +165,24 @@ __global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restri
         const int d0 = c * VE, p0 = d0 < HD / 2 ? d0 + HD / 2 : d0 - HD / 2;
         const float sgn = d0 < HD / 2 ? -1.0f : 1.0f;
         const long long table_row = pos < 0 ? 0 : pos < max_seq ? pos : max_seq - 1;
+        // all seven pieces are asked for before the first is used: one trip to memory, not three
+        const uint4 cos_piece = *reinterpret_cast<const uint4*>(fresh.cos_t + (size_t)table_row * HD + d0);
+        const uint4 sin_piece = *reinterpret_cast<const uint4*>(fresh.sin_t + (size_t)table_row * HD + d0);
+        const uint4 q_piece = *reinterpret_cast<const uint4*>(base + d0), q_partner = *reinterpret_cast<const uint4*>(base + p0);
+        const uint4 k_piece = *reinterpret_cast<const uint4*>(base + plane + d0), k_partner = *reinterpret_cast<const uint4*>(base + plane + p0);
+        v_new = *reinterpret_cast<const uint4*>(base + 2 * plane + d0);
         float cs[VE], sn[VE], x[VE], xp[VE];
-        unpack(*reinterpret_cast<const uint4*>(fresh.cos_t + (size_t)table_row * HD + d0), cs);
-        unpack(*reinterpret_cast<const uint4*>(fresh.sin_t + (size_t)table_row * HD + d0), sn);
-        unpack(*reinterpret_cast<const uint4*>(base + d0), x);
-        unpack(*reinterpret_cast<const uint4*>(base + p0), xp);
+        unpack(cos_piece, cs);
+        unpack(sin_piece, sn);
+        unpack(q_piece, x);
+        unpack(q_partner, xp);
 #pragma unroll
         for (int e = 0; e < VE; ++e) qv[e] = to_f(from_f<T>(rope_value(x[e], xp[e], cs[e], sn[e], sgn))) * scale;
-        unpack(*reinterpret_cast<const uint4*>(base + plane + d0), x);
-        unpack(*reinterpret_cast<const uint4*>(base + plane + p0), xp);
+        unpack(k_piece, x);
+        unpack(k_partner, xp);
         T* kt = reinterpret_cast<T*>(&k_new);
 #pragma unroll
         for (int e = 0; e < VE; ++e) kt[e] = from_f<T>(rope_value(x[e], xp[e], cs[e], sn[e], sgn));
-        v_new = *reinterpret_cast<const uint4*>(base + 2 * plane + d0);
     } else {
         float f[VE];
         unpack(*reinterpret_cast<const uint4*>(q + (size_t)bh * HD + c * VE), f);
