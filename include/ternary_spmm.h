@@ -51,8 +51,10 @@ extern "C" {
 #define TL_X_K_MAJOR 1   /* X is [K][ldx], M contiguous (what the reference kernel itself reads, */
                          /* ter_spmm_kernel.cuh:173)                                            */
 
+#define TL_PRODUCER_NONE 0        /* x = in                                                    */
 #define TL_PRODUCER_SILU_GATE 1   /* tl_spmv_fused: x = silu(in[:K]) * in[K:]                  */
 #define TL_PRODUCER_ADD_RMSNORM 2 /* tl_spmv_fused: x = RMSNorm(in + in2) * norm_weight        */
+#define TL_PRODUCER_RMSNORM 3     /* tl_spmv_fused: x = RMSNorm(in) * norm_weight, factor applied to the sums */
 
 #define TL_ACT_NONE 0
 #define TL_ACT_SILU_GATE 1 /* out = silu(gate) * up, for tl_mlp_gate_up */
@@ -330,12 +332,26 @@ int tl_decode_attention_rope(const void* qkv, const void* cos_table, const void*
  *   TL_PRODUCER_ADD_RMSNORM  s = in + in2 (in2 may be NULL), x = s * rsqrt(mean(s^2) + eps) * norm_weight;
  *                            s is also written to sum_out when that is not NULL (tl_add_rmsnorm followed
  *                            by tl_spmm).  sum_out must not alias in or in2.
+ *   TL_PRODUCER_RMSNORM      x = in * rsqrt(mean(in^2) + eps) * norm_weight, with the factor, one number for the
+ *                            row, applied to the column sums instead of the row: the row that is multiplied is
+ *                            in * norm_weight rounded to x_dtype, and no part of the kernel waits for the mean.
+ *                            Equal to TL_PRODUCER_ADD_RMSNORM with in2 == NULL up to that rounding; in2 and
+ *                            sum_out must be NULL.  (The residual add belongs to the product BEFORE the norm
+ *                            then: tl_spmv_add, tl_spmv_attn_combine_add.)
  * in, in2, norm_weight, sum_out are of x_dtype, K values each (2K for the gate | up row), 16-byte aligned.
  * Roundings are those of the separate kernels.  TL_ERR_UNSUPPORTED when K or the blob's tile height is not
  * a whole number of 16-byte pieces (use the separate kernels then). */
 int tl_spmv_fused(const tl_layout_header* header, const void* blob_dev, int producer,
                   const void* in, const void* in2, const void* norm_weight, float eps, void* sum_out, int x_dtype,
                   void* Y, int y_dtype, const void* scale, int scale_dtype, void* stream);
+
+/* Y[N] = residual[N] + (x * W) * scale for one contiguous, 16-byte aligned row x: the residual add of a decoder
+ * layer (the Hugging Face decoder layer the reference patches, TernaryLLM/TernaryLlama.py:69-75) in the epilogue of
+ * the product in front of it, rounded as a separate add of the stored product would round (the product to y_dtype,
+ * then the sum).  residual: N values of y_dtype; Y may be the residual row itself.  TL_ERR_UNSUPPORTED where the
+ * single-row kernels do not apply (K or the tile height not whole 16-byte pieces). */
+int tl_spmv_add(const tl_layout_header* header, const void* blob_dev, const void* x, int x_dtype, const void* residual,
+                void* Y, int y_dtype, const void* scale, int scale_dtype, void* stream);
 
 /* tl_spmv_fused with the epilogue of tl_spmm_gated: the weight's columns are (gate, up) pairs and Y holds the N / 2
  * values silu(y[2j]) * y[2j + 1].  Same arguments otherwise. */
@@ -353,6 +369,11 @@ int tl_spmv_fused_gated(const tl_layout_header* header, const void* blob_dev, in
 int tl_spmv_attn_combine(const tl_layout_header* header, const void* blob_dev, const void* pieces,
                          int splits, int head_dim, int x_dtype, void* Y, int y_dtype,
                          const void* scale, int scale_dtype, void* stream);
+
+/* tl_spmv_attn_combine with the residual add of tl_spmv_add in its epilogue. */
+int tl_spmv_attn_combine_add(const tl_layout_header* header, const void* blob_dev, const void* pieces,
+                             int splits, int head_dim, int x_dtype, const void* residual, void* Y, int y_dtype,
+                             const void* scale, int scale_dtype, void* stream);
 
 /* x_out = x + y, h_out = RMSNorm(x_out) * weight, row by row ([rows][width], one dtype): the residual
  * add of a decoder layer fused with the normalisation that follows (the reference leaves both to the

@@ -82,6 +82,7 @@ struct KernelArgs {
     int pro_hd;
     // gated epilogue: columns 2j, 2j + 1 of the weight are gate and up column j; Y[j] = silu(y[2j]) * y[2j + 1] (N / 2 outputs)
     int gated;
+    const void* residual;  // single-row kernels: null, or a row of N values of Y's type: Y[n] = residual[n] + the product (rounded to that type first)
     long long y_kld;      // gated epilogue of the 16-row kernel: 0, or the leading dimension of a K-major output [N / 2][y_kld]
 };
 
@@ -115,6 +116,14 @@ __device__ __forceinline__ float as_output(float v, int is_f16) { return is_f16 
 // silu(g) * u for a product's outputs g, u (already rounded to the output type), with the roundings of the separate
 // operator: the SiLU is rounded to the type before the product.
 __device__ __forceinline__ float gate_pair(float g, float u, int is_f16) { return as_output(g / (1.0f + __expf(-g)), is_f16) * u; }
+
+// One output of a single-row product on its way out: plain, or added to the residual row as a separate add of the
+// stored product would add it.
+__device__ __forceinline__ void store_result(const KernelArgs& a, int n, float v)
+{
+    if (a.residual) v = as_output(v, a.y_f16) + load_scale(a.residual, a.y_f16, n);
+    store_out(a.Y, a.y_f16, n, v);
+}
 
 __device__ __forceinline__ int run_pos_dwords(uint32_t d) { return (int)(((d & 0xffu) + 3u) >> 2); }
 __device__ __forceinline__ int run_neg_dwords(uint32_t d) { return (int)((((d >> 8) & 0xffu) + 3u) >> 2); }
@@ -882,6 +891,7 @@ __global__ __launch_bounds__(kBlockThreads) void tl_spmm_octet(KernelArgs a)
 // Roundings are those of the separate kernels (tl_silu_mul, tl_add_rmsnorm, tl_attn_combine): s, the SiLU and x
 // are rounded to the activation type.
 constexpr int kProNone = 0, kProSiluGate = 1, kProAddNorm = 2, kProAttnCombine = 3;
+constexpr int kProNormDeferred = 4;  // launcher only: RMSNorm whose factor multiplies the sums (tl_spmv_tiles), else kProAddNorm
 
 template <bool F16>
 __device__ __forceinline__ float round_to_x(float v)
@@ -1104,7 +1114,7 @@ __global__ __launch_bounds__(NT) void tl_spmv_direct(KernelArgs a)
             store_out(a.Y, a.y_f16, nb * (TL_BLOCK_COLUMNS / 2) + tid, gate_pair(sums[2 * tid], sums[2 * tid + 1], a.y_f16));
         return;
     }
-    if (lig == 0 && n < a.N) store_out(a.Y, a.y_f16, n, acc[0] * load_scale(a.w0.scale, a.scale_f16, n));
+    if (lig == 0 && n < a.N) store_result(a, n, acc[0] * load_scale(a.w0.scale, a.scale_f16, n));
 }
 
 // ---------------------------------------------------------------------------
@@ -1117,8 +1127,13 @@ __global__ __launch_bounds__(NT) void tl_spmv_direct(KernelArgs a)
 // barrier), while the loads of later tiles and of the other waves are still in flight.  The kernel's length is
 // then about the time the block's bytes take to arrive plus one tile's gather, where tl_spmv_direct, which splits
 // a tile's columns over the waves and so needs every wave's loads behind a barrier, adds the whole gather to it.
-// Only the plain product runs here: with a producer, whose operands must arrive and be worked on before the
-// first gather, tl_spmv_direct is the faster of the two.
+// With a producer whose operands must arrive and be worked on before the first gather, tl_spmv_direct is the
+// faster of the two (the residual add needs a third image in LDS, the normalisation a barrier in the middle).
+// The one producer that runs here is an RMSNorm whose factor is DEFERRED (NORM): the row in LDS is
+// in[k] * norm_w[k], made by each wave for its own tiles from two direct loads issued ahead of the chunks (waited
+// for by count, so the chunks stay in flight), the waves add up in[k]^2 on the side, and rsqrt(mean + eps), one
+// number for the whole row, multiplies the column sums at the very end -- no wave waits for another before it
+// gathers.  (The row is thus rounded to the activation type as in * norm_w, not as in * factor * norm_w.)
 
 // Waits until at most `later` of this wave's vector-memory instructions are outstanding (they complete in
 // order): everything issued before the last `later` has then arrived.  Counts above 13 wait for a few more.
@@ -1144,7 +1159,7 @@ __device__ __forceinline__ void tiles_wait_vm(int later)
 
 constexpr int kTilesMaxOwn = 8;  // tiles a wave of tl_spmv_tiles may own
 
-template <bool XF16, int NT>
+template <bool XF16, int NT, bool NORM = false>
 __global__ __launch_bounds__(NT) void tl_spmv_tiles(KernelArgs a)
 {
     extern __shared__ __align__(16) unsigned char lds[];
@@ -1161,10 +1176,24 @@ __global__ __launch_bounds__(NT) void tl_spmv_tiles(KernelArgs a)
     const unsigned char* Xb = static_cast<const unsigned char*>(a.X);
     unsigned char* xs = lds;                     // [T] tile images
     unsigned char* buf = lds + a.xs_bytes;       // the block's chunks, as they lie in the stream
-    float* red = reinterpret_cast<float*>(lds + a.xs_bytes + a.buf_bytes);  // [W][16] column sums of the waves
+    float* red = reinterpret_cast<float*>(lds + a.xs_bytes + a.buf_bytes);  // [W][16] column sums of the waves, then [W] sums of squares
+    unsigned char* weights = reinterpret_cast<unsigned char*>(red + ((W * (TL_BLOCK_COLUMNS + 1) + 3) & ~3));  // NORM: [T] images of norm_w
     using global_ptr = const __attribute__((address_space(1))) void*;
     using lds_ptr = __attribute__((address_space(3))) void*;
     const uint32_t base = cs[0];
+
+    if constexpr (NORM) {
+        // the row and the norm weight of this wave's tiles, ahead of every chunk
+#pragma unroll
+        for (int j = 0; j < kMaxOwn; ++j) {
+            const int t = wave + j * W;
+            if (t < a.T && lane * VE < min(a.tile_rows, a.K - t * a.tile_rows)) {
+                const size_t k = (size_t)t * a.tile_rows + (size_t)lane * VE, image = (size_t)t * PITCH * ES;
+                __builtin_amdgcn_global_load_lds((global_ptr)(Xb + k * ES), (lds_ptr)(xs + image), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((global_ptr)(static_cast<const unsigned char*>(a.norm_w) + k * ES), (lds_ptr)(weights + image), 16, 0, 0);
+            }
+        }
+    }
 
     // every load of this wave, tile after tile; loads[j] = vector-memory instructions of its j-th tile
     int loads[kMaxOwn];
@@ -1185,11 +1214,37 @@ __global__ __launch_bounds__(NT) void tl_spmv_tiles(KernelArgs a)
             // slot among them) is zeroed
             const int rows_here = min(a.tile_rows, a.K - t * a.tile_rows);
             unsigned char* image = xs + (size_t)t * PITCH * ES;
-            if (lane * VE < rows_here)
-                __builtin_amdgcn_global_load_lds((global_ptr)(Xb + ((size_t)t * a.tile_rows + (size_t)lane * VE) * ES), (lds_ptr)image, 16, 0, 0);
-            else if (lane * VE < kTileSlots)
-                *reinterpret_cast<u32x4*>(image + (size_t)lane * 16) = u32x4{0u, 0u, 0u, 0u};
-            ++loads[j];
+            if constexpr (!NORM) {
+                if (lane * VE < rows_here)
+                    __builtin_amdgcn_global_load_lds((global_ptr)(Xb + ((size_t)t * a.tile_rows + (size_t)lane * VE) * ES), (lds_ptr)image, 16, 0, 0);
+                ++loads[j];
+            }
+            if (lane * VE >= rows_here && lane * VE < kTileSlots) *reinterpret_cast<u32x4*>(image + (size_t)lane * 16) = u32x4{0u, 0u, 0u, 0u};
+        }
+    }
+
+    float squares = 0.f;  // NORM: this lane's share of sum(in^2)
+    if constexpr (NORM) {
+        int chunk_loads = 0;
+#pragma unroll
+        for (int j = 0; j < kMaxOwn; ++j) chunk_loads += loads[j];
+        tiles_wait_vm(chunk_loads);  // row and weight pieces are here when only the chunk loads are outstanding
+#pragma unroll 1
+        for (int t = wave; t < a.T; t += W) {
+            if (lane * VE < min(a.tile_rows, a.K - t * a.tile_rows)) {
+                const size_t at = (size_t)t * PITCH * ES + (size_t)lane * 16;
+                u32x4 v = *reinterpret_cast<const u32x4*>(xs + at);
+                const u32x4 wv = *reinterpret_cast<const u32x4*>(weights + at);
+                XT* x = reinterpret_cast<XT*>(&v);
+                const XT* w = reinterpret_cast<const XT*>(&wv);
+#pragma unroll
+                for (int e = 0; e < VE; ++e) {
+                    const float f = (float)x[e];
+                    squares = fmaf(f, f, squares);
+                    x[e] = XT(f * (float)w[e]);
+                }
+                *reinterpret_cast<u32x4*>(xs + at) = v;
+            }
         }
     }
 
@@ -1214,11 +1269,22 @@ __global__ __launch_bounds__(NT) void tl_spmv_tiles(KernelArgs a)
     acc[0] += __shfl_xor(acc[0], 1, 64);
     acc[0] += __shfl_xor(acc[0], 2, 64);
     if (lw == 0) red[wave * TL_BLOCK_COLUMNS + c16] = acc[0];
+    if constexpr (NORM) {
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) squares += __shfl_xor(squares, off, 64);
+        if (lane == 0) red[W * TL_BLOCK_COLUMNS + wave] = squares;
+    }
     __syncthreads();
     if (tid < TL_BLOCK_COLUMNS) {
         float sum = 0.f;
 #pragma unroll
         for (int w = 0; w < W; ++w) sum += red[w * TL_BLOCK_COLUMNS + tid];
+        if constexpr (NORM) {
+            float total = 0.f;
+#pragma unroll
+            for (int w = 0; w < W; ++w) total += red[W * TL_BLOCK_COLUMNS + w];
+            sum *= rsqrtf(total / (float)a.K + a.eps);
+        }
         const int n = nb * TL_BLOCK_COLUMNS + tid;
         if (a.gated) {
             const float y = n < a.N ? as_output(sum * load_scale(a.w0.scale, a.scale_f16, n), a.y_f16) : 0.f;
@@ -1226,7 +1292,7 @@ __global__ __launch_bounds__(NT) void tl_spmv_tiles(KernelArgs a)
             if (!(tid & 1) && n + 1 < a.N) store_out(a.Y, a.y_f16, n / 2, gate_pair(y, up, a.y_f16));
             return;
         }
-        if (n < a.N) store_out(a.Y, a.y_f16, n, sum * load_scale(a.w0.scale, a.scale_f16, n));
+        if (n < a.N) store_result(a, n, sum * load_scale(a.w0.scale, a.scale_f16, n));
     }
 }
 
@@ -2057,7 +2123,7 @@ int launch_spmv_direct_nt(KernelArgs a, const tl_layout_header* h, hipStream_t s
 
 // tl_spmv_tiles: every tile of the block resident (a wave loads its own and waits for nobody else's).
 // Returns TL_ERR_UNSUPPORTED when that does not fit; the caller then takes tl_spmv_direct.
-template <bool XF16, int NT>
+template <bool XF16, int NT, bool NORM = false>
 int launch_spmv_tiles_nt(KernelArgs a, const tl_layout_header* h, hipStream_t st)
 {
     constexpr int es = XF16 ? 2 : 4;
@@ -2066,10 +2132,11 @@ int launch_spmv_tiles_nt(KernelArgs a, const tl_layout_header* h, hipStream_t st
     if (a.T > (NT / 64) * kTilesMaxOwn) return TL_ERR_UNSUPPORTED;
     a.xs_bytes = a.T * tile_bytes;
     a.buf_bytes = (int)round_up((int64_t)a.T * chunk_bytes, 16);
-    const size_t lds = (size_t)a.xs_bytes + a.buf_bytes + (size_t)(NT / 64) * TL_BLOCK_COLUMNS * 4;
-    const int share = std::max(1, std::min(knob(TL_SPMV_SHARE, 4), (int)ceil_div(a.NB, compute_units())));
+    const size_t lds = (size_t)a.xs_bytes * (NORM ? 2 : 1) + a.buf_bytes + (size_t)(((NT / 64) * (TL_BLOCK_COLUMNS + 1) + 3) & ~3) * 4;
+    int share = std::max(1, std::min(knob(TL_SPMV_SHARE, 4), (int)ceil_div(a.NB, compute_units())));
+    if (NORM) share = std::min(share, 3);  // the second set of images: three workgroups of K = 4096 fit a compute unit, not four
     if (lds > (size_t)(160 * 1024 / share - 1024)) return TL_ERR_UNSUPPORTED;
-    auto kernel = tl_spmv_tiles<XF16, NT>;
+    auto kernel = tl_spmv_tiles<XF16, NT, NORM>;
     static bool raised = false;  // per instantiation; a repeated or racing call is harmless
     if (!raised) {
         if (int rc = raise_lds_limit(kernel, 160 * 1024)) return rc;
@@ -2085,14 +2152,22 @@ template <bool XF16, int PRO = kProNone>
 int launch_spmv_direct(const KernelArgs& a, const tl_layout_header* h, hipStream_t st)
 {
     const bool wide = knob(TL_SPMV_WIDE, a.NB <= compute_units() ? 1 : 0) != 0;
-    if constexpr (PRO == kProNone) {
-        // the tile-per-wave kernel where the block fits it; with a producer it is the slower of the two
+    if constexpr (PRO == kProNormDeferred) {
         if (knob(TL_SPMV_TILES, 1) != 0) {
-            const int rc = wide ? launch_spmv_tiles_nt<XF16, 1024>(a, h, st) : launch_spmv_tiles_nt<XF16, kBlockThreads>(a, h, st);
+            const int rc = wide ? launch_spmv_tiles_nt<XF16, 1024, true>(a, h, st) : launch_spmv_tiles_nt<XF16, kBlockThreads, true>(a, h, st);
             if (rc != TL_ERR_UNSUPPORTED) return rc;
         }
+        return wide ? launch_spmv_direct_nt<XF16, 1024, kProAddNorm>(a, h, st) : launch_spmv_direct_nt<XF16, kBlockThreads, kProAddNorm>(a, h, st);
+    } else {
+        if constexpr (PRO == kProNone) {
+            // the tile-per-wave kernel where the block fits it; with the other producers it is the slower of the two
+            if (knob(TL_SPMV_TILES, 1) != 0) {
+                const int rc = wide ? launch_spmv_tiles_nt<XF16, 1024>(a, h, st) : launch_spmv_tiles_nt<XF16, kBlockThreads>(a, h, st);
+                if (rc != TL_ERR_UNSUPPORTED) return rc;
+            }
+        }
+        return wide ? launch_spmv_direct_nt<XF16, 1024, PRO>(a, h, st) : launch_spmv_direct_nt<XF16, kBlockThreads, PRO>(a, h, st);
     }
-    return wide ? launch_spmv_direct_nt<XF16, 1024, PRO>(a, h, st) : launch_spmv_direct_nt<XF16, kBlockThreads, PRO>(a, h, st);
 }
 
 template <int MT>
@@ -2458,7 +2533,7 @@ extern "C" int tl_spmm_noalloc(const tl_layout_header* header, const void* blob_
 namespace {
 int spmv_fused_call(const tl_layout_header* header, const void* blob_dev, int producer,
                     const void* in, const void* in2, const void* norm_weight, float eps, void* sum_out, int x_dtype,
-                    void* Y, int y_dtype, const void* scale, int scale_dtype, void* stream, bool gated)
+                    void* Y, int y_dtype, const void* scale, int scale_dtype, void* stream, bool gated, const void* residual = nullptr)
 {
     if (int rc = check_header(header)) return rc;
     if (gated && header->columns % 2) return fail(TL_ERR_SHAPE, "N=%u: gate and up columns come in pairs", header->columns);
@@ -2466,11 +2541,14 @@ int spmv_fused_call(const tl_layout_header* header, const void* blob_dev, int pr
     if (int rc = check_dtype(y_dtype, "y")) return rc;
     if (scale)
         if (int rc = check_dtype(scale_dtype, "scale")) return rc;
-    if (producer != TL_PRODUCER_SILU_GATE && producer != TL_PRODUCER_ADD_RMSNORM) return fail(TL_ERR_ARG, "producer code %d unknown", producer);
+    if (producer != TL_PRODUCER_NONE && producer != TL_PRODUCER_SILU_GATE && producer != TL_PRODUCER_ADD_RMSNORM && producer != TL_PRODUCER_RMSNORM)
+        return fail(TL_ERR_ARG, "producer code %d unknown", producer);
+    if (residual && gated) return fail(TL_ERR_ARG, "a gated product has no residual row of its width");
+    if (reinterpret_cast<uintptr_t>(residual) % (y_dtype == TL_F16 ? 2 : 4)) return fail(TL_ERR_ALIGN, "residual is not aligned to its type");
     if (!blob_dev || !in || !Y) return fail(TL_ERR_ARG, "device pointer is null");
     if (reinterpret_cast<uintptr_t>(blob_dev) % 256) return fail(TL_ERR_ALIGN, "weight blob must be 256-byte aligned");
-    if (producer == TL_PRODUCER_ADD_RMSNORM && !norm_weight) return fail(TL_ERR_ARG, "norm_weight is null");
-    if (producer == TL_PRODUCER_SILU_GATE && (in2 || sum_out)) return fail(TL_ERR_ARG, "in2 and sum_out belong to TL_PRODUCER_ADD_RMSNORM");
+    if ((producer == TL_PRODUCER_ADD_RMSNORM || producer == TL_PRODUCER_RMSNORM) && !norm_weight) return fail(TL_ERR_ARG, "norm_weight is null");
+    if (producer != TL_PRODUCER_ADD_RMSNORM && (in2 || sum_out)) return fail(TL_ERR_ARG, "in2 and sum_out belong to TL_PRODUCER_ADD_RMSNORM");
     if (sum_out && (sum_out == in || sum_out == in2)) return fail(TL_ERR_ARG, "sum_out must not be one of the inputs: other workgroups still read them");
     const int es = x_dtype == TL_F16 ? 2 : 4, ve = 16 / es;
     // what the direct-load kernel needs of a row: whole aligned 16-byte pieces per tile
@@ -2489,9 +2567,14 @@ int spmv_fused_call(const tl_layout_header* header, const void* blob_dev, int pr
     a.x_f16 = x_dtype == TL_F16; a.y_f16 = y_dtype == TL_F16; a.scale_f16 = scale_dtype == TL_F16;
     a.one = 1.0f;
     a.gated = gated;
+    a.residual = residual;
     hipStream_t st = static_cast<hipStream_t>(stream);
     int rc;
-    if (producer == TL_PRODUCER_SILU_GATE)
+    if (producer == TL_PRODUCER_NONE)
+        rc = a.x_f16 ? launch_spmv_direct<true>(a, header, st) : launch_spmv_direct<false>(a, header, st);
+    else if (producer == TL_PRODUCER_RMSNORM)
+        rc = a.x_f16 ? launch_spmv_direct<true, kProNormDeferred>(a, header, st) : launch_spmv_direct<false, kProNormDeferred>(a, header, st);
+    else if (producer == TL_PRODUCER_SILU_GATE)
         rc = a.x_f16 ? launch_spmv_direct<true, kProSiluGate>(a, header, st) : launch_spmv_direct<false, kProSiluGate>(a, header, st);
     else
         rc = a.x_f16 ? launch_spmv_direct<true, kProAddNorm>(a, header, st) : launch_spmv_direct<false, kProAddNorm>(a, header, st);
@@ -2507,6 +2590,14 @@ extern "C" int tl_spmv_fused(const tl_layout_header* header, const void* blob_de
     return spmv_fused_call(header, blob_dev, producer, in, in2, norm_weight, eps, sum_out, x_dtype, Y, y_dtype, scale, scale_dtype, stream, false);
 }
 
+extern "C" int tl_spmv_add(const tl_layout_header* header, const void* blob_dev, const void* x, int x_dtype, const void* residual,
+                           void* Y, int y_dtype, const void* scale, int scale_dtype, void* stream)
+{
+    if (!residual) return fail(TL_ERR_ARG, "residual is null");
+    return spmv_fused_call(header, blob_dev, TL_PRODUCER_NONE, x, nullptr, nullptr, 0.f, nullptr, x_dtype, Y, y_dtype, scale, scale_dtype, stream, false,
+                           residual);
+}
+
 extern "C" int tl_spmv_fused_gated(const tl_layout_header* header, const void* blob_dev, int producer,
                                    const void* in, const void* in2, const void* norm_weight, float eps, void* sum_out, int x_dtype,
                                    void* Y, int y_dtype, const void* scale, int scale_dtype, void* stream)
@@ -2514,10 +2605,12 @@ extern "C" int tl_spmv_fused_gated(const tl_layout_header* header, const void* b
     return spmv_fused_call(header, blob_dev, producer, in, in2, norm_weight, eps, sum_out, x_dtype, Y, y_dtype, scale, scale_dtype, stream, true);
 }
 
-extern "C" int tl_spmv_attn_combine(const tl_layout_header* header, const void* blob_dev, const void* pieces, int splits, int head_dim,
-                                    int x_dtype, void* Y, int y_dtype, const void* scale, int scale_dtype, void* stream)
+namespace {
+int attn_combine_call(const tl_layout_header* header, const void* blob_dev, const void* pieces, int splits, int head_dim,
+                      int x_dtype, void* Y, int y_dtype, const void* scale, int scale_dtype, void* stream, const void* residual)
 {
     if (int rc = check_header(header)) return rc;
+    if (reinterpret_cast<uintptr_t>(residual) % (y_dtype == TL_F16 ? 2 : 4)) return fail(TL_ERR_ALIGN, "residual is not aligned to its type");
     if (int rc = check_dtype(x_dtype, "x")) return rc;
     if (int rc = check_dtype(y_dtype, "y")) return rc;
     if (scale)
@@ -2542,10 +2635,25 @@ extern "C" int tl_spmv_attn_combine(const tl_layout_header* header, const void* 
     a.NB = (int)header->n_blocks;
     a.x_f16 = x_dtype == TL_F16; a.y_f16 = y_dtype == TL_F16; a.scale_f16 = scale_dtype == TL_F16;
     a.one = 1.0f;
+    a.residual = residual;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int rc = a.x_f16 ? launch_spmv_direct<true, kProAttnCombine>(a, header, st) : launch_spmv_direct<false, kProAttnCombine>(a, header, st);
     if (rc) return rc;
     return finish_launch();
+}
+}  // namespace
+
+extern "C" int tl_spmv_attn_combine(const tl_layout_header* header, const void* blob_dev, const void* pieces, int splits, int head_dim,
+                                    int x_dtype, void* Y, int y_dtype, const void* scale, int scale_dtype, void* stream)
+{
+    return attn_combine_call(header, blob_dev, pieces, splits, head_dim, x_dtype, Y, y_dtype, scale, scale_dtype, stream, nullptr);
+}
+
+extern "C" int tl_spmv_attn_combine_add(const tl_layout_header* header, const void* blob_dev, const void* pieces, int splits, int head_dim,
+                                        int x_dtype, const void* residual, void* Y, int y_dtype, const void* scale, int scale_dtype, void* stream)
+{
+    if (!residual) return fail(TL_ERR_ARG, "residual is null");
+    return attn_combine_call(header, blob_dev, pieces, splits, head_dim, x_dtype, Y, y_dtype, scale, scale_dtype, stream, residual);
 }
 
 extern "C" int tl_mlp_gate_up(const tl_layout_header* gate_header, const void* gate_blob_dev,

@@ -237,16 +237,17 @@ class TernaryLlamaDecoder(nn.Module):
         (32 heads alone would leave seven compute units in eight idle) and leaves its result in pieces that the
         output projection folds while it stages its row (tl_spmv_attn_combine)."""
         eps = self.config.rms_norm_eps
-        y = None   # what the previous block still has to add to the residual stream
+        hd, dtype = self.config.head_dim, x.dtype
+        # x is the residual stream: every product that ends a block adds its result to it in the epilogue, and the
+        # products that start one normalise it on the way in (the factor applied to their sums)
         for layer in self.layers:
-            qkv, x = ops.spmv_fused(layer.qkv_proj.device_weight(), "add_rmsnorm", x, y, layer.input_layernorm.weight, eps,
-                                    layer.qkv_proj.w_scale, want_sum=True)
+            qkv = ops.spmv_fused(layer.qkv_proj.device_weight(), "rmsnorm", x, None, layer.input_layernorm.weight, eps, layer.qkv_proj.w_scale)
             pieces = self._attend(qkv, self._cache_of(layer, 0), self._cache_of(layer, 1), pos, False, pieces=True)
-            o = ops.spmv_attn_combine(layer.o_proj.device_weight(), pieces, self.config.head_dim, x.dtype, layer.o_proj.w_scale)
-            gated, x = ops.spmv_fused(layer.gate_up_proj.device_weight(), "add_rmsnorm", x, o, layer.post_attention_layernorm.weight, eps,
-                                      layer.gate_up_proj.w_scale, want_sum=True, gated=True)
-            y = ops.spmm(layer.down_proj.device_weight(), gated, layer.down_proj.w_scale)
-        return ops.spmv_fused(self.lm_head.device_weight(), "add_rmsnorm", x, y, self.norm.weight, eps, self.lm_head.w_scale)
+            x = ops.spmv_attn_combine(layer.o_proj.device_weight(), pieces, hd, dtype, layer.o_proj.w_scale, residual=x)
+            gated = ops.spmv_fused(layer.gate_up_proj.device_weight(), "rmsnorm", x, None, layer.post_attention_layernorm.weight, eps,
+                                   layer.gate_up_proj.w_scale, gated=True)
+            x = ops.spmv_add(layer.down_proj.device_weight(), gated, x, layer.down_proj.w_scale)
+        return ops.spmv_fused(self.lm_head.device_weight(), "rmsnorm", x, None, self.norm.weight, eps, self.lm_head.w_scale)
 
     def _attend(self, qkv, k_cache, v_cache, pos, kmajor, pieces=False):
         """Rotary embedding, cache update and attention for the token whose q | k | v the projection just wrote: one

@@ -203,22 +203,27 @@ def spmv_fused(weight, producer, inp, inp2=None, norm_weight=None, eps=0.0, scal
     """y[1, N] = (x @ W) * scale for one activation row x that the call produces itself (tl_spmv_fused):
     producer "silu_gate": x = silu(inp[:K]) * inp[K:] for a gate | up row inp of 2K values;
     producer "add_rmsnorm": s = inp + inp2 (inp2 may be None), x = rmsnorm(s) * norm_weight; with want_sum the
-    call also returns s (a new tensor).  Returns y, or (y, s).  Raises RuntimeError (TL_ERR_UNSUPPORTED) where the
+    call also returns s (a new tensor);
+    producer "rmsnorm": x = rmsnorm(inp) * norm_weight with the normalisation factor applied to the column sums (the
+    row multiplied is inp * norm_weight in inp's dtype; no part of the kernel waits for the mean).
+    Returns y, or (y, s).  Raises RuntimeError (TL_ERR_UNSUPPORTED) where the
     fused kernel does not apply (K or the tile height not whole 16-byte pieces); callers then use the separate operators.
     gated: the weight's columns are (gate, up) pairs and y is [1, N / 2] with y[j] = silu(y'[2j]) * y'[2j + 1]
     (tl_spmv_fused_gated)."""
     K, N = weight.inners, weight.columns
     if gated and N % 2:
         raise ValueError("gate and up columns come in pairs: N must be even")
-    code = {"silu_gate": _lib.TL_PRODUCER_SILU_GATE, "add_rmsnorm": _lib.TL_PRODUCER_ADD_RMSNORM}[producer]
+    code = {"silu_gate": _lib.TL_PRODUCER_SILU_GATE, "add_rmsnorm": _lib.TL_PRODUCER_ADD_RMSNORM, "rmsnorm": _lib.TL_PRODUCER_RMSNORM}[producer]
+    if producer == "rmsnorm" and (inp2 is not None or want_sum):
+        raise ValueError("the rmsnorm producer has no second summand: the residual add belongs to the product before it (spmv_add)")
     x_code = _code(inp.dtype, "inp")
     need = 2 * K if producer == "silu_gate" else K
     tensors = [inp] + [t for t in (inp2, norm_weight) if t is not None]
     for t in tensors:
         if t.numel() != (need if t is inp else K) or not t.is_contiguous() or t.dtype != inp.dtype or t.device != weight.device:
             raise ValueError("inputs must be contiguous rows of the weight's K (2K for a gate | up row), one dtype, on the weight's device")
-    if producer == "add_rmsnorm" and norm_weight is None:
-        raise ValueError("add_rmsnorm needs norm_weight")
+    if producer != "silu_gate" and norm_weight is None:
+        raise ValueError(f"{producer} needs norm_weight")
     out_dtype = out_dtype or inp.dtype
     y = torch.empty((1, N // 2 if gated else N), dtype=out_dtype, device=inp.device)
     s_out = torch.empty(K, dtype=inp.dtype, device=inp.device).view(inp.shape) if (want_sum and producer == "add_rmsnorm") else None
@@ -234,11 +239,30 @@ def spmv_fused(weight, producer, inp, inp2=None, norm_weight=None, eps=0.0, scal
     return (y, s_out) if want_sum else y
 
 
-def spmv_attn_combine(weight, pieces, head_dim, x_dtype, scale=None, out_dtype=None):
+def spmv_add(weight, x, residual, scale=None):
+    """residual + (x @ W) * scale for one contiguous row x [1, K] or [K] and a residual row of N values (tl_spmv_add):
+    the residual add of a decoder layer in the epilogue of the product in front of it, rounded as the separate add of
+    the stored product would round.  Returns a new [1, N] tensor of residual's dtype."""
+    K, N = weight.inners, weight.columns
+    if x.numel() != K or residual.numel() != N or not x.is_contiguous() or not residual.is_contiguous():
+        raise ValueError("x must be a contiguous row of K values and residual one of N")
+    if x.device != weight.device or residual.device != weight.device:
+        raise RuntimeError("x and residual must be on the weight's device")
+    y = torch.empty((1, N), dtype=residual.dtype, device=x.device)
+    scale, s_code = _scale_args(scale, N, x.device)
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().tl_spmv_add(ctypes.byref(weight.header), weight.blob.data_ptr(), x.data_ptr(), _code(x.dtype, "x"), residual.data_ptr(),
+                                    y.data_ptr(), _code(residual.dtype, "residual"), scale.data_ptr() if scale is not None else None, s_code,
+                                    _stream_ptr(x.device))
+    _lib.check(rc)
+    return y
+
+
+def spmv_attn_combine(weight, pieces, head_dim, x_dtype, scale=None, out_dtype=None, residual=None):
     """y[1, N] = (a @ W) * scale where a is the attention output (rounded to x_dtype) that `pieces` -- what
     decode_attention_pieces returned for batch 1 -- add up to: the output projection with the fold of the
-    pieces inside (tl_spmv_attn_combine).  Raises RuntimeError (TL_ERR_UNSUPPORTED) where the fused kernel
-    does not apply."""
+    pieces inside (tl_spmv_attn_combine).  residual: a row of N values of the output dtype that the result is
+    added to, as in spmv_add.  Raises RuntimeError (TL_ERR_UNSUPPORTED) where the fused kernel does not apply."""
     K, N = weight.inners, weight.columns
     if pieces.dtype != torch.float32 or pieces.dim() != 3 or not pieces.is_contiguous() or pieces.device != weight.device:
         raise ValueError("pieces must be a contiguous float32 [heads, splits, head_dim + 4] tensor on the weight's device")
@@ -246,12 +270,19 @@ def spmv_attn_combine(weight, pieces, head_dim, x_dtype, scale=None, out_dtype=N
     if width != head_dim + 4 or heads * head_dim != K:
         raise ValueError(f"pieces of shape {tuple(pieces.shape)} do not make a row of K={K} with head_dim={head_dim}")
     out_dtype = out_dtype or x_dtype
+    if residual is not None and (residual.numel() != N or residual.dtype != out_dtype or not residual.is_contiguous() or residual.device != weight.device):
+        raise ValueError("residual must be a contiguous row of N values of the output dtype on the weight's device")
     y = torch.empty((1, N), dtype=out_dtype, device=pieces.device)
     scale, s_code = _scale_args(scale, N, pieces.device)
     with torch.cuda.device(pieces.device):
-        rc = _lib.lib().tl_spmv_attn_combine(ctypes.byref(weight.header), weight.blob.data_ptr(), pieces.data_ptr(), splits, head_dim,
-                                             _code(x_dtype, "x_dtype"), y.data_ptr(), _code(out_dtype, "out_dtype"),
-                                             scale.data_ptr() if scale is not None else None, s_code, _stream_ptr(pieces.device))
+        if residual is None:
+            rc = _lib.lib().tl_spmv_attn_combine(ctypes.byref(weight.header), weight.blob.data_ptr(), pieces.data_ptr(), splits, head_dim,
+                                                 _code(x_dtype, "x_dtype"), y.data_ptr(), _code(out_dtype, "out_dtype"),
+                                                 scale.data_ptr() if scale is not None else None, s_code, _stream_ptr(pieces.device))
+        else:
+            rc = _lib.lib().tl_spmv_attn_combine_add(ctypes.byref(weight.header), weight.blob.data_ptr(), pieces.data_ptr(), splits, head_dim,
+                                                     _code(x_dtype, "x_dtype"), residual.data_ptr(), y.data_ptr(), _code(out_dtype, "out_dtype"),
+                                                     scale.data_ptr() if scale is not None else None, s_code, _stream_ptr(pieces.device))
     _lib.check(rc)
     return y
 

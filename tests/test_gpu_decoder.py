@@ -259,6 +259,8 @@ def test_split_attention_and_its_fold_inside_the_output_projection(cuda, oracle)
                 unfused = ops.spmm(dw, a, scale)
                 # the folded row may differ from the separately folded one in its last bit (fp32 sums in another order)
                 assert max_rel_err(out.double().cpu().numpy(), unfused.double().cpu().numpy(), a.double().cpu().numpy(), w) <= tol
+                res = torch.randn(N, generator=g).to(dtype).to(cuda)
+                assert torch.equal(ops.spmv_attn_combine(dw, pieces, hd, dtype, scale, residual=res), out + res[None])
     with pytest.raises(ValueError):
         ops.spmv_attn_combine(dw, torch.zeros((H, 2, hd + 3), device=cuda), hd, torch.float16)
     with pytest.raises(ValueError, match="splits"):
@@ -339,8 +341,9 @@ def test_add_rmsnorm_and_silu_mul(cuda):
 @pytest.mark.parametrize("dtype,tol", [(torch.float16, 2e-3), (torch.float32, 1e-5)])
 def test_fused_producers_of_the_single_row_product(cuda, oracle, dtype, tol):
     """tl_spmv_fused: the residual add + RMSNorm and the SiLU gate computed inside the product's kernel, against a
-    float64 restatement and against the separate kernels followed by the plain product."""
-    from tests.util import max_rel_err, ternary_weight
+    float64 restatement and against the separate kernels followed by the plain product; the RMSNorm whose factor is
+    applied to the sums, and the residual add in a product's epilogue."""
+    from tests.util import knobs, max_rel_err, ternary_weight
     from ternaryllm_amd import ops
     from ternaryllm_amd.packing import PackedWeight
     g = torch.Generator().manual_seed(14)
@@ -371,6 +374,22 @@ def test_fused_producers_of_the_single_row_product(cuda, oracle, dtype, tol):
         act = ops.silu_mul(gu[None])
         unfused = ops.spmm(dw, act, sc)    # same roundings of the row; the plain product may sum in another order
         assert max_rel_err(out.double().cpu().numpy(), unfused.double().cpu().numpy(), act.double().cpu().numpy(), w) <= tol
+        # RMSNorm with the factor applied to the sums (both single-row kernels), and the residual add in the epilogue
+        for second in (None, y):
+            base = x if second is None else x + second
+            h64 = base.double() * torch.rsqrt(base.double().pow(2).mean() + 1e-5) * nw.double()
+            ref = (h64.cpu().numpy()[None, :] @ wd) * sc.double().cpu().numpy()[None, :]
+            for setting in ({}, {"TL_SPMV_TILES": "0"}, {"TL_SPMV_WIDE": "0"}, {"TL_SPMV_WIDE": "1"}):
+                with knobs(**setting):
+                    out = ops.spmv_fused(dw, "rmsnorm", base, None, nw, 1e-5, sc)
+                    assert max_rel_err(out.double().cpu().numpy(), ref, h64.cpu().numpy()[None, :], w) <= 2 * tol, (K, N, setting)
+                    if N % 2 == 0:
+                        assert torch.equal(ops.spmv_fused(dw, "rmsnorm", base, None, nw, 1e-5, sc, gated=True), ops.silu_mul(out, pairs=True))
+                    res = torch.randn(N, generator=g).to(dtype).to(cuda)
+                    act = torch.randn((1, K), generator=g).to(dtype).to(cuda)
+                    assert torch.equal(ops.spmv_add(dw, act, res, sc), ops.spmm(dw, act, sc) + res[None]), (K, N, setting)
+        with pytest.raises(ValueError, match="residual add belongs"):
+            ops.spmv_fused(dw, "rmsnorm", x, y, nw, 1e-5, sc)
     with pytest.raises(RuntimeError, match="UNSUPPORTED"):   # a tile height that is not whole 16-byte pieces: the separate kernels are the way then
         odd = ops.DeviceWeight(PackedWeight.from_dense(ternary_weight(1000, 40, 0.7, 3), tile_rows=250), cuda)
         ops.spmv_fused(odd, "silu_gate", torch.zeros(2000, dtype=dtype, device=cuda))
