@@ -231,11 +231,13 @@ class TernaryLlamaDecoder(nn.Module):
         return self.lm_head(h)
 
     def _decode_step_fused(self, x, pos):
-        """One row: the residual add + RMSNorm in front of the q|k|v and gate|up products and the SiLU gate in
-        front of the down projection are computed inside those products' kernels (tl_spmv_fused), and the
-        rotary embedding and the cache update inside the attention's: five launches per layer instead of nine.  The attention shares the cache rows of a head out among several workgroups
-        (32 heads alone would leave seven compute units in eight idle) and leaves its result in pieces that the
-        output projection folds while it stages its row (tl_spmv_attn_combine)."""
+        """One row, five launches per layer instead of nine, none of them an elementwise kernel: q|k|v and gate|up
+        normalise their input themselves (RMSNorm with the factor applied to the sums, tl_spmv_fused "rmsnorm"); the
+        gate|up product applies the SiLU gate in its epilogue (columns packed as gate/up pairs); the attention rotates
+        q and k and writes the cache row, shares the cache rows of a head out among several workgroups (32 heads alone
+        would leave seven compute units in eight idle) and leaves its result in pieces that the output projection
+        folds while it stages its row (tl_spmv_attn_combine); the o and down projections add their result to the
+        residual stream in their epilogue."""
         eps = self.config.rms_norm_eps
         hd, dtype = self.config.head_dim, x.dtype
         # x is the residual stream: every product that ends a block adds its result to it in the epilogue, and the
