@@ -128,6 +128,10 @@ class TernaryLlamaDecoder(nn.Module):
             self.lm_head._header.tile_rows % 8 == 0 and H % 8 == 0
         # the attention kernel rotates q and k and writes the token's cache row itself; False runs the separate kernel first
         self.fused_rope = True
+        # single-row steps: share the cache rows of a head out among several workgroups and fold the pieces inside the
+        # output projection.  That pays once a head's rows are many: up to about a thousand rows one workgroup per
+        # head and a plain output projection (the faster single-row kernel) are quicker together.
+        self.split_attention = self.max_seq_len > 1024
         self._layer_index = {id(layer): i for i, layer in enumerate(self.layers)}
 
     # -- pieces ------------------------------------------------------------------------------
@@ -234,24 +238,28 @@ class TernaryLlamaDecoder(nn.Module):
         """One row, five launches per layer instead of nine, none of them an elementwise kernel: q|k|v and gate|up
         normalise their input themselves (RMSNorm with the factor applied to the sums, tl_spmv_fused "rmsnorm"); the
         gate|up product applies the SiLU gate in its epilogue (columns packed as gate/up pairs); the attention rotates
-        q and k and writes the cache row, shares the cache rows of a head out among several workgroups (32 heads alone
-        would leave seven compute units in eight idle) and leaves its result in pieces that the output projection
-        folds while it stages its row (tl_spmv_attn_combine); the o and down projections add their result to the
-        residual stream in their epilogue."""
+        q and k and writes the cache row; with a long cache (split_attention) it shares the cache rows of a head out
+        among several workgroups (32 heads alone leave seven compute units in eight idle) and leaves its result in
+        pieces that the output projection folds while it stages its row (tl_spmv_attn_combine); the o and down
+        projections add their result to the residual stream in their epilogue."""
         eps = self.config.rms_norm_eps
         hd, dtype = self.config.head_dim, x.dtype
         # x is the residual stream: every product that ends a block adds its result to it in the epilogue, and the
         # products that start one normalise it on the way in (the factor applied to their sums)
         for layer in self.layers:
             qkv = ops.spmv_fused(layer.qkv_proj.device_weight(), "rmsnorm", x, None, layer.input_layernorm.weight, eps, layer.qkv_proj.w_scale)
-            pieces = self._attend(qkv, self._cache_of(layer, 0), self._cache_of(layer, 1), pos, False, pieces=True)
-            x = ops.spmv_attn_combine(layer.o_proj.device_weight(), pieces, hd, dtype, layer.o_proj.w_scale, residual=x)
+            if self.split_attention:
+                pieces = self._attend(qkv, self._cache_of(layer, 0), self._cache_of(layer, 1), pos, False, pieces=True)
+                x = ops.spmv_attn_combine(layer.o_proj.device_weight(), pieces, hd, dtype, layer.o_proj.w_scale, residual=x)
+            else:
+                att = self._attend(qkv, self._cache_of(layer, 0), self._cache_of(layer, 1), pos, False, splits=1)
+                x = ops.spmv_add(layer.o_proj.device_weight(), att, x, layer.o_proj.w_scale)
             gated = ops.spmv_fused(layer.gate_up_proj.device_weight(), "rmsnorm", x, None, layer.post_attention_layernorm.weight, eps,
                                    layer.gate_up_proj.w_scale, gated=True)
             x = ops.spmv_add(layer.down_proj.device_weight(), gated, x, layer.down_proj.w_scale)
         return ops.spmv_fused(self.lm_head.device_weight(), "rmsnorm", x, None, self.norm.weight, eps, self.lm_head.w_scale)
 
-    def _attend(self, qkv, k_cache, v_cache, pos, kmajor, pieces=False):
+    def _attend(self, qkv, k_cache, v_cache, pos, kmajor, pieces=False, splits=None):
         """Rotary embedding, cache update and attention for the token whose q | k | v the projection just wrote: one
         launch, or (fused_rope False) the rotary + cache kernel followed by the attention."""
         q, fresh = None, (qkv, self.rope_cos, self.rope_sin)
@@ -261,8 +269,8 @@ class TernaryLlamaDecoder(nn.Module):
             ops.rope_cache_update(qkv, self.rope_cos, self.rope_sin, pos, q, k_cache, v_cache)
             fresh = None
         if pieces:
-            return ops.decode_attention_pieces(q, k_cache, v_cache, pos, fresh=fresh)
-        return ops.decode_attention(q, k_cache, v_cache, pos, kmajor=kmajor, fresh=fresh)
+            return ops.decode_attention_pieces(q, k_cache, v_cache, pos, splits=splits, fresh=fresh)
+        return ops.decode_attention(q, k_cache, v_cache, pos, kmajor=kmajor, splits=splits, fresh=fresh)
 
     def _cache_of(self, layer, which):
         return self._cache[self._layer_index[id(layer)], which]

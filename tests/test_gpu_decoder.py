@@ -476,8 +476,10 @@ def test_fused_single_row_step_equals_the_unfused_one(tiny, cuda):
     tokens = torch.randint(0, tiny.config.vocab_size, (1, 30), generator=g).to(cuda)
     assert tiny.fused_decode
     outs = {}
-    for fused in (False, True):
-        tiny.fused_decode = fused
+    assert not tiny.split_attention   # a short cache: one workgroup per head; the split form is forced below
+    for fused in (False, True, "split"):
+        tiny.fused_decode = bool(fused)
+        tiny.split_attention = fused == "split"
         tiny._graph = None
         tiny.prefill(tokens[:, :28])
         st = tiny._decode_state(1)
@@ -489,9 +491,11 @@ def test_fused_single_row_step_equals_the_unfused_one(tiny, cuda):
             logits.append(tiny._decode_step(st["token"], st["pos"], st["mask"]).float())
         outs[fused] = torch.stack(logits)
     tiny.fused_decode = True
+    tiny.split_attention = False
     tiny._state = None
     tiny._graph = None
     assert (outs[True] - outs[False]).abs().max().item() <= 2e-3 * outs[False].abs().max().item()
+    assert (outs["split"] - outs[False]).abs().max().item() <= 2e-3 * outs[False].abs().max().item()
     eager = tiny.generate(tokens, 10, use_graph=False)
     graphed = tiny.generate(tokens, 10, use_graph=True)
     again = tiny.generate(tokens, 10, use_graph=True)
