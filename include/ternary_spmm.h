@@ -353,6 +353,35 @@ int tl_spmv_fused(const tl_layout_header* header, const void* blob_dev, int prod
 int tl_spmv_add(const tl_layout_header* header, const void* blob_dev, const void* x, int x_dtype, const void* residual,
                 void* Y, int y_dtype, const void* scale, int scale_dtype, void* stream);
 
+/* A decoder layer at 9 to 16 fp16 rows without kernels of its own for the residual add and the RMSNorm (the Hugging
+ * Face decoder layer the reference patches, TernaryLLM/TernaryLlama.py:69-75): the products on either side do them.
+ * The product that ENDS a block (o, down) adds the residual rows and leaves, beside the new residual rows Y, what the
+ * next norm needs: the K-major image of Y[m][n] * next_norm_weight[n] (the activations of the product that follows)
+ * and, per block of 16 columns, the sum of Y[m][n]^2 over the block.  The product that STARTS a block (q|k|v,
+ * gate|up, head) multiplies that image and applies rsqrt(mean square + eps) of each row to its sums -- the
+ * normalisation factor is one number per row, so it can wait until the end (the image is then rounded as
+ * Y * weight, not Y * factor * weight). */
+typedef struct tl_chain {
+    const void* residual;         /* NULL, or [M][residual_ld] of y_dtype: Y = residual + product (may be Y itself) */
+    int64_t residual_ld;
+    const void* next_norm_weight; /* NULL, or [N] of y_dtype; with it: */
+    void* image_out;              /*   K-major [N][image_ld] of y_dtype, image_ld >= M, rows M..image_ld-1 zeroed */
+    int64_t image_ld;
+    float* squares_out;           /*   [ceil(N / 16)][16] */
+    const float* squares_in;      /* NULL, or [squares_blocks][16] as a chained product left them: the rows of X are */
+    int32_t squares_blocks;       /*   those of an image_out, and the sums are scaled by rsqrt(sum / K + eps) per row */
+    float eps;
+} tl_chain;
+
+/* tl_spmm (y_layout < 0) or tl_spmm_gated (y_layout = TL_X_ROW_MAJOR / TL_X_K_MAJOR) with the chain steps above.
+ * TL_ERR_UNSUPPORTED unless 9 <= M <= 16 and x, y are fp16; the residual / image epilogue only in the kernel for
+ * N < 64 * compute units (wider outputs: the separate tl_add_rmsnorm). */
+int tl_spmm_chain(const tl_layout_header* header, const void* blob_dev,
+                  const void* X, int x_dtype, int x_layout, int64_t ldx, int64_t M,
+                  void* Y, int y_dtype, int64_t ldy, int y_layout,
+                  const void* scale, int scale_dtype, const tl_chain* chain,
+                  void* workspace, int64_t workspace_bytes, void* stream);
+
 /* tl_spmv_fused with the epilogue of tl_spmm_gated: the weight's columns are (gate, up) pairs and Y holds the N / 2
  * values silu(y[2j]) * y[2j + 1].  Same arguments otherwise. */
 int tl_spmv_fused_gated(const tl_layout_header* header, const void* blob_dev, int producer,

@@ -26,6 +26,13 @@ ERROR_NAMES = {
 _VALUE_ERRORS = {-1, -2, -3, -4, -7, -8, -9}
 
 
+class Chain(ctypes.Structure):
+    """Mirror of tl_chain (the residual / RMSNorm steps a 9-16-row product may take over)."""
+    _fields_ = [("residual", ctypes.c_void_p), ("residual_ld", ctypes.c_int64), ("next_norm_weight", ctypes.c_void_p),
+                ("image_out", ctypes.c_void_p), ("image_ld", ctypes.c_int64), ("squares_out", ctypes.c_void_p),
+                ("squares_in", ctypes.c_void_p), ("squares_blocks", ctypes.c_int32), ("eps", ctypes.c_float)]
+
+
 class LayoutHeader(ctypes.Structure):
     """Mirror of tl_layout_header (256 bytes)."""
     _fields_ = [
@@ -72,6 +79,7 @@ SIGNATURES = {
     "tl_spmv_fused": (_INT, [_HDRP, _VP, _INT, _VP, _VP, _VP, ctypes.c_float, _VP, _INT, _VP, _INT, _VP, _INT, _VP]),
     "tl_spmv_fused_gated": (_INT, [_HDRP, _VP, _INT, _VP, _VP, _VP, ctypes.c_float, _VP, _INT, _VP, _INT, _VP, _INT, _VP]),
     "tl_spmm_gated": (_INT, [_HDRP, _VP, _VP, _INT, _INT, _I64, _I64, _VP, _INT, _I64, _INT, _VP, _INT, _VP, _I64, _VP]),
+    "tl_spmm_chain": (_INT, [_HDRP, _VP, _VP, _INT, _INT, _I64, _I64, _VP, _INT, _I64, _INT, _VP, _INT, ctypes.POINTER(Chain), _VP, _I64, _VP]),
     "tl_mlp_gate_up": (_INT, [_HDRP, _VP, _HDRP, _VP, _VP, _INT, _INT, _I64, _I64, _VP, _INT, _I64, _VP, _VP, _INT, _INT,
                               _VP, _I64, _VP]),
     "tl_spmm_time": (_INT, [_HDRP, _VP, _VP, _INT, _INT, _I64, _I64, _VP, _INT, _I64, _VP, _INT, _VP, _I64, _VP, _INT,

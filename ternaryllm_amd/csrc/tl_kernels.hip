@@ -84,7 +84,41 @@ struct KernelArgs {
     int gated;
     const void* residual;  // single-row kernels: null, or a row of N values of Y's type: Y[n] = residual[n] + the product (rounded to that type first)
     long long y_kld;      // gated epilogue of the 16-row kernel: 0, or the leading dimension of a K-major output [N / 2][y_kld]
+    // 16-row kernels, a decoder layer without kernels for the residual add and the RMSNorm (tl_spmm_chain):
+    const void* chain_res;    // [M][chain_ldres], Y's type: Y = chain_res + product
+    long long chain_ldres;
+    const void* chain_w;      // [N] weight of the NEXT norm: chain_image[n][m] = Y[m][n] * chain_w[n], chain_sq_out[block][m] = sum over the block's columns of Y[m][n]^2
+    void* chain_image;        // K-major [N][chain_ild], Y's type, rows M .. chain_ild - 1 zeroed
+    long long chain_ild;
+    float* chain_sq_out;      // [NB][16]
+    const float* chain_sq_in; // [chain_sq_blocks][16] sums of squares of the rows X was made from: the product is multiplied by rsqrt(sum / K + eps), row by row
+    int chain_sq_blocks;
 };
+
+// rsqrt(mean square + eps) of the rows behind a chained product.  Called by the first 64 threads of a workgroup (one
+// wave), all of them; lane L gets the factors of rows 4 * (L % 4) .. + 3.  The partial sums [blocks][16] are read as
+// 16-byte pieces, several in flight per lane (one after the other they would cost a trip to memory each).
+__device__ __forceinline__ float4 chain_row_factors(const KernelArgs& a, int lane)
+{
+    const float4* pieces = reinterpret_cast<const float4*>(a.chain_sq_in);  // piece i: block i / 4, rows 4 * (i % 4) .. + 3
+    const int count = a.chain_sq_blocks * 4;
+    constexpr int U = 16;  // pieces of a lane in flight together: 256 blocks (K = 4096) in one trip
+    float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int first = lane; first < count; first += 64 * U) {
+        float4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = first + 64 * u < count ? pieces[first + 64 * u] : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int u = 0; u < U; ++u) { sum.x += v[u].x; sum.y += v[u].y; sum.z += v[u].z; sum.w += v[u].w; }
+    }
+#pragma unroll
+    for (int off = 4; off < 64; off <<= 1) {  // the lanes with the same rows
+        sum.x += __shfl_xor(sum.x, off, 64); sum.y += __shfl_xor(sum.y, off, 64);
+        sum.z += __shfl_xor(sum.z, off, 64); sum.w += __shfl_xor(sum.w, off, 64);
+    }
+    const float k = 1.0f / (float)a.K;
+    return make_float4(rsqrtf(sum.x * k + a.eps), rsqrtf(sum.y * k + a.eps), rsqrtf(sum.z * k + a.eps), rsqrtf(sum.w * k + a.eps));
+}
 
 __device__ __forceinline__ float load_scale(const void* scale, int is_f16, int n)
 {
@@ -637,6 +671,19 @@ __global__ __launch_bounds__(NT) void tl_spmm_quad(KernelArgs a)
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
 
     issue(0, min(TG, a.T), 0);
+    float4 row_factors = make_float4(1.f, 1.f, 1.f, 1.f);  // chained product, first wave: the factors of rows 4 * (lane % 4) .. + 3
+    if (MT == 16 && a.chain_sq_in && tid < 64) row_factors = chain_row_factors(a, tid);
+    // what the chained epilogue of the first wave adds and multiplies, asked for now rather than at the very end
+    float res_early[4] = {0.f, 0.f, 0.f, 0.f}, w_early = 0.f;
+    if (MT == 16 && tid < 64) {
+        const int n = nb * TL_BLOCK_COLUMNS + ((tid / Q) & 15);
+        if (a.chain_res && n < a.N) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if ((tid % Q) * 4 + j < a.M) res_early[j] = load_scale(a.chain_res, a.y_f16, (long long)((tid % Q) * 4 + j) * a.chain_ldres + n);
+        }
+        if (a.chain_image && n < a.N) w_early = load_scale(a.chain_w, a.y_f16, n);
+    }
     int which = 0;
     for (int t = 0; t < a.T; t += TG, which ^= 1) {
         const int nt = min(TG, a.T - t);
@@ -687,12 +734,42 @@ __global__ __launch_bounds__(NT) void tl_spmm_quad(KernelArgs a)
             sum.x += o.x; sum.y += o.y; sum.z += o.z; sum.w += o.w;
         }
         const int n = nb * TL_BLOCK_COLUMNS + c16;
+        const float sc = n < a.N ? load_scale(a.w0.scale, a.scale_f16, n) : 0.f;
+        float out[4] = {sum.x * sc, sum.y * sc, sum.z * sc, sum.w * sc};
+        if constexpr (MT == 16) {
+            // chained products (one wave here: 16 columns x 4 row quads)
+            if (a.chain_sq_in) {  // q == lane % 4: the lane's own rows
+                out[0] *= row_factors.x; out[1] *= row_factors.y; out[2] *= row_factors.z; out[3] *= row_factors.w;
+            }
+            if (a.chain_res) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    if (n < a.N && q * 4 + j < a.M) out[j] = as_output(out[j], a.y_f16) + res_early[j];
+            }
+            if (a.chain_image) {
+                const float w = w_early;
+                float sq[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float v = (n < a.N && q * 4 + j < a.M) ? as_output(out[j], a.y_f16) : 0.f;  // what Y will hold
+                    sq[j] = v * v;
+                    if (n < a.N && q * 4 + j < a.chain_ild) store_out(a.chain_image, a.y_f16, (long long)n * a.chain_ild + q * 4 + j, v * w);
+                }
+#pragma unroll
+                for (int off = 4; off < 64; off <<= 1) {  // over the 16 columns of the block
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) sq[j] += __shfl_xor(sq[j], off, 64);
+                }
+                if (c16 == 0) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) a.chain_sq_out[(size_t)nb * 16 + q * 4 + j] = sq[j];
+                }
+            }
+        }
         if (n < a.N) {
-            const float sc = load_scale(a.w0.scale, a.scale_f16, n);
-            const float out[4] = {sum.x, sum.y, sum.z, sum.w};
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                if (m0 + q * 4 + j < a.M) store_out(a.Y, a.y_f16, (long long)(m0 + q * 4 + j) * a.ldy + n, out[j] * sc);
+                if (m0 + q * 4 + j < a.M) store_out(a.Y, a.y_f16, (long long)(m0 + q * 4 + j) * a.ldy + n, out[j]);
         }
     }
 }
@@ -779,6 +856,8 @@ __global__ __launch_bounds__(kBlockThreads) void tl_spmm_octet(KernelArgs a)
     };
 
     issue(0, min(TG, a.T), 0);
+    float4 row_factors = make_float4(1.f, 1.f, 1.f, 1.f);  // chained product, first wave: the factors of rows 4 * (lane % 4) .. + 3
+    if (a.chain_sq_in && tid < 64) row_factors = chain_row_factors(a, tid);
     int which = 0;
     for (int t = 0; t < a.T; t += TG, which ^= 1) {
         const int nt = min(TG, a.T - t);
@@ -832,7 +911,12 @@ __global__ __launch_bounds__(kBlockThreads) void tl_spmm_octet(KernelArgs a)
         const int n = (nb0 + blk) * TL_BLOCK_COLUMNS + c16;
         const bool real = blk < bs && n < a.N;
         const float sc = real ? load_scale(a.w0.scale, a.scale_f16, n) : 0.f;
-        const float out[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+        float out[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+        if (a.chain_sq_in) {  // rows 8q .. 8q + 7: the row quads of lanes 2q and 2q + 1
+            const float f[4] = {row_factors.x, row_factors.y, row_factors.z, row_factors.w};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) out[j] *= __shfl(f[j & 3], 2 * q + (j >> 2), 64);
+        }
         if (a.gated) {
             // gate and up column of a pair sit two lanes apart (same rows): the even column's lane writes the eight products
             float h[8];
@@ -2219,6 +2303,10 @@ int launch_small(KernelArgs a, const tl_layout_header* h, int x_dtype, void* wor
         // fp16, 16 rows: eight rows per lane and two blocks per workgroup where the workgroups still fill the chip
         const bool octet = mt == 16 && a.x_f16 && knob(TL_OCTET, ceil_div(a.NB, 2) * ceil_div(a.M, 16) >= 2 * (int64_t)compute_units() ? 1 : 0) != 0;
         if (a.gated && !octet) return fail(TL_ERR_UNSUPPORTED, "no gated epilogue in the kernel for M=%d, N=%d (tl_spmm, then tl_silu_mul_pairs)", a.M, a.N);
+        const bool chain_out = a.chain_res || a.chain_image;
+        if ((chain_out || a.chain_sq_in) && (mt != 16 || !a.x_f16 || !a.y_f16 || a.M > 16))
+            return fail(TL_ERR_UNSUPPORTED, "chained products are for 9 to 16 fp16 rows");
+        if (chain_out && octet) return fail(TL_ERR_UNSUPPORTED, "no residual / image epilogue in the kernel for N=%d", a.N);
         if (mt == 8) return a.x_f16 ? launch_quad_kernel<8, true>(a, h, st) : launch_quad_kernel<8, false>(a, h, st);
         if (octet) return launch_octet_kernel(a, h, st);
         if (wide) return a.x_f16 ? launch_quad_kernel<16, true, 1024>(a, h, st) : launch_quad_kernel<16, false, 1024>(a, h, st);
@@ -2229,6 +2317,7 @@ int launch_small(KernelArgs a, const tl_layout_header* h, int x_dtype, void* wor
         knob(TL_SPMV_DIRECT, 1))
         return a.x_f16 ? launch_spmv_direct<true>(a, h, st) : launch_spmv_direct<false>(a, h, st);
     if (a.gated) return fail(TL_ERR_UNSUPPORTED, "no gated epilogue in the kernel for M=%d and this activation layout (tl_spmm, then tl_silu_mul_pairs)", a.M);
+    if (a.chain_res || a.chain_image || a.chain_sq_in) return fail(TL_ERR_UNSUPPORTED, "chained products are for 9 to 16 fp16 rows");
     // Column blocks per workgroup.  A compute unit works through ceil(workgroups / 256) workgroups of
     // `set` blocks each: the narrowest set that keeps that product smallest.
     int set = 1;
@@ -2433,7 +2522,7 @@ namespace {
 // tl_spmm, or (y_layout >= 0) tl_spmm_gated with that output layout
 int spmm_call(const tl_layout_header* header, const void* blob_dev, const void* X, int x_dtype, int x_layout, int64_t ldx, int64_t M,
               void* Y, int y_dtype, int64_t ldy, int y_layout, const void* scale, int scale_dtype, void* workspace, int64_t workspace_bytes,
-              void* stream)
+              void* stream, const tl_chain* chain = nullptr)
 {
     if (int rc = check_header(header)) return rc;
     const bool gated = y_layout >= 0;
@@ -2451,6 +2540,19 @@ int spmm_call(const tl_layout_header* header, const void* blob_dev, const void* 
     std::memset(&a, 0, sizeof(a));
     a.gated = gated;
     if (gated && y_layout == TL_X_K_MAJOR) a.y_kld = ldy;
+    if (chain) {
+        const bool out = chain->next_norm_weight || chain->image_out || chain->squares_out;
+        if (out && !(chain->next_norm_weight && chain->image_out && chain->squares_out))
+            return fail(TL_ERR_ARG, "next_norm_weight, image_out and squares_out come together");
+        if ((out || chain->residual) && gated) return fail(TL_ERR_ARG, "a gated product has no residual or image epilogue");
+        if (M > 16) return fail(TL_ERR_UNSUPPORTED, "chained products are for 9 to 16 fp16 rows");
+        if (chain->residual && chain->residual_ld < (int64_t)header->columns) return fail(TL_ERR_SHAPE, "residual_ld=%lld smaller than N", (long long)chain->residual_ld);
+        if (out && chain->image_ld < M) return fail(TL_ERR_SHAPE, "image_ld=%lld smaller than M", (long long)chain->image_ld);
+        if (chain->squares_in && chain->squares_blocks <= 0) return fail(TL_ERR_ARG, "squares_blocks must be positive");
+        a.chain_res = chain->residual; a.chain_ldres = chain->residual_ld;
+        a.chain_w = chain->next_norm_weight; a.chain_image = chain->image_out; a.chain_ild = chain->image_ld; a.chain_sq_out = chain->squares_out;
+        a.chain_sq_in = chain->squares_in; a.chain_sq_blocks = chain->squares_blocks; a.eps = chain->eps;
+    }
     a.w0 = weight_ptrs(header, blob_dev, scale);
     a.X = X; a.Y = Y;
     a.ldx = ldx; a.ldy = ldy;
@@ -2473,6 +2575,16 @@ extern "C" int tl_spmm(const tl_layout_header* header, const void* blob_dev,
                        void* workspace, int64_t workspace_bytes, void* stream)
 {
     return spmm_call(header, blob_dev, X, x_dtype, x_layout, ldx, M, Y, y_dtype, ldy, -1, scale, scale_dtype, workspace, workspace_bytes, stream);
+}
+
+extern "C" int tl_spmm_chain(const tl_layout_header* header, const void* blob_dev,
+                             const void* X, int x_dtype, int x_layout, int64_t ldx, int64_t M,
+                             void* Y, int y_dtype, int64_t ldy, int y_layout,
+                             const void* scale, int scale_dtype, const tl_chain* chain,
+                             void* workspace, int64_t workspace_bytes, void* stream)
+{
+    if (!chain) return fail(TL_ERR_ARG, "chain is null");
+    return spmm_call(header, blob_dev, X, x_dtype, x_layout, ldx, M, Y, y_dtype, ldy, y_layout, scale, scale_dtype, workspace, workspace_bytes, stream, chain);
 }
 
 extern "C" int tl_spmm_gated(const tl_layout_header* header, const void* blob_dev,

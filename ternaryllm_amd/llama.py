@@ -132,6 +132,9 @@ class TernaryLlamaDecoder(nn.Module):
         # output projection.  That pays once a head's rows are many: up to about a thousand rows one workgroup per
         # head and a plain output projection (the faster single-row kernel) are quicker together.
         self.split_attention = self.max_seq_len > 1024
+        # steps of 9 to 16 fp16 rows: the products do the residual adds and the RMSNorms around them (tl_spmm_chain);
+        # switched off by the first step whose shapes have no such kernel
+        self.chain_decode = dtype == torch.float16
         self._layer_index = {id(layer): i for i, layer in enumerate(self.layers)}
 
     # -- pieces ------------------------------------------------------------------------------
@@ -221,6 +224,13 @@ class TernaryLlamaDecoder(nn.Module):
         if B == 1 and self.fused_decode:
             return self._decode_step_fused(x, pos)
         km = 5 <= B <= 48 and c.hidden_size != B and c.intermediate_size != B
+        if km and 9 <= B <= 16 and self.chain_decode:
+            try:
+                return self._decode_step_chain(x, pos)
+            except RuntimeError as e:
+                if "TL_ERR_UNSUPPORTED" not in str(e) or torch.cuda.is_current_stream_capturing():
+                    raise
+                self.chain_decode = False
         _, h = ops.add_rmsnorm(x, None, self.layers[0].input_layernorm.weight, eps, kmajor=km)
         for li, layer in enumerate(self.layers):
             qkv = layer.qkv_proj(h)
@@ -233,6 +243,30 @@ class TernaryLlamaDecoder(nn.Module):
             nxt = self.layers[li + 1].input_layernorm.weight if li + 1 < len(self.layers) else self.norm.weight
             x, h = ops.add_rmsnorm(x, y, nxt, eps, kmajor=km)  # the residual add, and the norm the next layer (or the head) starts with
         return self.lm_head(h)
+
+    def _decode_step_chain(self, x, pos):
+        """9 to 16 rows, five launches per layer, none of them elementwise: the o and down projections add the residual
+        rows and leave the next norm's image (rows * norm weight) and sums of squares; q|k|v, gate|up (SiLU gate in
+        its epilogue) and the head apply the normalisation factor to their sums.  Only the very first norm has a
+        kernel of its own."""
+        eps = self.config.rms_norm_eps
+        K_MAJOR = _lib.TL_X_K_MAJOR
+        _, h = ops.add_rmsnorm(x, None, self.layers[0].input_layernorm.weight, eps, kmajor=True)
+        squares = None
+        for li, layer in enumerate(self.layers):
+            if squares is None:
+                qkv = layer.qkv_proj(h)
+            else:
+                qkv = ops.spmm_chain(layer.qkv_proj.device_weight(), h, layer.qkv_proj.w_scale, K_MAJOR, squares_in=squares, eps=eps)
+            a = self._attend(qkv, self._cache[li, 0], self._cache[li, 1], pos, True)
+            x, h, squares = ops.spmm_chain(layer.o_proj.device_weight(), a, layer.o_proj.w_scale, K_MAJOR, residual=x,
+                                           next_norm_weight=layer.post_attention_layernorm.weight)
+            gated = ops.spmm_chain(layer.gate_up_proj.device_weight(), h, layer.gate_up_proj.w_scale, K_MAJOR, squares_in=squares, eps=eps,
+                                   gated=True, kmajor=True)
+            nxt = self.layers[li + 1].input_layernorm.weight if li + 1 < len(self.layers) else self.norm.weight
+            x, h, squares = ops.spmm_chain(layer.down_proj.device_weight(), gated, layer.down_proj.w_scale, K_MAJOR, residual=x,
+                                           next_norm_weight=nxt)
+        return ops.spmm_chain(self.lm_head.device_weight(), h, self.lm_head.w_scale, K_MAJOR, squares_in=squares, eps=eps)
 
     def _decode_step_fused(self, x, pos):
         """One row, five launches per layer instead of nine, none of them an elementwise kernel: q|k|v and gate|up

@@ -171,6 +171,65 @@ def spmm_gated(weight, x, scale=None, x_layout=_lib.TL_X_ROW_MAJOR, kmajor=False
     return silu_mul(spmm(weight, x, scale, x_layout=x_layout), kmajor=kmajor, pairs=True)
 
 
+def spmm_chain(weight, x, scale=None, x_layout=_lib.TL_X_ROW_MAJOR, residual=None, next_norm_weight=None, squares_in=None,
+               eps=0.0, gated=False, kmajor=False):
+    """A product of 9 to 16 fp16 rows that takes over the residual add and the RMSNorm around it (tl_spmm_chain), for a
+    decoder layer without elementwise kernels.
+      residual [M, N]: the result is residual + (x @ W) * scale;
+      next_norm_weight [N]: the call also returns the K-major image of result * next_norm_weight (a [N, M] view: the
+        activations of the next product, x_layout=1) and squares [N / 16, 16] float32, per block of 16 columns the sum
+        of result^2 -- what that product needs as squares_in;
+      squares_in: x is such an image; the sums are scaled by rsqrt(mean square + eps) of each row;
+      gated / kmajor: as in spmm_gated (where the kernel for the width has no gated epilogue the gate is a second launch).
+    Returns y, or (y, image, squares) with next_norm_weight.  Raises RuntimeError (TL_ERR_UNSUPPORTED) where the kernel
+    for the shape has no such step."""
+    if x.device != weight.device:
+        raise RuntimeError(f"x is on {x.device}, the weight on {weight.device}")
+    x_code = _code(x.dtype, "x")
+    xg, M, ldx = _x_geometry(x, weight.inners, x_layout)
+    N = weight.columns
+    if kmajor and not gated:
+        raise ValueError("a K-major result is written by the gated epilogue only (next_norm_weight gives the image of a plain product)")
+    width = N // 2 if gated else N
+    if kmajor:
+        y, ldy = _kmajor_image(M, width, x)
+    else:
+        y, ldy = torch.empty((M, width), dtype=x.dtype, device=x.device), width
+    chain = _lib.Chain()
+    keep = []
+    if residual is not None:
+        if residual.shape != (M, N) or residual.dtype != x.dtype or residual.stride(1) != 1 or residual.device != x.device:
+            raise ValueError("residual must be an [M, N] tensor of x's dtype with unit column stride")
+        chain.residual, chain.residual_ld = residual.data_ptr(), residual.stride(0)
+    image = squares = None
+    if next_norm_weight is not None:
+        if next_norm_weight.numel() != N or next_norm_weight.dtype != x.dtype or not next_norm_weight.is_contiguous():
+            raise ValueError("next_norm_weight must be a contiguous [N] tensor of x's dtype")
+        image, ild = _kmajor_image(M, N, x)
+        squares = torch.empty(((N + 15) // 16, 16), dtype=torch.float32, device=x.device)
+        chain.next_norm_weight, chain.image_out, chain.image_ld, chain.squares_out = next_norm_weight.data_ptr(), image.data_ptr(), ild, squares.data_ptr()
+    if squares_in is not None:
+        if squares_in.dtype != torch.float32 or squares_in.dim() != 2 or squares_in.shape[1] != 16 or not squares_in.is_contiguous():
+            raise ValueError("squares_in must be a contiguous float32 [blocks, 16] tensor")
+        chain.squares_in, chain.squares_blocks = squares_in.data_ptr(), squares_in.shape[0]
+    chain.eps = float(eps)
+    sc, s_code = _scale_args(scale, N, x.device)
+    ws, ws_bytes = _workspace(weight.header, M, x_code, x_layout, x.device)
+    y_layout = -1 if not gated else (_lib.TL_X_K_MAJOR if kmajor else _lib.TL_X_ROW_MAJOR)
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().tl_spmm_chain(ctypes.byref(weight.header), weight.blob.data_ptr(), xg.data_ptr(), x_code, x_layout, ldx, M,
+                                      y.data_ptr(), x_code, ldy, y_layout, sc.data_ptr() if sc is not None else None, s_code,
+                                      ctypes.byref(chain), ws.data_ptr() if ws is not None else None, ws_bytes, _stream_ptr(x.device))
+    if rc == _lib.TL_ERR_UNSUPPORTED and gated:
+        # no gated epilogue in the kernel for this width: the gate takes a launch of its own
+        plain = spmm_chain(weight, x, scale, x_layout, squares_in=squares_in, eps=eps)
+        return silu_mul(plain, kmajor=kmajor, pairs=True)
+    _lib.check(rc)
+    if kmajor:
+        y = y[:, :M]
+    return (y, image[:, :M], squares) if next_norm_weight is not None else y
+
+
 def mlp_gate_up(gate, up, x, gate_scale=None, up_scale=None, out_dtype=None):
     """h[M, N] = silu((x @ Wg) * sg) * ((x @ Wu) * su) in one pass over x (M > 48), else two products."""
     if gate.columns != up.columns or gate.inners != up.inners:

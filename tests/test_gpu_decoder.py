@@ -161,6 +161,58 @@ def test_batched_decode_step_on_k_major_activations(tiny, cuda):
     assert (outs[True] - outs[False]).abs().max().item() <= 1e-2 * outs[False].abs().max().item()
 
 
+def test_chained_decode_step_without_elementwise_kernels(tiny, full_width, cuda):
+    """9 to 16 rows: the step whose products do the residual adds and the RMSNorms (tl_spmm_chain) against the step with
+    tl_add_rmsnorm and tl_silu_mul launches, and against torch operators; then the pieces of one chained pair by
+    themselves against a float64 restatement."""
+    from tests.util import max_rel_err, ternary_weight
+    from ternaryllm_amd import ops
+    from ternaryllm_amd.packing import PackedWeight
+    g = torch.Generator().manual_seed(33)
+    for model, B, S in ((tiny, 16, 20), (tiny, 9, 20), (full_width, 16, 6)):
+        tokens = torch.randint(0, model.config.vocab_size, (B, S + 2), generator=g).to(cuda)
+        outs = {}
+        for mode in ("torch", "launches", "chain"):
+            model.native_decode = mode != "torch"
+            model.chain_decode = mode == "chain"
+            model._graph = None
+            model.prefill(tokens[:, :S])
+            st = model._decode_state(B)
+            logits = []
+            for j in range(2):
+                st["token"].copy_(tokens[:, S + j])
+                st["pos"].fill_(S + j)
+                st["mask"].copy_((torch.arange(model.max_seq_len, device=cuda) <= S + j)[None, None, None])
+                logits.append(model._decode_step(st["token"], st["pos"], st["mask"]).float())
+            outs[mode] = torch.stack(logits)
+            if mode == "chain":
+                assert model.chain_decode   # the chained kernels exist for these shapes: nothing fell back
+        model.native_decode, model.chain_decode, model._state, model._graph = True, True, None, None
+        top = outs["torch"].abs().max().item()
+        assert (outs["chain"] - outs["launches"]).abs().max().item() <= 4e-3 * top, (B, (outs["chain"] - outs["launches"]).abs().max().item() / top)
+        assert (outs["chain"] - outs["torch"]).abs().max().item() <= 1e-2 * top
+    # one pair: a product that ends a block, the product behind the norm
+    K, N, N2, M = 1000, 272, 96, 13
+    w1, w2 = ternary_weight(K, N, 0.7, 1), ternary_weight(N, N2, 0.7, 2)
+    d1, d2 = ops.DeviceWeight(PackedWeight.from_dense(w1), cuda), ops.DeviceWeight(PackedWeight.from_dense(w2), cuda)
+    x = torch.randn((M, K), generator=g).half().to(cuda)
+    res = torch.randn((M, N), generator=g).half().to(cuda)
+    nw = (1 + 0.1 * torch.randn(N, generator=g)).half().to(cuda)
+    sc1, sc2 = (0.05 + 0.01 * torch.rand(N, generator=g)).half().to(cuda), (0.5 + torch.rand(N2, generator=g)).half().to(cuda)
+    y, image, squares = ops.spmm_chain(d1, x, sc1, residual=res, next_norm_weight=nw)
+    assert torch.equal(y, ops.spmm(d1, x, sc1) + res)                      # the separate add, bit for bit
+    assert torch.equal(image.t(), (y.float() * nw.float()).half())         # rows * weight, rounded once
+    assert image.stride(0) == 16 and not image.as_strided((N, 16), (16, 1))[:, M:].any()
+    want_sq = y.float().pow(2).reshape(M, N // 16, 16).sum(-1).t()
+    assert torch.allclose(squares[:, :M], want_sq, rtol=1e-5, atol=1e-6)
+    out = ops.spmm_chain(d2, image, sc2, x_layout=1, squares_in=squares, eps=1e-5)
+    h64 = y.double() * torch.rsqrt(y.double().pow(2).mean(-1, keepdim=True) + 1e-5) * nw.double()
+    ref = (h64.cpu().numpy() @ w2.astype("float64")) * sc2.double().cpu().numpy()[None, :]
+    assert max_rel_err(out.double().cpu().numpy(), ref, h64.cpu().numpy(), w2) <= 4e-3
+    with pytest.raises(RuntimeError, match="UNSUPPORTED"):
+        ops.spmm_chain(d1, x[:5], sc1, residual=res[:5])                   # five rows: another kernel
+
+
 def test_decode_kernels_against_fp32(cuda):
     """tl_rope_cache_update and tl_decode_attention alone, fp16 and fp32, against a float64 restatement."""
     from ternaryllm_amd import ops
