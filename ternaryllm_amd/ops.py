@@ -196,7 +196,6 @@ def spmm_chain(weight, x, scale=None, x_layout=_lib.TL_X_ROW_MAJOR, residual=Non
     else:
         y, ldy = torch.empty((M, width), dtype=x.dtype, device=x.device), width
     chain = _lib.Chain()
-    keep = []
     if residual is not None:
         if residual.shape != (M, N) or residual.dtype != x.dtype or residual.stride(1) != 1 or residual.device != x.device:
             raise ValueError("residual must be an [M, N] tensor of x's dtype with unit column stride")
