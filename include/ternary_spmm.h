@@ -365,9 +365,9 @@ typedef struct tl_chain {
     const void* residual;         /* NULL, or [M][residual_ld] of y_dtype: Y = residual + product (may be Y itself) */
     int64_t residual_ld;
     const void* next_norm_weight; /* NULL, or [N] of y_dtype; with it: */
-    void* image_out;              /*   K-major [N][image_ld] of y_dtype, image_ld >= M, rows M..image_ld-1 zeroed */
+    void* image_out;              /*   K-major [N][image_ld] of y_dtype, M <= image_ld <= 16, rows M..image_ld-1 zeroed */
     int64_t image_ld;
-    float* squares_out;           /*   [ceil(N / 16)][16] */
+    float* squares_out;           /*   [ceil(N / 16)][16], 16-byte aligned (as squares_in) */
     const float* squares_in;      /* NULL, or [squares_blocks][16] as a chained product left them: the rows of X are */
     int32_t squares_blocks;       /*   those of an image_out, and the sums are scaled by rsqrt(sum / K + eps) per row */
     float eps;

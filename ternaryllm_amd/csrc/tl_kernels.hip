@@ -2547,8 +2547,14 @@ int spmm_call(const tl_layout_header* header, const void* blob_dev, const void* 
         if ((out || chain->residual) && gated) return fail(TL_ERR_ARG, "a gated product has no residual or image epilogue");
         if (M > 16) return fail(TL_ERR_UNSUPPORTED, "chained products are for 9 to 16 fp16 rows");
         if (chain->residual && chain->residual_ld < (int64_t)header->columns) return fail(TL_ERR_SHAPE, "residual_ld=%lld smaller than N", (long long)chain->residual_ld);
-        if (out && chain->image_ld < M) return fail(TL_ERR_SHAPE, "image_ld=%lld smaller than M", (long long)chain->image_ld);
+        if (out && (chain->image_ld < M || chain->image_ld > 16))  // the epilogue writes (and zeroes) 16 rows of the image at most
+            return fail(TL_ERR_SHAPE, "image_ld=%lld outside M=%lld .. 16", (long long)chain->image_ld, (long long)M);
         if (chain->squares_in && chain->squares_blocks <= 0) return fail(TL_ERR_ARG, "squares_blocks must be positive");
+        const uintptr_t es = y_dtype == TL_F16 ? 2 : 4;
+        for (const void* p : {chain->residual, chain->next_norm_weight, static_cast<const void*>(chain->image_out)})
+            if (reinterpret_cast<uintptr_t>(p) % es) return fail(TL_ERR_ALIGN, "residual, next_norm_weight and image_out must be aligned to y_dtype");
+        for (const void* p : {static_cast<const void*>(chain->squares_out), static_cast<const void*>(chain->squares_in)})
+            if (reinterpret_cast<uintptr_t>(p) % 16) return fail(TL_ERR_ALIGN, "squares_out and squares_in must be 16-byte aligned");
         a.chain_res = chain->residual; a.chain_ldres = chain->residual_ld;
         a.chain_w = chain->next_norm_weight; a.chain_image = chain->image_out; a.chain_ild = chain->image_ld; a.chain_sq_out = chain->squares_out;
         a.chain_sq_in = chain->squares_in; a.chain_sq_blocks = chain->squares_blocks; a.eps = chain->eps;

@@ -191,24 +191,27 @@ def test_chained_decode_step_without_elementwise_kernels(tiny, full_width, cuda)
         top = outs["torch"].abs().max().item()
         assert (outs["chain"] - outs["launches"]).abs().max().item() <= 4e-3 * top, (B, (outs["chain"] - outs["launches"]).abs().max().item() / top)
         assert (outs["chain"] - outs["torch"]).abs().max().item() <= 1e-2 * top
-    # one pair: a product that ends a block, the product behind the norm
-    K, N, N2, M = 1000, 272, 96, 13
-    w1, w2 = ternary_weight(K, N, 0.7, 1), ternary_weight(N, N2, 0.7, 2)
-    d1, d2 = ops.DeviceWeight(PackedWeight.from_dense(w1), cuda), ops.DeviceWeight(PackedWeight.from_dense(w2), cuda)
-    x = torch.randn((M, K), generator=g).half().to(cuda)
-    res = torch.randn((M, N), generator=g).half().to(cuda)
-    nw = (1 + 0.1 * torch.randn(N, generator=g)).half().to(cuda)
-    sc1, sc2 = (0.05 + 0.01 * torch.rand(N, generator=g)).half().to(cuda), (0.5 + torch.rand(N2, generator=g)).half().to(cuda)
-    y, image, squares = ops.spmm_chain(d1, x, sc1, residual=res, next_norm_weight=nw)
-    assert torch.equal(y, ops.spmm(d1, x, sc1) + res)                      # the separate add, bit for bit
-    assert torch.equal(image.t(), (y.float() * nw.float()).half())         # rows * weight, rounded once
-    assert image.stride(0) == 16 and not image.as_strided((N, 16), (16, 1))[:, M:].any()
-    want_sq = y.float().pow(2).reshape(M, N // 16, 16).sum(-1).t()
-    assert torch.allclose(squares[:, :M], want_sq, rtol=1e-5, atol=1e-6)
-    out = ops.spmm_chain(d2, image, sc2, x_layout=1, squares_in=squares, eps=1e-5)
-    h64 = y.double() * torch.rsqrt(y.double().pow(2).mean(-1, keepdim=True) + 1e-5) * nw.double()
-    ref = (h64.cpu().numpy() @ w2.astype("float64")) * sc2.double().cpu().numpy()[None, :]
-    assert max_rel_err(out.double().cpu().numpy(), ref, h64.cpu().numpy(), w2) <= 4e-3
+    # one pair: a product that ends a block, the product behind the norm; widths that are and are not whole blocks of 16
+    for K, N, N2, M in ((1000, 272, 96, 13), (520, 270, 40, 9), (300, 43, 33, 16)):
+        w1, w2 = ternary_weight(K, N, 0.7, 1), ternary_weight(N, N2, 0.7, 2)
+        d1, d2 = ops.DeviceWeight(PackedWeight.from_dense(w1), cuda), ops.DeviceWeight(PackedWeight.from_dense(w2), cuda)
+        x = torch.randn((M, K), generator=g).half().to(cuda)
+        res = torch.randn((M, N), generator=g).half().to(cuda)
+        nw = (1 + 0.1 * torch.randn(N, generator=g)).half().to(cuda)
+        sc1, sc2 = (0.05 + 0.01 * torch.rand(N, generator=g)).half().to(cuda), (0.5 + torch.rand(N2, generator=g)).half().to(cuda)
+        y, image, squares = ops.spmm_chain(d1, x, sc1, residual=res, next_norm_weight=nw)
+        assert torch.equal(y, ops.spmm(d1, x, sc1) + res)                      # the separate add, bit for bit
+        assert torch.equal(image.t(), (y.float() * nw.float()).half())         # rows * weight, rounded once
+        assert image.stride(0) == 16 and not image.as_strided((N, 16), (16, 1))[:, M:].any()
+        blocks = -(-N // 16)
+        padded = torch.zeros((M, blocks * 16), device=cuda)
+        padded[:, :N] = y.float().pow(2)
+        assert squares.shape[0] == blocks
+        assert torch.allclose(squares[:, :M], padded.reshape(M, blocks, 16).sum(-1).t(), rtol=1e-5, atol=1e-6)
+        out = ops.spmm_chain(d2, image, sc2, x_layout=1, squares_in=squares, eps=1e-5)
+        h64 = y.double() * torch.rsqrt(y.double().pow(2).mean(-1, keepdim=True) + 1e-5) * nw.double()
+        ref = (h64.cpu().numpy() @ w2.astype("float64")) * sc2.double().cpu().numpy()[None, :]
+        assert max_rel_err(out.double().cpu().numpy(), ref, h64.cpu().numpy(), w2) <= 4e-3, (K, N, N2, M)
     with pytest.raises(RuntimeError, match="UNSUPPORTED"):
         ops.spmm_chain(d1, x[:5], sc1, residual=res[:5])                   # five rows: another kernel
 
