@@ -1409,6 +1409,41 @@ __global__ __launch_bounds__(256) void tl_relayout_x(const T* __restrict__ X, lo
     }
 }
 
+// The same image from row-major fp16 rows whose 16-byte pieces are whole and aligned (K and ldx multiples of 8):
+// 16 bytes per lane on both sides.  A workgroup turns 128 rows x 64 inner positions; a thread loads the same
+// piece of two neighbouring rows and writes them to LDS as (row 2p, row 2p + 1) pairs, one dword per position.
+__global__ __launch_bounds__(256) void tl_relayout_rows_h(const __half* __restrict__ X, long long ldx, __half* __restrict__ XT,
+                                                          long long ldm, int M, int K)
+{
+    constexpr int TM = 128, TK = 64, PITCH = TM + 8;  // halves; a row of the turned tile is 272 bytes, whole 16-byte pieces
+    __shared__ __align__(16) __half tile[TK][PITCH];
+    const int k0 = blockIdx.x * TK, m0 = blockIdx.y * TM, tid = threadIdx.x;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int e = tid + 256 * i, p = e >> 3, c = e & 7;  // row pair p of 64, piece c of 8
+        const int m = m0 + 2 * p, k = k0 + 8 * c;
+        u32x4 lo = {0u, 0u, 0u, 0u}, hi = {0u, 0u, 0u, 0u};
+        if (k < K) {
+            if (m < M) lo = *reinterpret_cast<const u32x4*>(X + (long long)m * ldx + k);
+            if (m + 1 < M) hi = *reinterpret_cast<const u32x4*>(X + (long long)(m + 1) * ldx + k);
+        }
+        const uint32_t* l = reinterpret_cast<const uint32_t*>(&lo);
+        const uint32_t* h = reinterpret_cast<const uint32_t*>(&hi);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {  // dword j holds positions 2j, 2j + 1 of both rows
+            *reinterpret_cast<uint32_t*>(&tile[8 * c + 2 * j][2 * p]) = (l[j] & 0xffffu) | (h[j] << 16);
+            *reinterpret_cast<uint32_t*>(&tile[8 * c + 2 * j + 1][2 * p]) = (l[j] >> 16) | (h[j] & 0xffff0000u);
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int e = tid + 256 * i, k = e >> 4, mc = e & 15;  // position k of 64, piece mc of 16
+        if (k0 + k < K)
+            *reinterpret_cast<u32x4*>(XT + (long long)(k0 + k) * ldm + m0 + 8 * mc) = *reinterpret_cast<const u32x4*>(&tile[k][8 * mc]);
+    }
+}
+
 // ---------------------------------------------------------------------------
 // Row-parallel kernel.
 // ---------------------------------------------------------------------------
@@ -2443,7 +2478,10 @@ int launch_rows(KernelArgs a, int x_dtype, void* workspace, int64_t workspace_by
             return fail(TL_ERR_SIZE, "workspace has %lld bytes, %lld needed", (long long)workspace_bytes, (long long)need);
         if (reinterpret_cast<uintptr_t>(workspace) % 16) return fail(TL_ERR_ALIGN, "workspace must be 16-byte aligned");
         dim3 tgrid((unsigned)ceil_div(a.K, 64), (unsigned)(ldm / 64));
-        if (x_dtype == TL_F16)
+        if (x_dtype == TL_F16 && !a.x_kmajor && a.K % 8 == 0 && a.ldx % 8 == 0 && reinterpret_cast<uintptr_t>(a.X) % 16 == 0)
+            hipLaunchKernelGGL(tl_relayout_rows_h, dim3((unsigned)ceil_div(a.K, 64), (unsigned)(ldm / 128)), dim3(256), 0, st,
+                               static_cast<const __half*>(a.X), a.ldx, static_cast<__half*>(workspace), ldm, a.M, a.K);
+        else if (x_dtype == TL_F16)
             hipLaunchKernelGGL(tl_relayout_x<__half>, tgrid, dim3(256), 0, st, static_cast<const __half*>(a.X), a.ldx, a.x_kmajor,
                                static_cast<__half*>(workspace), ldm, a.M, a.K);
         else
