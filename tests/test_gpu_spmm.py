@@ -31,7 +31,7 @@ SHAPES = [
     (1, 512, 256, 0.66), (1, 4096, 4096, 0.66), (2, 1000, 130, 0.5), (3, 777, 65, 0.8), (5, 4096, 1024, 0.9),
     (8, 2048, 512, 0.8), (16, 4096, 4096, 0.5), (17, 1024, 320, 0.66), (33, 600, 200, 0.8), (48, 512, 512, 0.9),
     (49, 512, 192, 0.8), (64, 1024, 256, 0.66), (100, 777, 130, 0.5), (256, 2048, 512, 0.8), (300, 4096, 1000, 0.9),
-    (1024, 4096, 1024, 0.8),
+    (1024, 4096, 1024, 0.8), (77, 520, 96, 0.7),
 ]
 
 
