@@ -12,6 +12,7 @@
 //     (block, tile): 16 descriptors followed by the block's runs.  What a workgroup needs
 //     for a range of tiles is then a single contiguous piece of memory.
 #include <climits>
+#include <cmath>
 #include <cstring>
 #include <algorithm>
 #include <vector>
@@ -95,15 +96,16 @@ int count_device_tiles(const int32_t* row, const int32_t* off_tiled, int columns
 }
 
 // Order of the rows inside runs.  The sum does not depend on it; the single-row kernel's speed does: a lane
-// reads one activation per index from the LDS image of its tile, 64 lanes at a time, and reads that fall on
-// one LDS bank (of 32, four bytes wide) but on different words are served one after the other.  That kernel
-// works on neighbouring tiles of a column side by side, four lanes to a run (lane l on dwords l, l + 4, ... of
-// the +1 run followed by the -1 run); all lanes read byte b of their k-th dword together.  So the rows of
-// a group of 8 tiles (32 lanes) are dealt out read by read: each lane takes from what is left of its run the
-// row whose bank the read has used least so far (the padding bytes, which read the tile's zero slot, are
+// reads one activation per index from the LDS image of its tile, and the LDS serves half a wave, 32 lanes, at a
+// time: reads of those 32 that fall on one LDS bank (of 32, four bytes wide) but on different words are served
+// one after the other.  The plain single-row kernel (tl_spmv_tiles) gives a wave a whole tile: 16 columns, four
+// lanes to a run (lane l on dwords l, l + 4, ... of the +1 run followed by the -1 run), lanes 0-31 on columns
+// 0-7 of the block; all lanes read byte b of their k-th dword together.  So the rows of a group of 8
+// neighbouring columns of a tile (32 lanes) are dealt out read by read: each lane takes from what is left of its
+// run the row whose bank the read has used least so far (the padding bytes, which read the tile's zero slot, are
 // counted first); then rows are swapped between the reads of a run while that lowers the number of lanes
-// that share a bank.  Blobs whose runs are longer on average get more lanes per run from the kernel; the
-// order is then no better than any other, and no worse.
+// that share a bank.  Kernels with another lane assignment (tiles side by side in tl_spmv_direct, more lanes
+// per run for long runs) find an order that is no better than any other, and no worse.
 struct RunRef {
     uint8_t* bytes;  // start of the +1 run (the -1 run follows its padded end)
     int n_pos, n_neg;
@@ -111,7 +113,7 @@ struct RunRef {
 };
 
 constexpr int kLanesPerRun = 4;
-constexpr int kSpreadSweeps = 1;
+constexpr int kSpreadSweeps = 2;
 
 // LDS bank of a row's activation in the single-row kernel: fp16 values, two to a bank word; the image of
 // tile t starts kSpmvImageSkew bytes further round the banks than that of tile t - 1 (tl_common.h).
@@ -163,36 +165,73 @@ void spread_over_banks(const RunRef* runs, int n_runs, int sweeps)
                 run.bytes[(neg ? 4 * pd : 0) + e] = row;
             }
     }
-    // swaps inside a run, between two of its reads, that lower the sum of squared bank loads
+    // Swaps inside a run, between two of its reads.  What a read costs is the largest number of different words that
+    // any one bank has to deliver (lanes on the same word are served together), so a read with one shared bank
+    // costs as much as a read with five: the swaps move shared banks out of the reads that have few of them and
+    // into reads that have some already.  Potential of a read: sqrt(banks with two words or more) + 10 * (words
+    // beyond two on a bank).
+    struct ReadState {
+        uint8_t words[128];  // lanes per word of the tile image (two fp16 rows to a word)
+        uint8_t per_bank[32];
+        int two, three;      // banks that deliver two or more different words; words beyond two, summed over the banks
+    };
+    std::vector<ReadState> state((size_t)reads);
+    std::memset(state.data(), 0, state.size() * sizeof(ReadState));
+    auto add = [&](int q, int word, int tile) {
+        ReadState& s = state[(size_t)q];
+        if (s.words[word]++ == 0) {
+            const int n = ++s.per_bank[bank_of((uint8_t)(word * 2), tile)];
+            s.two += n == 2;
+            s.three += n >= 3;
+        }
+    };
+    auto drop = [&](int q, int word, int tile) {
+        ReadState& s = state[(size_t)q];
+        if (--s.words[word] == 0) {
+            const int n = s.per_bank[bank_of((uint8_t)(word * 2), tile)]--;
+            s.two -= n == 2;
+            s.three -= n >= 3;
+        }
+    };
+    float root[33];
+    for (int i = 0; i <= 32; ++i) root[i] = std::sqrt((float)i);
+    auto potential = [&](int q) { return root[state[(size_t)q].two] + 10.0f * (float)state[(size_t)q].three; };
+    for (int r = 0; r < n_runs; ++r) {
+        const RunRef& run = runs[r];
+        const int pd = (run.n_pos + 3) / 4, nd = (run.n_neg + 3) / 4;
+        for (int e = 0; e < 4 * (pd + nd); ++e) add(((e / 4) / kLanesPerRun) * 4 + (e & 3), run.bytes[e] >> 1, run.tile);
+    }
     for (int sweep = 0; sweep < sweeps; ++sweep) {
         bool any = false;
         for (int r = 0; r < n_runs; ++r) {
             const RunRef& run = runs[r];
-            const int pd = (run.n_pos + 3) / 4;
+            const int pd = (run.n_pos + 3) / 4, tile = run.tile;
             for (int sign = 0; sign < 2; ++sign) {
                 uint8_t* rows = run.bytes + (sign ? 4 * pd : 0);
                 const int n = sign ? run.n_neg : run.n_pos;
                 const int first_dword = sign ? pd : 0;
                 auto read_of = [&](int e) { return ((first_dword + e / 4) / kLanesPerRun) * 4 + (e & 3); };
                 for (int e1 = 0; e1 < n; ++e1) {
-                    const int q1 = read_of(e1), b1 = bank_of(rows[e1], run.tile);
-                    if (load[(size_t)q1 * 32 + b1] < 2) continue;  // alone on its bank: nothing to gain
-                    int best = -1, best_gain = 0;
+                    const int q1 = read_of(e1), w1 = rows[e1] >> 1, b1 = bank_of(rows[e1], tile);
+                    // only a row that is alone on its word, on a bank that delivers another word too, is worth moving
+                    if (state[(size_t)q1].words[w1] != 1 || state[(size_t)q1].per_bank[b1] < 2) continue;
+                    int best = -1;
+                    float best_gain = 1e-6f;
                     for (int e2 = 0; e2 < n; ++e2) {
                         const int q2 = read_of(e2);
                         if (q2 == q1) continue;
-                        const int b2 = bank_of(rows[e2], run.tile);
-                        if (b1 == b2) continue;
-                        // before: l(q1,b1), l(q1,b2), l(q2,b1), l(q2,b2); moving b1 to q2 and b2 to q1
-                        const int a = load[(size_t)q1 * 32 + b1], b = load[(size_t)q1 * 32 + b2];
-                        const int c = load[(size_t)q2 * 32 + b1], d = load[(size_t)q2 * 32 + b2];
-                        const int gain = 2 * (a - 1 - b) + 2 * (d - 1 - c);  // decrease of the sum of squares
+                        const int w2 = rows[e2] >> 1, b2 = bank_of(rows[e2], tile);
+                        // the row that comes must not bring a shared bank of its own
+                        if (b2 == b1 || (state[(size_t)q1].words[w2] == 0 && state[(size_t)q1].per_bank[b2] != 0)) continue;
+                        const float before = potential(q1) + potential(q2);
+                        drop(q1, w1, tile); add(q1, w2, tile); drop(q2, w2, tile); add(q2, w1, tile);
+                        const float gain = before - potential(q1) - potential(q2);
+                        drop(q2, w1, tile); add(q2, w2, tile); drop(q1, w2, tile); add(q1, w1, tile);
                         if (gain > best_gain) { best_gain = gain; best = e2; }
                     }
                     if (best >= 0) {
-                        const int q2 = read_of(best), b2 = bank_of(rows[best], run.tile);
-                        --load[(size_t)q1 * 32 + b1]; ++load[(size_t)q1 * 32 + b2];
-                        --load[(size_t)q2 * 32 + b2]; ++load[(size_t)q2 * 32 + b1];
+                        const int q2 = read_of(best), w2 = rows[best] >> 1;
+                        drop(q1, w1, tile); add(q1, w2, tile); drop(q2, w2, tile); add(q2, w1, tile);
                         std::swap(rows[e1], rows[best]);
                         any = true;
                     }
@@ -324,17 +363,20 @@ extern "C" int tl_layout_build(const int32_t* neg_row, const int32_t* neg_off_ti
                     bytes[cursor[2 * (k / g.tile_rows) + sign]++] = (uint8_t)(k % g.tile_rows);
                 }
         }
-        // the column is complete: order the rows inside every group of 8 neighbouring tiles (the 32 lanes that
-        // the single-row kernel puts on them read together)
-        for (int t0 = 0; t0 < T; t0 += 8) {
-            const int gsz = std::min(8, T - t0);
-            for (int i = 0; i < gsz; ++i) {
-                const uint64_t c0 = chunkstart[(size_t)nb * T + t0 + i];
-                const uint32_t d = stream[c0 + j];
-                runs[i] = RunRef{bytes + (c0 + (d >> 16)) * 4, (int)(d & 0xff), (int)((d >> 8) & 0xff), t0 + i};
+        // the block is complete: order the rows inside every group of 8 neighbouring columns of a tile (the single-row
+        // kernel puts 32 lanes, half a wave, on them: four per column, and the LDS serves half a wave at a time)
+        if (j == kBlock - 1 || y == columns - 1)
+            for (int t = 0; t < T; ++t) {
+                const uint64_t c0 = chunkstart[(size_t)nb * T + t];
+                for (int j0 = 0; j0 <= j; j0 += 8) {
+                    const int gsz = std::min(8, j + 1 - j0);
+                    for (int i = 0; i < gsz; ++i) {
+                        const uint32_t d = stream[c0 + j0 + i];
+                        runs[i] = RunRef{bytes + (c0 + (d >> 16)) * 4, (int)(d & 0xff), (int)((d >> 8) & 0xff), t};
+                    }
+                    spread_over_banks(runs.data(), gsz, kSpreadSweeps);
+                }
             }
-            spread_over_banks(runs.data(), gsz, kSpreadSweeps);
-        }
     }
 
     tl_layout_header h;
