@@ -1090,8 +1090,10 @@ __global__ __launch_bounds__(NT) void tl_spmv_direct(KernelArgs a)
 
     const int lpc_shift = a.lpc_shift, lw_shift = a.lw_shift;
     const int LPC = 1 << lpc_shift, LW = 1 << lw_shift, TP = LPC >> lw_shift;
-    const int c16 = tid >> lpc_shift, lig = tid & (LPC - 1);
-    const int tp = lig >> lw_shift, lw = lig & (LW - 1);
+    // The LW lanes of a run sit side by side, the 16 columns of a tile next to each other, the TP tiles that are worked on
+    // together one after the other: with four lanes per run a wave reads one tile, 8 neighbouring columns per half wave
+    // -- the lanes that the packer's order of the rows inside runs keeps off each other's LDS banks.
+    const int c16 = (tid >> lw_shift) & (TL_BLOCK_COLUMNS - 1), lw = tid & (LW - 1), tp = tid >> (lw_shift + 4);
     float acc[1] = {0.f};
     constexpr int TU = 2;  // tiles of one lane whose LDS reads are issued together
 
@@ -1184,21 +1186,26 @@ __global__ __launch_bounds__(NT) void tl_spmv_direct(KernelArgs a)
             }
         }
     }
+    // fold: the LW lanes of a run by shuffles, the TP sums of a column through LDS (no wave may still be gathering from it)
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1)
-        if (off < LPC) acc[0] += __shfl_xor(acc[0], off, 64);
-    const int n = nb * TL_BLOCK_COLUMNS + c16;
-    if (a.gated) {
-        // the 16 column sums of the block meet in LDS (no wave may still be gathering from it), eight products go out
-        __syncthreads();
-        float* sums = reinterpret_cast<float*>(lds);
-        if (lig == 0) sums[c16] = n < a.N ? as_output(acc[0] * load_scale(a.w0.scale, a.scale_f16, n), a.y_f16) : 0.f;
-        __syncthreads();
-        if (tid < TL_BLOCK_COLUMNS / 2 && nb * TL_BLOCK_COLUMNS + 2 * tid + 1 < a.N)
-            store_out(a.Y, a.y_f16, nb * (TL_BLOCK_COLUMNS / 2) + tid, gate_pair(sums[2 * tid], sums[2 * tid + 1], a.y_f16));
-        return;
+    for (int off = 1; off < 64; off <<= 1)
+        if (off < LW) acc[0] += __shfl_xor(acc[0], off, 64);
+    __syncthreads();
+    float* red = reinterpret_cast<float*>(lds);  // [TP][16]
+    if (lw == 0) red[tp * TL_BLOCK_COLUMNS + c16] = acc[0];
+    __syncthreads();
+    if (tid < TL_BLOCK_COLUMNS) {
+        float sum = 0.f;
+        for (int i = 0; i < TP; ++i) sum += red[i * TL_BLOCK_COLUMNS + tid];
+        const int n = nb * TL_BLOCK_COLUMNS + tid;
+        if (a.gated) {
+            const float y = n < a.N ? as_output(sum * load_scale(a.w0.scale, a.scale_f16, n), a.y_f16) : 0.f;
+            const float up = __shfl_xor(y, 1, 64);  // the odd neighbour's
+            if (!(tid & 1) && n + 1 < a.N) store_out(a.Y, a.y_f16, n / 2, gate_pair(y, up, a.y_f16));
+            return;
+        }
+        if (n < a.N) store_result(a, n, sum * load_scale(a.w0.scale, a.scale_f16, n));
     }
-    if (lig == 0 && n < a.N) store_result(a, n, acc[0] * load_scale(a.w0.scale, a.scale_f16, n));
 }
 
 // ---------------------------------------------------------------------------

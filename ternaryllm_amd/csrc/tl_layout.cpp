@@ -104,8 +104,9 @@ int count_device_tiles(const int32_t* row, const int32_t* off_tiled, int columns
 // neighbouring columns of a tile (32 lanes) are dealt out read by read: each lane takes from what is left of its
 // run the row whose bank the read has used least so far (the padding bytes, which read the tile's zero slot, are
 // counted first); then rows are swapped between the reads of a run while that lowers the number of lanes
-// that share a bank.  Kernels with another lane assignment (tiles side by side in tl_spmv_direct, more lanes
-// per run for long runs) find an order that is no better than any other, and no worse.
+// that share a bank.  tl_spmv_direct assigns its lanes the same way; kernels with another assignment (more
+// lanes per run for long runs, the 8- and 16-row kernels) find an order that is no better than any other, and
+// no worse.
 struct RunRef {
     uint8_t* bytes;  // start of the +1 run (the -1 run follows its padded end)
     int n_pos, n_neg;
