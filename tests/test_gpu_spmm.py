@@ -118,6 +118,39 @@ def test_k_major_input_and_tile_heights(cuda, oracle):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("M", [49, 200, 257])
+def test_row_kernel_activation_layouts(cuda, oracle, M, dtype):
+    """Every way activations reach the row-parallel kernel: contiguous rows of whole 16-byte pieces (the 16-byte-per-lane
+    re-layout for fp16), rows with an odd leading dimension or an odd K (the element-wise re-layout), a K-major image
+    padded to the row tile (no pre-pass) and K-major with an odd leading dimension."""
+    from ternaryllm_amd import ops
+    from ternaryllm_amd.packing import PackedWeight
+    for K, N in ((520, 96), (777, 50)):
+        w = ternary_weight(K, N, 0.7, 43 + K)
+        dw = ops.DeviceWeight(PackedWeight.from_dense(w), cuda)
+        x = activations(M, K, 44 + M, dtype, integer=True)
+        ref = oracle.fast_product(x.double().numpy(), w)
+        xd = x.to(cuda)
+        cases = {"row-major": (xd, 0)}
+        wide = torch.zeros((M, K + 3), dtype=dtype, device=cuda)           # rows with an odd leading dimension
+        wide[:, :K] = xd
+        cases["row-major, strided"] = (wide[:, :K], 0)
+        wide8 = torch.zeros((M, K + 8), dtype=dtype, device=cuda)          # aligned rows further apart than K
+        wide8[:, :K] = xd
+        cases["row-major, aligned stride"] = (wide8[:, :K], 0)
+        padded = torch.zeros((K, -(-M // 256) * 256), dtype=dtype, device=cuda)  # the kernel's own layout
+        padded[:, :M] = xd.t()
+        cases["k-major, padded"] = (padded[:, :M], 1)
+        widek = torch.zeros((K, M + 5), dtype=dtype, device=cuda)          # K-major with an odd leading dimension
+        widek[:, :M] = xd.t()
+        cases["k-major, strided"] = (widek[:, :M], 1)
+        for name, (xin, layout) in cases.items():
+            print(f"case M={M} K={K} dtype={dtype} {name}", flush=True)
+            y = ops.spmm(dw, xin, x_layout=layout).float().cpu().numpy()
+            assert np.array_equal(y.astype(np.float64), ref), (M, K, name)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 @pytest.mark.parametrize("M", [1, 3, 4, 9, 16, 40])
 def test_small_m_activation_layouts(cuda, oracle, M, dtype):
     """Every way the small-M kernel stages activations: whole row vectors, single elements (odd leading
