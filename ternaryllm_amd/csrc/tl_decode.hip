@@ -10,6 +10,7 @@
 
 #include <algorithm>
 #include <atomic>
+#include <climits>
 
 #include "tl_common.h"
 
@@ -509,6 +510,7 @@ extern "C" int tl_rope_cache_update(const void* qkv, int dtype, int64_t batch, i
     if (int rc = check_common(dtype, batch, heads, head_dim, max_seq, pos_dev)) return rc;
     if (!qkv || !cos_table || !sin_table || !q_out || !k_cache || !v_cache) return fail(TL_ERR_ARG, "device pointer is null");
     const int64_t total = batch * heads * head_dim;
+    if (ceil_div(total, 256) > INT32_MAX) return fail(TL_ERR_SHAPE, "batch x heads x head_dim = %lld is more than one launch takes", (long long)total);
     dim3 grid((unsigned)ceil_div(total, 256));
     hipStream_t st = static_cast<hipStream_t>(stream);
     const long long* pos = reinterpret_cast<const long long*>(pos_dev);
@@ -632,6 +634,8 @@ int silu_mul_call(const void* gate_up, int dtype, int64_t rows, int width, void*
     if (rows <= 0 || width <= 0 || rows * width > (1ll << 40)) return fail(TL_ERR_SHAPE, "rows and width must be positive");
     if (out_kmajor_ld && out_kmajor_ld < rows) return fail(TL_ERR_SHAPE, "out_kmajor_ld=%lld is less than the rows", (long long)out_kmajor_ld);
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (out_kmajor_ld > (1ll << 40) / width || ceil_div((out_kmajor_ld ? out_kmajor_ld : rows) * width, 256) > INT32_MAX)
+        return fail(TL_ERR_SHAPE, "rows x width is more than one launch takes");
     const unsigned blocks = (unsigned)ceil_div((out_kmajor_ld ? out_kmajor_ld : rows) * width, 256);
     if (dtype == TL_F16)
         hipLaunchKernelGGL(tl_silu_mul_k<__half>, dim3(blocks), dim3(256), 0, st, static_cast<const __half*>(gate_up), static_cast<__half*>(out),
