@@ -375,6 +375,17 @@ def main():
         torch.cuda.synchronize()
         mlp_ms = (time.perf_counter() - t0) * 1e3 / 10
         extra["c3_mlp_block_fused"] = {"ms": round(mlp_ms, 4), "tokens_per_s": round(M / (mlp_ms * 1e-3), 1)}
+        # the same block on one gate|up weight of (gate, up) column pairs, the gate in that product's epilogue
+        mlp.paired = True
+        for _ in range(3):
+            mlp(xb)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(10):
+            mlp(xb)
+        torch.cuda.synchronize()
+        pair_ms = (time.perf_counter() - t0) * 1e3 / 10
+        extra["c3_mlp_block_pairs"] = {"ms": round(pair_ms, 4), "tokens_per_s": round(M / (pair_ms * 1e-3), 1)}
     if not args.no_extra and not args.only_decoder:
         if not only:
             extra["balanced_vs_iid_weights"] = balanced_leg(dev, args.steps, args.warmup)

@@ -427,9 +427,11 @@ int tl_silu_mul_pairs(const void* gate_up, int dtype, int64_t rows, int width, v
  * rounded to y_dtype where those would store them), without the launch and the trip through memory.
  *   y_layout   TL_X_ROW_MAJOR: Y [M][ldy], ldy >= N / 2;  TL_X_K_MAJOR: Y [N / 2][ldy], ldy >= M, rows M..ldy-1
  *              zeroed -- the image tl_spmm multiplies 5 to 48 rows from (9 to 16 rows only)
- * The kernels with this epilogue are those of M = 1 (a contiguous aligned row) and of 9 to 16 fp16 rows with
- * N >= 64 * compute units; any other call returns TL_ERR_UNSUPPORTED and the two separate calls do the work
- * (for more than 48 rows and separate gate and up weights there is tl_mlp_gate_up). */
+ * The kernels with this epilogue are those of M = 1 (a contiguous aligned row), of fp16 rows in groups of 16
+ * (9 to 48 rows) with N >= 64 * compute units, and of more than 48 rows (row-major Y); any other call returns
+ * TL_ERR_UNSUPPORTED and the two separate calls do the work.  (For separate gate and up weights and more than
+ * 48 rows there is tl_mlp_gate_up; the paired weight is the faster of the two, one launch over twice the
+ * columns.) */
 int tl_spmm_gated(const tl_layout_header* header, const void* blob_dev,
                   const void* X, int x_dtype, int x_layout, int64_t ldx, int64_t M,
                   void* Y, int y_dtype, int64_t ldy, int y_layout,

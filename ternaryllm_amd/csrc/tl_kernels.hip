@@ -1730,7 +1730,7 @@ __device__ __forceinline__ void regs_to_lds(const u32x4 (&pf)[PER], unsigned cha
 // free by now): lanes write their C columns of a row side by side, then the workgroup stores whole
 // rows of WAVES * C columns, 8 or 16 bytes per lane.  Output tiles that the matrix edge cuts, or whose
 // rows are not aligned for that, are stored value by value.
-template <typename XT, int R, int C, int WAVES, bool GATED>
+template <typename XT, int R, int C, int WAVES, bool GATED, bool PAIRS>
 __device__ __forceinline__ void rows_store(const KernelArgs& a, int m0, int n_wg, int wave, int lane, const float (&acc)[C][R],
                                            const float (&acc2)[GATED ? C : 1][R], unsigned char* smem)
 {
@@ -1738,6 +1738,69 @@ __device__ __forceinline__ void rows_store(const KernelArgs& a, int m0, int n_wg
     constexpr int COLS = WAVES * C;
     static_assert(C % 4 == 0, "the staged store moves groups of four columns per lane");
     const int n0 = n_wg + wave * C;
+    if constexpr (PAIRS) {
+        // One weight whose columns are (gate, up) pairs: a wave's C columns are C / 2 whole pairs, and column n / 2 of
+        // the output is silu(y[n]) * y[n + 1], both rounded to the output type first, as the product followed by
+        // the pairs form of the SiLU kernel rounds.  The tile that goes out is half as wide.
+        static_assert(!GATED && C % 8 == 0, "pairs of the plain kernel's columns, four outputs per lane and staged piece");
+        constexpr int HC = C / 2, HCOLS = COLS / 2;
+        float h[HC][R];
+#pragma unroll
+        for (int p = 0; p < HC; ++p) {
+            const int n = min(n0 + 2 * p, a.N - 1), nu = min(n0 + 2 * p + 1, a.N - 1);
+            const float sg = load_scale(a.w0.scale, a.scale_f16, n), su = load_scale(a.w0.scale, a.scale_f16, nu);
+#pragma unroll
+            for (int j = 0; j < R; ++j)
+                h[p][j] = gate_pair(as_output(acc[2 * p][j] * sg, a.y_f16), as_output(acc[2 * p + 1][j] * su, a.y_f16), a.y_f16);
+        }
+        const int es = a.y_f16 ? 2 : 4;
+        const int stride = HCOLS * es + 4 * es;
+        const bool whole = n_wg + COLS <= a.N && (a.ldy * es) % (4 * es) == 0 &&
+                           (reinterpret_cast<uintptr_t>(a.Y) + (size_t)(n_wg / 2) * es) % (4 * es) == 0 &&
+                           (size_t)MTILE * stride <= (size_t)kSentinel * MTILE * sizeof(XT);
+        if (!whole) {
+#pragma unroll
+            for (int p = 0; p < HC; ++p) {
+                const int n = n0 + 2 * p;
+                if (n + 1 >= a.N) continue;
+#pragma unroll
+                for (int j = 0; j < R; ++j) {
+                    const int m = m0 + R * lane + j;
+                    if (m < a.M) store_out(a.Y, a.y_f16, (long long)m * a.ldy + n / 2, h[p][j]);
+                }
+            }
+            return;
+        }
+        __syncthreads();  // every wave is done reading the activation tile
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+            const int r = R * lane + j;
+#pragma unroll
+            for (int g = 0; g < HC; g += 4) {
+                unsigned char* dst = smem + (size_t)r * stride + (size_t)(wave * HC + g) * es;
+                if (a.y_f16) {
+                    const __half2 lo = __floats2half2_rn(settled(h[g][j]), settled(h[g + 1][j])), hi = __floats2half2_rn(settled(h[g + 2][j]), settled(h[g + 3][j]));
+                    *reinterpret_cast<uint2*>(dst) = make_uint2(*reinterpret_cast<const uint32_t*>(&lo), *reinterpret_cast<const uint32_t*>(&hi));
+                } else {
+                    *reinterpret_cast<float4*>(dst) = make_float4(h[g][j], h[g + 1][j], h[g + 2][j], h[g + 3][j]);
+                }
+            }
+        }
+        __syncthreads();
+        constexpr int LANES_PER_ROW = HCOLS / 4;
+        constexpr int ROWS_PER_PASS = WAVES * 64 / LANES_PER_ROW;
+        const int q = (int)threadIdx.x % LANES_PER_ROW, r0 = (int)threadIdx.x / LANES_PER_ROW;
+#pragma unroll
+        for (int r = r0; r < MTILE; r += ROWS_PER_PASS) {
+            const int m = m0 + r;
+            if (m >= a.M) continue;
+            const unsigned char* src = smem + (size_t)r * stride + (size_t)q * 4 * es;
+            unsigned char* out = static_cast<unsigned char*>(a.Y) + ((size_t)m * a.ldy + n_wg / 2 + q * 4) * es;
+            if (a.y_f16) *reinterpret_cast<uint2*>(out) = *reinterpret_cast<const uint2*>(src);
+            else *reinterpret_cast<float4*>(out) = *reinterpret_cast<const float4*>(src);
+        }
+        return;
+    }
     float v[C][R];
 #pragma unroll
     for (int c = 0; c < C; ++c) {
@@ -1814,7 +1877,7 @@ __device__ __forceinline__ float* partial_slot(float* base, int lin, int which)
 __device__ __host__ inline long long split_begin(long long lin, long long S, long long G) { return lin * S / G; }
 __device__ __host__ inline long long split_owner(long long step, long long S, long long G) { return ((step + 1) * G - 1) / S; }
 
-template <typename XT, int R, int C, int WAVES, bool GATED>
+template <typename XT, int R, int C, int WAVES, bool GATED, bool PAIRS = false>
 __global__ __launch_bounds__(WAVES * 64) void tl_spmm_rows(KernelArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -1906,7 +1969,7 @@ __global__ __launch_bounds__(WAVES * 64) void tl_spmm_rows(KernelArgs a)
         }
 
         if (t0 == 0 && t1 == a.T) {
-            rows_store<XT, R, C, WAVES, GATED>(a, m0, (unit % n_col_tiles) * (WAVES * C), wave, lane, acc, acc2, smem);
+            rows_store<XT, R, C, WAVES, GATED, PAIRS>(a, m0, (unit % n_col_tiles) * (WAVES * C), wave, lane, acc, acc2, smem);
         } else {
             float* part = partial_slot<R, C, WAVES, GATED>(a.partial, lin, t0 > 0 ? 0 : 1);
 #pragma unroll
@@ -1922,7 +1985,7 @@ __global__ __launch_bounds__(WAVES * 64) void tl_spmm_rows(KernelArgs a)
 
 // One workgroup per shared-out output tile: adds up the partial sums its workgroups left and finishes
 // the tile (nothing to do when the whole tile fell into one workgroup's share).
-template <typename XT, int R, int C, int WAVES, bool GATED>
+template <typename XT, int R, int C, int WAVES, bool GATED, bool PAIRS = false>
 __global__ __launch_bounds__(WAVES * 64) void tl_rows_fixup(KernelArgs a, int G)
 {
     constexpr int MTILE = 64 * R;
@@ -1957,7 +2020,7 @@ __global__ __launch_bounds__(WAVES * 64) void tl_rows_fixup(KernelArgs a, int G)
             }
     }
     extern __shared__ __align__(16) unsigned char smem[];
-    rows_store<XT, R, C, WAVES, GATED>(a, m0, (unit % n_col_tiles) * (WAVES * C), wave, lane, acc, acc2, smem);
+    rows_store<XT, R, C, WAVES, GATED, PAIRS>(a, m0, (unit % n_col_tiles) * (WAVES * C), wave, lane, acc, acc2, smem);
 }
 
 // ---------------------------------------------------------------------------
@@ -2408,13 +2471,13 @@ int launch_small(KernelArgs a, const tl_layout_header* h, int x_dtype, void* wor
 constexpr int64_t kRowsPartialBytes = (int64_t)kMaxComputeUnits * 2 * 2 * kRowsWaves * kRowsCols * 4 * 64 * sizeof(float);
 static_assert(kRowsColsPlain == 2 * kRowsCols, "one accumulator set of the plain kernel is as large as the fused kernel's two");
 
-template <typename XT, int R, bool GATED>
+template <typename XT, int R, bool GATED, bool PAIRS = false>
 int launch_rows_t(KernelArgs a, void* partial, int64_t partial_bytes, hipStream_t st)
 {
     constexpr int MTILE = 64 * R;
     const size_t lds = (size_t)kTileSlots * MTILE * sizeof(XT);
     constexpr int COLS = GATED ? kRowsCols : kRowsColsPlain;
-    auto kernel = tl_spmm_rows<XT, R, COLS, kRowsWaves, GATED>;
+    auto kernel = tl_spmm_rows<XT, R, COLS, kRowsWaves, GATED, PAIRS>;
     static bool raised = false;  // per instantiation; a repeated call is harmless
     if (!raised) {
         // the kernel addresses its activation tile from LDS offset 0: it must own no static LDS
@@ -2443,7 +2506,7 @@ int launch_rows_t(KernelArgs a, void* partial, int64_t partial_bytes, hipStream_
         hipLaunchKernelGGL(kernel, dim3((unsigned)G), dim3(kRowsWaves * 64), lds, st, a);
         // LDS of the fix-up: the staged output tile (fp32 at most, padded rows)
         const size_t fix_lds = (size_t)MTILE * (kRowsWaves * COLS * 4 + 16);
-        auto fixup = tl_rows_fixup<XT, R, COLS, kRowsWaves, GATED>;
+        auto fixup = tl_rows_fixup<XT, R, COLS, kRowsWaves, GATED, PAIRS>;
         static bool fix_raised = false;
         if (!fix_raised) {
             if (int rc = raise_lds_limit(fixup, fix_lds)) return rc;
@@ -2508,6 +2571,11 @@ int launch_rows(KernelArgs a, int x_dtype, void* workspace, int64_t workspace_by
     if (workspace && workspace_bytes >= image + kRowsPartialBytes) {
         partial = static_cast<unsigned char*>(workspace) + image;
         partial_bytes = workspace_bytes - image;
+    }
+    if (a.gated) {  // one weight with (gate, up) column pairs: the plain kernel with the pair epilogue
+        if (gated) return fail(TL_ERR_ARG, "the two-weight kernel has its own gate");
+        return x_dtype == TL_F16 ? launch_rows_t<__half, 4, false, true>(a, partial, partial_bytes, st)
+                                 : launch_rows_t<float, 2, false, true>(a, partial, partial_bytes, st);
     }
     if (x_dtype == TL_F16)
         return gated ? launch_rows_t<__half, 4, true>(a, partial, partial_bytes, st) : launch_rows_t<__half, 4, false>(a, partial, partial_bytes, st);
@@ -2578,7 +2646,6 @@ int spmm_call(const tl_layout_header* header, const void* blob_dev, const void* 
         if (header->columns % 2) return fail(TL_ERR_SHAPE, "N=%u: gate and up columns come in pairs", header->columns);
         const int64_t min_ldy = y_layout == TL_X_K_MAJOR ? M : (int64_t)header->columns / 2;
         if (ldy < min_ldy) return fail(TL_ERR_SHAPE, "ldy=%lld smaller than %lld", (long long)ldy, (long long)min_ldy);
-        if (M > kSmallMaxM) return fail(TL_ERR_UNSUPPORTED, "no gated epilogue for M=%lld (tl_spmm, then tl_silu_mul_pairs; or tl_mlp_gate_up)", (long long)M);
         if (y_layout == TL_X_K_MAJOR && (M <= 8 || M > 16)) return fail(TL_ERR_UNSUPPORTED, "a K-major gated output is written for 9 to 16 rows");
     }
     KernelArgs a;

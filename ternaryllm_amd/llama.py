@@ -145,8 +145,9 @@ class TernaryLlamaDecoder(nn.Module):
         return x * cos + rot * sin
 
     def _mlp(self, layer, x2):
-        gu = layer.gate_up_proj(x2)   # columns 2j, 2j + 1: gate and up of output j
-        return layer.down_proj(torch.nn.functional.silu(gu[:, 0::2]) * gu[:, 1::2])
+        # columns 2j, 2j + 1 of the gate|up weight are gate and up of output j: the product's epilogue applies the gate
+        gated = ops.spmm_gated(layer.gate_up_proj.device_weight(), x2, layer.gate_up_proj.w_scale)
+        return layer.down_proj(gated)
 
     def allocate_cache(self, batch):
         c = self.config

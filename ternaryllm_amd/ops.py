@@ -143,8 +143,9 @@ def spmm(weight, x, scale=None, out_dtype=None, x_layout=_lib.TL_X_ROW_MAJOR, ou
 def spmm_gated(weight, x, scale=None, x_layout=_lib.TL_X_ROW_MAJOR, kmajor=False):
     """h[M, N / 2] with h[:, j] = silu(y[:, 2j]) * y[:, 2j + 1], y = (x @ W) * scale, for a gate | up weight whose
     columns are (gate, up) pairs.  One launch (tl_spmm_gated) where the shape's kernel has the epilogue -- one
-    aligned row, or 9 to 16 fp16 rows and a wide N -- else the product followed by silu_mul(pairs=True); the result
-    is the same bit for bit.  With kmajor the transpose [N / 2, M] is returned, a view of a K-major image."""
+    aligned row, 9 to 16 fp16 rows and a wide N, or more than 48 rows -- else the product followed by
+    silu_mul(pairs=True); the result is the same bit for bit.  With kmajor the transpose [N / 2, M] is returned, a
+    view of a K-major image."""
     if x.device != weight.device:
         raise RuntimeError(f"x is on {x.device}, the weight on {weight.device}")
     if weight.columns % 2:
@@ -152,8 +153,7 @@ def spmm_gated(weight, x, scale=None, x_layout=_lib.TL_X_ROW_MAJOR, kmajor=False
     x_code = _code(x.dtype, "x")
     xg, M, ldx = _x_geometry(x, weight.inners, x_layout)
     half = weight.columns // 2
-    fused = M == 1 or (9 <= M <= 16 and x.dtype == torch.float16)
-    if fused and not (kmajor and M == 1):
+    if not (kmajor and (M == 1 or M > 16)):  # the library says TL_ERR_UNSUPPORTED where the shape's kernel has no such epilogue
         if kmajor:
             out, ld = _kmajor_image(M, half, x)
         else:

@@ -453,8 +453,8 @@ def test_fused_producers_of_the_single_row_product(cuda, oracle, dtype, tol):
 def test_silu_gate_in_the_epilogue_of_the_gate_up_product(cuda):
     """tl_spmm_gated / tl_spmv_fused_gated on a weight whose columns are (gate, up) pairs against the product followed
     by tl_silu_mul_pairs: bit for bit -- one row (both single-row kernels, with and without a producer), 9 to 16 fp16
-    rows on a wide output (row-major and as a K-major image with zeroed padding rows), and the shapes without the
-    epilogue, which take the two launches."""
+    rows on a wide output (row-major and as a K-major image with zeroed padding rows), more than 48 rows (the
+    row-parallel kernel), and the shapes without the epilogue, which take the two launches."""
     import ctypes
     from tests.util import knobs, ternary_weight
     from ternaryllm_amd import _lib, ops
@@ -513,12 +513,33 @@ def test_silu_gate_in_the_epilogue_of_the_gate_up_product(cuda):
     # shapes whose kernels have no such epilogue: same result from two launches
     x32 = torch.randn((16, K), generator=g).to(cuda)
     assert fused_rc(dw, x32, 16) == _lib.TL_ERR_UNSUPPORTED
-    for x in (torch.randn((5, K), generator=g).half().to(cuda), torch.randn((3, K), generator=g).half().to(cuda),
-              torch.randn((60, K), generator=g).half().to(cuda), x32):
+    for x in (torch.randn((5, K), generator=g).half().to(cuda), torch.randn((3, K), generator=g).half().to(cuda), x32):
         assert fused_rc(dw, x, x.shape[0]) == _lib.TL_ERR_UNSUPPORTED
         assert torch.equal(ops.spmm_gated(dw, x, sc.to(x.dtype)), ops.silu_mul(ops.spmm(dw, x, sc.to(x.dtype)), pairs=True))
+    # 17 to 48 fp16 rows on a wide output: the eight-rows-per-lane kernel, one workgroup per 16 rows
+    x40 = torch.randn((40, K), generator=g).half().to(cuda)
+    assert fused_rc(dw, x40, 40) == 0
+    assert torch.equal(ops.spmm_gated(dw, x40, sc), ops.silu_mul(ops.spmm(dw, x40, sc), pairs=True))
     narrow = ops.DeviceWeight(PackedWeight.from_dense(ternary_weight(K, 96, 0.8, 6)), cuda)
     assert fused_rc(narrow, torch.zeros((16, K), dtype=torch.float16, device=cuda), 16) == _lib.TL_ERR_UNSUPPORTED
+    # more than 48 rows: the row-parallel kernel with the pair epilogue, whole output tiles and tiles that the matrix
+    # edge cuts, with and without K tiles shared out among the workgroups
+    sc96 = (0.5 + torch.rand(96, generator=g)).half().to(cuda)
+    for dtype in (torch.float16, torch.float32):
+        for M in (60, 300, 1100):
+            x = torch.randn((M, K), generator=g).to(dtype).to(cuda)
+            for weight, scale in ((dw, sc), (narrow, sc96)):
+                assert fused_rc(weight, x, M) == 0
+                for setting in ({}, {"TL_ROWS_SPLIT": "0"}):
+                    with knobs(**setting):
+                        got = ops.spmm_gated(weight, x, scale.to(dtype))
+                        want = ops.silu_mul(ops.spmm(weight, x, scale.to(dtype)), pairs=True)
+                    assert got.shape == (M, weight.columns // 2)
+                    assert torch.equal(got, want), (dtype, M, weight.columns, setting)
+    image = torch.empty((dw.columns // 2, 64), dtype=torch.float16, device=cuda)
+    x60 = torch.zeros((60, K), dtype=torch.float16, device=cuda)
+    assert L.tl_spmm_gated(ctypes.byref(dw.header), dw.blob.data_ptr(), x60.data_ptr(), 1, 0, K, 60, image.data_ptr(), 1, 64, 1, None, 0,
+                           None, 0, None) == _lib.TL_ERR_UNSUPPORTED   # no K-major image of that many rows
     odd = ops.DeviceWeight(PackedWeight.from_dense(ternary_weight(K, 33, 0.8, 7)), cuda)
     with pytest.raises(ValueError, match="pairs"):
         ops.spmm_gated(odd, torch.zeros((1, K), dtype=torch.float16, device=cuda))

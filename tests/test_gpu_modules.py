@@ -190,6 +190,12 @@ def test_mlp_block_fp16(cuda, tokens):
     # y carries the rounding of h (fp16) through ~280 signed adds per output: compare on the output's RMS scale
     err_y = (y[0].double().cpu() - y_ref).abs() / y_ref.abs().clamp_min(y_ref.pow(2).mean().sqrt())
     assert err_y.max().item() <= 4 * FP16_TOL
+    # the same block on one weight of (gate, up) column pairs with the gate in the product's epilogue
+    mlp.paired = True
+    yp = mlp(x.to(cuda).reshape(1, tokens, 512))
+    assert yp.shape == y.shape and mlp._pairs[0].columns == 2 * 1408
+    err_p = (yp[0].double().cpu() - y_ref).abs() / y_ref.abs().clamp_min(y_ref.pow(2).mean().sqrt())
+    assert err_p.max().item() <= 4 * FP16_TOL
 
 
 def test_attention_block_against_torch(cuda):
