@@ -297,7 +297,7 @@ def main():
         "tokens_per_s": round(M / (wall_ms * 1e-3), 1),
         "roofline": {"bound": "hbm", "achieved": round(B / (ev_ms * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(B / (ev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 5), "traffic": traffic, "traffic_note": traffic_note,
-                     "kernel": "tl_relayout_rows_h + tl_spmm_rows<__half, 4, 8, 16, false> + tl_rows_fixup<__half, 4, 8, 16, false> "
+                     "kernel": "tl_relayout_rows_h + tl_spmm_rows<__half, 4, 8, 16, false, false> + tl_rows_fixup<__half, 4, 8, 16, false, false> "
                                "(the three launches of one tl_spmm call on row-major activations)",
                      "kernel_ms": round(ev_ms, 5)},
     }
