@@ -1737,6 +1737,10 @@ __device__ __forceinline__ void rows_store(const KernelArgs& a, int m0, int n_wg
     constexpr int MTILE = 64 * R;
     constexpr int COLS = WAVES * C;
     static_assert(C % 4 == 0, "the staged store moves groups of four columns per lane");
+    // The store's addresses are worked out here: left to the compiler they are computed at the top of the kernel and
+    // spilled across the tile loop (a dozen dwords per thread of scratch traffic, written and read back).
+    int tid = (int)threadIdx.x;
+    asm volatile("" : "+v"(tid), "+v"(lane));
     const int n0 = n_wg + wave * C;
     if constexpr (PAIRS) {
         // One weight whose columns are (gate, up) pairs: a wave's C columns are C / 2 whole pairs, and column n / 2 of
@@ -1789,7 +1793,7 @@ __device__ __forceinline__ void rows_store(const KernelArgs& a, int m0, int n_wg
         __syncthreads();
         constexpr int LANES_PER_ROW = HCOLS / 4;
         constexpr int ROWS_PER_PASS = WAVES * 64 / LANES_PER_ROW;
-        const int q = (int)threadIdx.x % LANES_PER_ROW, r0 = (int)threadIdx.x / LANES_PER_ROW;
+        const int q = tid % LANES_PER_ROW, r0 = tid / LANES_PER_ROW;
 #pragma unroll
         for (int r = r0; r < MTILE; r += ROWS_PER_PASS) {
             const int m = m0 + r;
@@ -1850,7 +1854,7 @@ __device__ __forceinline__ void rows_store(const KernelArgs& a, int m0, int n_wg
     __syncthreads();
     constexpr int LANES_PER_ROW = COLS / 4;             // each lane moves four columns
     constexpr int ROWS_PER_PASS = WAVES * 64 / LANES_PER_ROW;
-    const int q = (int)threadIdx.x % LANES_PER_ROW, r0 = (int)threadIdx.x / LANES_PER_ROW;
+    const int q = tid % LANES_PER_ROW, r0 = tid / LANES_PER_ROW;
 #pragma unroll
     for (int r = r0; r < MTILE; r += ROWS_PER_PASS) {
         const int m = m0 + r;
