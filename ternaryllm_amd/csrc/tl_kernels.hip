@@ -605,6 +605,49 @@ void tl_spmm_block(KernelArgs a)
     }
 }
 
+// The activation images of a group of tiles, global -> LDS, for tl_spmm_quad and tl_spmm_octet.  Piece p = p0 + tid of
+// the group (16 bytes; VPS pieces per slot, 256 slots per tile) belongs to tile p / PT, slot (p % PT) / VPS.  NT and
+// PT = 256 * VPS are powers of two, so the part of that which depends on the thread is the same in every turn of the
+// loop: it is worked out once per kernel (ImageLane), and a turn adds a wave-uniform base address -- two or three
+// vector instructions per piece instead of the 64-bit multiplications of the full address.
+struct ImageLane {
+    int tile, row;      // the thread's tile within a turn (workgroups wider than a tile) and its slot's share of the row index
+    uint32_t offset;    // bytes from the turn's base address to the thread's piece
+};
+
+template <int VPS, int NT>
+__device__ __forceinline__ ImageLane image_lane(const KernelArgs& a, int tid, size_t row_bytes)
+{
+    constexpr int PT = kTileSlots * VPS;
+    ImageLane l;
+    l.tile = NT >= PT ? tid / PT : 0;
+    const int rem = NT >= PT ? tid % PT : tid;
+    l.row = rem / VPS;
+    l.offset = (uint32_t)(l.tile * a.tile_rows + l.row) * (uint32_t)row_bytes + (uint32_t)(rem % VPS) * 16u;
+    return l;
+}
+
+template <int VPS, int NT>
+__device__ __forceinline__ void issue_images(const KernelArgs& a, const unsigned char* Xb, size_t row_bytes, unsigned char* xs, int t, int nt,
+                                             int wave, int lane, const ImageLane& l)
+{
+    using global_ptr = const __attribute__((address_space(1))) void*;
+    using lds_ptr = __attribute__((address_space(3))) void*;
+    constexpr int PT = kTileSlots * VPS;
+    const int pieces = nt * PT;  // a multiple of 64: whole waves
+    for (int p0 = 0; p0 + wave * 64 < pieces; p0 += NT) {
+        const int first = p0 + wave * 64;
+        const int tile_u = p0 / PT, row_u = (p0 % PT) / VPS;  // wave-uniform: the turn's first tile and row
+        const int r = row_u + l.row, k = (t + tile_u + l.tile) * a.tile_rows + r;
+        if (r < a.tile_rows && k < a.K) {
+            const unsigned char* base = Xb + ((size_t)(t + tile_u) * a.tile_rows + row_u) * row_bytes;
+            __builtin_amdgcn_global_load_lds((global_ptr)(base + l.offset), (lds_ptr)(xs + (size_t)first * 16), 16, 0, 0);
+        } else {
+            *reinterpret_cast<u32x4*>(xs + (size_t)(first + lane) * 16) = u32x4{0u, 0u, 0u, 0u};
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------
 // Small-M kernel for slots of 8 and 16 rows, staged by direct global -> LDS loads.
 // ---------------------------------------------------------------------------
@@ -644,18 +687,11 @@ __global__ __launch_bounds__(NT) void tl_spmm_quad(KernelArgs a)
     using lds_ptr = __attribute__((address_space(3))) void*;
 
     // global -> LDS buffer `which` for the tiles [t, t + nt)
+    const ImageLane image = image_lane<VPS, NT>(a, tid, row_bytes);
     auto issue = [&](int t, int nt, int which) {
         unsigned char* xs = lds + which * stage_bytes;
         unsigned char* buf = xs + a.xs_bytes;
-        const int pieces = nt * kTileSlots * VPS;  // a multiple of 64: whole waves
-        for (int first = wave * 64; first < pieces; first += NT) {
-            const int p = first + lane, slot = p / VPS, v = p % VPS;
-            const int r = slot & (kTileSlots - 1), k = (t + (slot >> 8)) * a.tile_rows + r;
-            if (r < a.tile_rows && k < a.K)
-                __builtin_amdgcn_global_load_lds((global_ptr)(Xb + (size_t)k * row_bytes + v * 16), (lds_ptr)(xs + (size_t)first * 16), 16, 0, 0);
-            else
-                *reinterpret_cast<u32x4*>(xs + (size_t)p * 16) = u32x4{0u, 0u, 0u, 0u};
-        }
+        issue_images<VPS, NT>(a, Xb, row_bytes, xs, t, nt, wave, lane, image);
         const uint32_t lo = cs[t];
         const int vectors = (int)((cs[t + nt] - lo) / 4);
         for (int first = wave * 64; first < vectors; first += NT)
@@ -806,6 +842,8 @@ __global__ __launch_bounds__(kBlockThreads) void tl_spmm_octet(KernelArgs a)
     auto issue = [&](int t, int nt, int which) {
         unsigned char* xs = lds + which * stage_bytes;
         unsigned char* buf = xs + a.xs_bytes;
+        // (the full address per piece: the precomputed lane shares of tl_spmm_quad would take this kernel past 80
+        // registers, a wave per SIMD less)
         const int pieces = nt * kTileSlots * VPS;  // a multiple of 64: whole waves
         for (int first = wave * 64; first < pieces; first += NT) {
             const int p = first + lane, slot = p / VPS, v = p % VPS;
