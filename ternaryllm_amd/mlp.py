@@ -46,8 +46,9 @@ class LlamaTernaryMLP(nn.Module):
             both = torch.empty((g.shape[0], 2 * g.shape[1]), dtype=torch.int32)
             both[:, 0::2], both[:, 1::2] = g, u
             scale = None
-            if self.gate_proj.w_scale is not None or self.up_proj.w_scale is not None:
-                ones = torch.ones(g.shape[1], dtype=torch.float16, device=device)
+            given = [t for t in (self.gate_proj.w_scale, self.up_proj.w_scale) if t is not None]
+            if given:  # a projection without a scale counts as one of ones, in the other's type
+                ones = torch.ones(g.shape[1], dtype=given[0].dtype, device=device)
                 sg = self.gate_proj.w_scale if self.gate_proj.w_scale is not None else ones
                 su = self.up_proj.w_scale if self.up_proj.w_scale is not None else ones
                 scale = torch.stack([sg.to(device), su.to(device).to(sg.dtype)], 1).reshape(-1).contiguous()
