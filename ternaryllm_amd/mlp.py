@@ -21,7 +21,7 @@ class LlamaTernaryMLP(nn.Module):
         super().__init__()
         self.config = config
         self.paired = paired
-        self._pairs = None  # (DeviceWeight, scale or None) of the paired weight
+        self._pairs = None  # (DeviceWeight, scale or None, what it was built from) of the paired weight
         self.hidden_size = config.hidden_size
         self.intermediate_size = config.intermediate_size
         if config.hidden_act != "silu":
@@ -41,7 +41,9 @@ class LlamaTernaryMLP(nn.Module):
 
     def _paired_weight(self, device):
         """The (gate, up) pair weight on `device`: column 2j the gate, column 2j + 1 the up projection of output j."""
-        if self._pairs is None or self._pairs[0].blob.device != device:
+        # built again when the device or either projection's packed buffer changes (a move, a state_dict load)
+        key = (device, self.gate_proj.w_packed.data_ptr(), self.up_proj.w_packed.data_ptr())
+        if self._pairs is None or self._pairs[2] != key:
             g, u = self.gate_proj.ternary_weight, self.up_proj.ternary_weight
             both = torch.empty((g.shape[0], 2 * g.shape[1]), dtype=torch.int32)
             both[:, 0::2], both[:, 1::2] = g, u
@@ -52,8 +54,8 @@ class LlamaTernaryMLP(nn.Module):
                 sg = self.gate_proj.w_scale if self.gate_proj.w_scale is not None else ones
                 su = self.up_proj.w_scale if self.up_proj.w_scale is not None else ones
                 scale = torch.stack([sg.to(device), su.to(device).to(sg.dtype)], 1).reshape(-1).contiguous()
-            self._pairs = (ops.DeviceWeight(PackedWeight.from_dense(both.numpy()), device), scale)
-        return self._pairs
+            self._pairs = (ops.DeviceWeight(PackedWeight.from_dense(both.numpy()), device), scale, key)
+        return self._pairs[:2]
 
     def forward(self, x):
         lead = x.shape[:-1]
