@@ -63,9 +63,9 @@ const char* tl_last_error(void);
 int tl_version(void);
 
 /* The launchers' tuning knobs (environment variables TL_SMALL_LDS, TL_TILE_GROUP, TL_QUAD_SHARE, TL_LW,
- * TL_SPMV_SHARE, TL_SPMV_WIDE, TL_SMALL_MT, TL_SPMV_DIRECT, TL_BLOCK_SET, TL_ROWS_SPLIT; unset = the
- * launcher's own choice) are read once per process.  This reads them again -- for tests and tuning runs
- * that change them between calls. */
+ * TL_SPMV_SHARE, TL_SPMV_WIDE, TL_SPMV_TILES, TL_SMALL_MT, TL_SPMV_DIRECT, TL_BLOCK_SET, TL_ROWS_SPLIT,
+ * TL_OCTET, TL_QUAD_WIDE, TL_RES16; unset = the launcher's own choice) are read once per process.  This
+ * reads them again -- for tests and tuning runs that change them between calls. */
 int tl_reload_options(void);
 
 /* ======================================================================== */
@@ -133,8 +133,8 @@ int tl_tiled_mcsc_to_dense(const void* merged_row, int index_width, int64_t n_in
 /*     then added that many times) and may sit in both runs (it cancels):   */
 /*     a blob built from dense ternary weights holds every row once, one    */
 /*     built from the reference's merged arrays holds what they encode.     */
-/*     The builder orders the rows of a run so that the single-row kernel's */
-/*     LDS reads spread over the banks.                                     */
+/*     The builder orders the rows of a run so that the LDS reads of the    */
+/*     single-row kernel and of the 16-row kernel spread over the banks.    */
 /*   - the stream is block-major: all tiles of block 0, then block 1, ...;  */
 /*     chunkstart[block * T + tile] is the dword where a chunk begins       */
 /*     (one extra entry marks the end).                                     */

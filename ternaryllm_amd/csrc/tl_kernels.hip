@@ -41,6 +41,7 @@ namespace {
 // Loads through this pointer type may use the scalar (constant) path when the address is wave-uniform.
 typedef const __attribute__((address_space(4))) uint32_t* const_u32_ptr;
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));  // one 16-byte chunk in registers
+typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));  // the same, loaded from a dword-aligned address
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Wold-style-cast"
 __device__ __forceinline__ const_u32_ptr as_const(const uint32_t* p) { return (const_u32_ptr)p; }
@@ -648,6 +649,60 @@ __device__ __forceinline__ void issue_images(const KernelArgs& a, const unsigned
     }
 }
 
+// What the chained epilogue of a 16-row block adds and multiplies: the residual values of a lane's four rows of
+// column n and the next norm's weight of that column.  Asked for early, so that they are there at the very end.
+struct ChainOperands {
+    float res[4];
+    float w;
+};
+
+__device__ __forceinline__ ChainOperands chain_operands(const KernelArgs& a, int n, int q)
+{
+    ChainOperands o = {{0.f, 0.f, 0.f, 0.f}, 0.f};
+    if (a.chain_res && n < a.N) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (q * 4 + j < a.M) o.res[j] = load_scale(a.chain_res, a.y_f16, (long long)(q * 4 + j) * a.chain_ldres + n);
+    }
+    if (a.chain_image && n < a.N) o.w = load_scale(a.chain_w, a.y_f16, n);
+    return o;
+}
+
+// The chained part of the way out of a block of 16 columns x 16 rows.  Called by one whole wave: lane = column
+// c16 = lane / 4 of block nb (n = its column), rows 4q .. 4q + 3 (q = lane % 4); `out` = the lane's four sums times
+// the column's scale on the way in, what Y gets on the way out.
+__device__ __forceinline__ void chain_epilogue16(const KernelArgs& a, int nb, int n, int c16, int q, float (&out)[4], const float4& row_factors,
+                                                 const ChainOperands& early)
+{
+    if (a.chain_sq_in) {  // q == lane % 4: the lane's own rows
+        out[0] *= row_factors.x; out[1] *= row_factors.y; out[2] *= row_factors.z; out[3] *= row_factors.w;
+    }
+    if (a.chain_res) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (n < a.N && q * 4 + j < a.M) out[j] = as_output(out[j], a.y_f16) + early.res[j];
+    }
+    if (a.chain_image) {
+        const float w = early.w;
+        float sq[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float v = (n < a.N && q * 4 + j < a.M) ? as_output(out[j], a.y_f16) : 0.f;  // what Y will hold
+            sq[j] = v * v;
+            if (n < a.N && q * 4 + j < a.chain_ild) store_out(a.chain_image, a.y_f16, (long long)n * a.chain_ild + q * 4 + j, v * w);
+        }
+#pragma unroll
+        for (int off = 4; off < 64; off <<= 1) {  // over the 16 columns of the block
+#pragma unroll
+            for (int j = 0; j < 4; ++j) sq[j] += __shfl_xor(sq[j], off, 64);
+        }
+        if (c16 == 0) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) a.chain_sq_out[(size_t)nb * 16 + q * 4 + j] = sq[j];
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------
 // Small-M kernel for slots of 8 and 16 rows, staged by direct global -> LDS loads.
 // ---------------------------------------------------------------------------
@@ -710,16 +765,8 @@ __global__ __launch_bounds__(NT) void tl_spmm_quad(KernelArgs a)
     float4 row_factors = make_float4(1.f, 1.f, 1.f, 1.f);  // chained product, first wave: the factors of rows 4 * (lane % 4) .. + 3
     if (MT == 16 && a.chain_sq_in && tid < 64) row_factors = chain_row_factors(a, tid);
     // what the chained epilogue of the first wave adds and multiplies, asked for now rather than at the very end
-    float res_early[4] = {0.f, 0.f, 0.f, 0.f}, w_early = 0.f;
-    if (MT == 16 && tid < 64) {
-        const int n = nb * TL_BLOCK_COLUMNS + ((tid / Q) & 15);
-        if (a.chain_res && n < a.N) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                if ((tid % Q) * 4 + j < a.M) res_early[j] = load_scale(a.chain_res, a.y_f16, (long long)((tid % Q) * 4 + j) * a.chain_ldres + n);
-        }
-        if (a.chain_image && n < a.N) w_early = load_scale(a.chain_w, a.y_f16, n);
-    }
+    ChainOperands early = {{0.f, 0.f, 0.f, 0.f}, 0.f};
+    if (MT == 16 && tid < 64) early = chain_operands(a, nb * TL_BLOCK_COLUMNS + ((tid / Q) & 15), tid % Q);
     int which = 0;
     for (int t = 0; t < a.T; t += TG, which ^= 1) {
         const int nt = min(TG, a.T - t);
@@ -772,36 +819,7 @@ __global__ __launch_bounds__(NT) void tl_spmm_quad(KernelArgs a)
         const int n = nb * TL_BLOCK_COLUMNS + c16;
         const float sc = n < a.N ? load_scale(a.w0.scale, a.scale_f16, n) : 0.f;
         float out[4] = {sum.x * sc, sum.y * sc, sum.z * sc, sum.w * sc};
-        if constexpr (MT == 16) {
-            // chained products (one wave here: 16 columns x 4 row quads)
-            if (a.chain_sq_in) {  // q == lane % 4: the lane's own rows
-                out[0] *= row_factors.x; out[1] *= row_factors.y; out[2] *= row_factors.z; out[3] *= row_factors.w;
-            }
-            if (a.chain_res) {
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    if (n < a.N && q * 4 + j < a.M) out[j] = as_output(out[j], a.y_f16) + res_early[j];
-            }
-            if (a.chain_image) {
-                const float w = w_early;
-                float sq[4];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const float v = (n < a.N && q * 4 + j < a.M) ? as_output(out[j], a.y_f16) : 0.f;  // what Y will hold
-                    sq[j] = v * v;
-                    if (n < a.N && q * 4 + j < a.chain_ild) store_out(a.chain_image, a.y_f16, (long long)n * a.chain_ild + q * 4 + j, v * w);
-                }
-#pragma unroll
-                for (int off = 4; off < 64; off <<= 1) {  // over the 16 columns of the block
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) sq[j] += __shfl_xor(sq[j], off, 64);
-                }
-                if (c16 == 0) {
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) a.chain_sq_out[(size_t)nb * 16 + q * 4 + j] = sq[j];
-                }
-            }
-        }
+        if constexpr (MT == 16) chain_epilogue16(a, nb, n, c16, q, out, row_factors, early);  // (one wave here: 16 columns x 4 row quads)
         if (n < a.N) {
 #pragma unroll
             for (int j = 0; j < 4; ++j)
@@ -987,6 +1005,256 @@ __global__ __launch_bounds__(kBlockThreads) void tl_spmm_octet(KernelArgs a)
 #pragma unroll
             for (int j = 0; j < 8; ++j)
                 if (m0 + q * 8 + j < a.M) store_out(a.Y, a.y_f16, (long long)(m0 + q * 8 + j) * a.ldy + n, out[j] * sc);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Up to 16 fp16 rows: the whole activation image resident in LDS, the index stream straight into registers.
+// ---------------------------------------------------------------------------
+// One workgroup of 16 waves per compute unit.  The 16-row image of ALL of K ([tile][256 slots][16 rows], 8 KB a
+// tile) is loaded once per workgroup and stays; from then on only weights move, and they never touch LDS: a lane
+// loads the dwords of its own run from the stream into registers, one (block, tile) unit ahead of their use, its
+// descriptor two units ahead, the chunk offset three.  A workgroup owns a range of whole column blocks; its
+// (block, tile) units, in block-major order (= the order of the stream), are cut into 16 contiguous pieces, one per
+// wave, so that after the barrier behind the image no wave waits for another until the column sums meet at the end.
+// In a unit the 64 lanes are 2 signs x 16 columns x 2 row octets: a lane walks ONE run (the +1 or the -1 rows of
+// its column) from start to end for eight rows -- one 16-byte LDS read and eight accumulates per index, the sign a
+// constant of the lane.  Where a wave's units pass from one block to the next it leaves its sums for the block in
+// an LDS slot; slot (wave + block) is unique because both only grow along the unit order.  After the one barrier
+// at the end the slots of a block are added in wave order (the same order every time) and the sums go out.
+constexpr int kResWaves = 16;
+constexpr int kResSlotFloats = TL_BLOCK_COLUMNS * 16;  // sums of one block: [column][row]
+
+template <int NP>  // 16-byte pieces of a run that a lane holds in registers (longer runs: the rest dword by dword)
+__global__ __launch_bounds__(kResWaves * 64) void tl_spmm_res16(KernelArgs a)
+{
+    extern __shared__ __align__(16) unsigned char lds[];
+    constexpr int NT = kResWaves * 64, W = kResWaves, MT = 16, ES = 2, VPS = MT * ES / 16;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int G = (int)gridDim.x, g = (int)blockIdx.x;
+    const int b0 = (int)((long long)g * a.NB / G), nblk = (int)((long long)(g + 1) * a.NB / G) - b0;
+    const int T = a.T;
+    const int U = nblk * T;                                    // units of this workgroup, unit u = (block u / T, tile u % T)
+    const int u0 = wave * U / W, u1 = (wave + 1) * U / W;      // this wave's
+    unsigned char* image = lds;                                // [T][256 slots][16 rows]
+    float* slots = reinterpret_cast<float*>(lds + a.xs_bytes); // [W + nblk - 1][column][row]
+    using global_ptr = const __attribute__((address_space(1))) void*;
+    using lds_ptr = __attribute__((address_space(3))) void*;
+
+    // chunk offsets of the wave's first units, ahead of everything else (entries past the wave's units are read and
+    // not used; past the table's end lies the stream)
+    const_u32_ptr cs = as_const(a.w0.chunkstart) + (size_t)b0 * T;
+    const int last = max(u1 - 1, u0);  // units past the wave's last stand for it (loaded again, never used)
+    const uint32_t cs_a = cs[u0], cs_b = cs[u0 + 1], cs_c = cs[u0 + 2];
+
+    {   // the image: rows of the K-major activations, zeros behind a tile's rows and behind K
+        const unsigned char* Xb = static_cast<const unsigned char*>(a.X);
+        const size_t row_bytes = (size_t)a.ldx * ES;
+        const int pieces = T * kTileSlots * VPS;  // a multiple of 64: whole waves
+        for (int first = wave * 64; first < pieces; first += NT) {
+            const int p = first + lane, slot = p / VPS, v = p % VPS;
+            const int r = slot & (kTileSlots - 1), k = (slot >> 8) * a.tile_rows + r;
+            if (r < a.tile_rows && k < a.K)
+                __builtin_amdgcn_global_load_lds((global_ptr)(Xb + (size_t)k * row_bytes + v * 16), (lds_ptr)(image + (size_t)first * 16), 16, 0, 0);
+            else
+                *reinterpret_cast<u32x4*>(image + (size_t)p * 16) = u32x4{0u, 0u, 0u, 0u};
+        }
+    }
+
+    // The LDS serves a 16-byte read of a wave in four passes of 16 lanes: lanes 0-3, 12-15, 20-27 / 4-11, 16-19, 28-31 and
+    // the same of lanes 32-63 (measured: two lanes of a pass on one bank cost a cycle more, lanes of different passes
+    // do not).  Lanes are given columns so that a pass holds 8 NEIGHBOURING columns of one sign, two lanes (the row
+    // octets) to a column: the packer orders the rows of such a group so that, position by position, they differ
+    // modulo 8, i.e. fall on different banks.
+    const int sgn = lane >> 5, h = lane & 1;
+    const int c16 = 2 * (int)((0x73261540u >> (4 * ((lane >> 2) & 7))) & 7u) + ((lane >> 1) & 1);
+    const float sign = sgn ? -1.0f : 1.0f;
+    // A lane past the end of its run gathers zeros: from the slot behind the tile's rows that lies in the class of its
+    // column (slots 248 .. 255 are all zero when a tile has 248 rows at most), so that it stays out of the way of the
+    // pass's other columns -- the packer counts on that; taller tiles have the one zero slot.
+    const uint32_t zero_word = (uint32_t)(a.tile_rows <= kMaxTileRows - 7 ? kMaxTileRows - 7 + (c16 & 7) : kSentinel) * 0x01010101u;
+    const uint32_t* stream = a.w0.stream;
+    // where this lane's run of the unit with descriptor d and chunk offset c starts, and its dwords
+    auto run_of = [&](uint32_t d, uint32_t c, uint32_t& start, int& len) {
+        const int pd = run_pos_dwords(d), nd = run_neg_dwords(d);
+        start = c + (d >> 16) + (sgn ? (uint32_t)pd : 0u);
+        len = sgn ? nd : pd;
+    };
+    auto load_pieces = [&](u32x4 (&p)[NP], uint32_t start) {
+#pragma unroll
+        for (int j = 0; j < NP; ++j)  // dword-aligned 16-byte loads; what lies past the run is never used
+            p[j] = *reinterpret_cast<const u32x4_a4*>(stream + start + 4 * j);
+    };
+    uint32_t c_cur = cs_a, c_nxt = u0 + 1 <= last ? cs_b : cs_a, c_nx2 = u0 + 2 <= last ? cs_c : c_nxt, d_cur = 0, d_nxt = 0;
+    uint32_t touched = 0;  // every 64th byte of the first two chunks, so that the runs behind the descriptors come from the cache
+    u32x4 p_cur[NP], p_nxt[NP];
+    if (u0 < u1) {
+        d_cur = stream[c_cur + c16];
+        d_nxt = stream[c_nxt + c16];
+        if ((uint32_t)lane * 16u < cs_b - cs_a) touched = stream[cs_a + lane * 16];
+        if (u0 + 1 <= last && (uint32_t)lane * 16u < cs_c - cs_b) touched ^= stream[cs_b + lane * 16];
+    }
+    // the blocks this wave sends out at the end (b = wave, wave + 16, ...): what their chained epilogue needs, asked for now
+    float4 row_factors = make_float4(1.f, 1.f, 1.f, 1.f);
+    ChainOperands early = {{0.f, 0.f, 0.f, 0.f}, 0.f};
+    if (wave < nblk) {
+        if (a.chain_sq_in) row_factors = chain_row_factors(a, lane);
+        early = chain_operands(a, (b0 + wave) * TL_BLOCK_COLUMNS + (lane >> 2), lane & 3);
+    }
+    if (u0 < u1) {
+        uint32_t start;
+        int len;
+        run_of(d_cur, c_cur, start, len);
+        load_pieces(p_nxt, start);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of the image (and its first loads)
+    __syncthreads();
+
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+    auto issue4 = [](u32x4 (&v)[4], const unsigned char* xq, uint32_t word) {
+        using lds_cptr = const __attribute__((address_space(3))) void*;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const uint32_t r = (word >> (8 * b)) & 0xffu;
+            const uint32_t addr = (uint32_t)reinterpret_cast<uintptr_t>((lds_cptr)(xq + r * (MT * ES)));
+            asm volatile("ds_read_b128 %0, %1" : "=v"(v[b]) : "v"(addr) : "memory");
+        }
+    };
+    auto add4 = [&](const u32x4 (&v)[4]) {
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                acc[2 * e] = fmaf(__half2float(__ushort_as_half((unsigned short)(v[b][e] & 0xffffu))), sign, acc[2 * e]);
+                acc[2 * e + 1] = fmaf(__half2float(__ushort_as_half((unsigned short)(v[b][e] >> 16))), sign, acc[2 * e + 1]);
+            }
+    };
+
+    for (int u = u0; u < u1; ++u) {
+        // the pieces of this unit are here (asked for one unit ago); so is the next unit's descriptor
+        uint32_t start;
+        int len;
+        run_of(d_cur, c_cur, start, len);
+#pragma unroll
+        for (int j = 0; j < NP; ++j) p_cur[j] = p_nxt[j];
+        {
+            uint32_t nstart;
+            int nlen;
+            run_of(d_nxt, c_nxt, nstart, nlen);
+            load_pieces(p_nxt, nstart);
+        }
+        const uint32_t d_nx2 = stream[c_nx2 + c16];
+        const uint32_t c_nx3 = cs[min(u + 3, last)];
+
+        const int b = u / T, tl = u - b * T;
+        const unsigned char* xq = image + (size_t)tl * kTileSlots * MT * ES + h * 16;
+        u32x4 va[4], vb[4];
+#pragma unroll
+        for (int j = 0; j < NP; ++j) {
+            // two dwords at a time, as far as the longest run of the wave goes (the branches are wave-uniform, so the
+            // counted waits see the reads they count)
+            if (__builtin_amdgcn_ballot_w64(len > 4 * j) == 0) break;
+            uint32_t w[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) w[k] = 4 * j + k < len ? p_cur[j][k] : zero_word;  // past the run: four gathers of zero
+            issue4(va, xq, w[0]);
+            issue4(vb, xq, w[1]);
+            quad_wait<4>(va);
+            add4(va);
+            if (__builtin_amdgcn_ballot_w64(len > 4 * j + 2) != 0) {
+                issue4(va, xq, w[2]);
+                quad_wait<4>(vb);
+                add4(vb);
+                issue4(vb, xq, w[3]);
+                quad_wait<4>(va);
+                add4(va);
+            }
+            quad_wait<0>(vb);
+            add4(vb);
+        }
+        for (int i = 4 * NP; __builtin_amdgcn_ballot_w64(i < len) != 0; ++i) {  // runs longer than the registers hold
+            const uint32_t word = i < len ? stream[start + i] : zero_word;
+            issue4(va, xq, word);
+            quad_wait<0>(va);
+            add4(va);
+        }
+
+        if (u + 1 == u1 || (u + 1) / T != b) {
+            // last unit of this wave in block b: fold the two signs of a column, leave the sums in slot (wave + b)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[e] += __shfl_xor(acc[e], 32, 64);
+            if (sgn == 0) {
+                float4* out = reinterpret_cast<float4*>(slots + (size_t)(wave + b) * kResSlotFloats + c16 * 16 + h * 8);
+                out[0] = make_float4(acc[0], acc[1], acc[2], acc[3]);
+                out[1] = make_float4(acc[4], acc[5], acc[6], acc[7]);
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+        }
+        c_cur = c_nxt; c_nxt = c_nx2; c_nx2 = c_nx3;
+        d_cur = d_nxt; d_nxt = d_nx2;
+    }
+    if (touched == 0x5a5aa5a5u && a.M < 0) slots[0] = 0.f;  // (never: keeps the cache-warming loads in the program)
+    __syncthreads();
+    // Block b goes out through wave b % 16: lane = column lane / 4, rows 4 * (lane % 4) .. + 3, the slots of the waves
+    // that had units in the block added in wave order.
+    for (int b = wave; b < nblk; b += W) {
+        const int col = lane >> 2, q = lane & 3;
+        // the waves with units in block b, in order: unit x belongs to wave ((x + 1) * W - 1) / U
+        const int w_first = ((b * T + 1) * W - 1) / U, w_last = ((b + 1) * T * W - 1) / U;
+        float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int w = w_first; w <= w_last; ++w)
+            if (w * U / W < (w + 1) * U / W) {  // (a wave without units left nothing)
+                const float4 o = *reinterpret_cast<const float4*>(slots + (size_t)(w + b) * kResSlotFloats + col * 16 + q * 4);
+                sum.x += o.x; sum.y += o.y; sum.z += o.z; sum.w += o.w;
+            }
+        const int nb = b0 + b, n = nb * TL_BLOCK_COLUMNS + col;
+        const float sc = n < a.N ? load_scale(a.w0.scale, a.scale_f16, n) : 0.f;
+        if (b >= W) {  // (more than 16 blocks per workgroup: asked for late)
+            if (a.chain_sq_in) row_factors = chain_row_factors(a, lane);
+            early = chain_operands(a, n, q);
+        }
+        if (a.gated) {
+            // gate and up column of a pair sit four lanes apart (same rows): the even column's lane writes the four products
+            // (the row factor multiplies the scaled sum, as in the plain product that tl_silu_mul_pairs would follow)
+            const float f[4] = {row_factors.x, row_factors.y, row_factors.z, row_factors.w};
+            const float s4[4] = {sum.x, sum.y, sum.z, sum.w};
+            float hh[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float y = n < a.N ? as_output(a.chain_sq_in ? s4[j] * sc * f[j] : s4[j] * sc, a.y_f16) : 0.f;
+                const float up = __shfl_xor(y, 4, 64);
+                hh[j] = q * 4 + j < a.M ? gate_pair(y, up, a.y_f16) : 0.f;  // zeros in the padding rows of a K-major image
+            }
+            if (!(col & 1) && n + 1 < a.N) {
+                const int m = q * 4;
+                if (a.y_kld && a.y_f16 && a.y_kld % 4 == 0 && m + 4 <= a.y_kld && reinterpret_cast<uintptr_t>(a.Y) % 8 == 0) {
+                    // four neighbouring rows of one column of the image: one 8-byte store
+                    uint2 packed;
+                    __half* ph = reinterpret_cast<__half*>(&packed);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) ph[j] = __float2half(settled(hh[j]));
+                    *reinterpret_cast<uint2*>(static_cast<__half*>(a.Y) + (long long)(n / 2) * a.y_kld + m) = packed;
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        if (m + j < a.M) store_out(a.Y, a.y_f16, a.y_kld ? (long long)(n / 2) * a.y_kld + m + j : (long long)(m + j) * a.ldy + n / 2, hh[j]);
+                        else if (m + j < a.y_kld) store_out(a.Y, a.y_f16, (long long)(n / 2) * a.y_kld + m + j, 0.f);
+                    }
+                }
+            }
+            continue;
+        }
+        float out[4] = {sum.x * sc, sum.y * sc, sum.z * sc, sum.w * sc};
+        chain_epilogue16(a, nb, n, col, q, out, row_factors, early);
+        if (n < a.N) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (q * 4 + j < a.M) store_out(a.Y, a.y_f16, (long long)(q * 4 + j) * a.ldy + n, out[j]);
         }
     }
 }
@@ -2095,9 +2363,9 @@ inline int rows_mtile(int x_dtype) { return x_dtype == TL_F16 ? 256 : 128; }
 // Tuning knobs (environment variables of the same names).  They are read once, at the first launch of the
 // process; tl_reload_options() reads them again.  A knob that is not set leaves the launcher's own choice.
 enum Knob { TL_SMALL_LDS, TL_TILE_GROUP, TL_QUAD_SHARE, TL_LW, TL_SPMV_SHARE, TL_SPMV_WIDE, TL_SMALL_MT, TL_SPMV_DIRECT,
-            TL_BLOCK_SET, TL_ROWS_SPLIT, TL_OCTET, TL_QUAD_WIDE, TL_SPMV_TILES, kKnobCount };
+            TL_BLOCK_SET, TL_ROWS_SPLIT, TL_OCTET, TL_QUAD_WIDE, TL_SPMV_TILES, TL_RES16, kKnobCount };
 const char* const kKnobNames[kKnobCount] = {"TL_SMALL_LDS", "TL_TILE_GROUP", "TL_QUAD_SHARE", "TL_LW", "TL_SPMV_SHARE", "TL_SPMV_WIDE",
-                                            "TL_SMALL_MT", "TL_SPMV_DIRECT", "TL_BLOCK_SET", "TL_ROWS_SPLIT", "TL_OCTET", "TL_QUAD_WIDE", "TL_SPMV_TILES"};
+                                            "TL_SMALL_MT", "TL_SPMV_DIRECT", "TL_BLOCK_SET", "TL_ROWS_SPLIT", "TL_OCTET", "TL_QUAD_WIDE", "TL_SPMV_TILES", "TL_RES16"};
 struct Knobs {
     bool set[kKnobCount];
     int value[kKnobCount];
@@ -2312,6 +2580,36 @@ int launch_octet_kernel(KernelArgs a, const tl_layout_header* h, hipStream_t st)
     return TL_OK;
 }
 
+// tl_spmm_res16: one workgroup per compute unit, each with a range of whole blocks.  It fits when the image of all of
+// K and the slots of the block sums fit the LDS, and the runs are short enough for a lane's registers.
+inline int res16_workgroups(const KernelArgs& a) { return std::min(compute_units(), a.NB); }
+
+inline size_t res16_lds(const KernelArgs& a)
+{
+    const int nblk_max = (int)ceil_div(a.NB, res16_workgroups(a));
+    return (size_t)a.T * kTileSlots * 16 * 2 + (size_t)(kResWaves + nblk_max - 1) * kResSlotFloats * 4;
+}
+
+inline bool res16_fits(const KernelArgs& a, const tl_layout_header* h)
+{
+    // a lane keeps 16 dwords (64 rows) of a run in registers and fetches the rest one by one: for sparse weights only
+    return res16_lds(a) <= 160 * 1024 && h->mean_run_dwords_x16 <= 16 * 26;
+}
+
+int launch_res16_kernel(KernelArgs a, const tl_layout_header* h, hipStream_t st)
+{
+    (void)h;
+    a.xs_bytes = a.T * kTileSlots * 16 * 2;
+    auto kernel = tl_spmm_res16<4>;
+    static bool raised = false;  // a repeated or racing call is harmless
+    if (!raised) {
+        if (int rc = raise_lds_limit(kernel, 160 * 1024)) return rc;
+        raised = true;
+    }
+    hipLaunchKernelGGL(kernel, dim3((unsigned)res16_workgroups(a)), dim3(kResWaves * 64), res16_lds(a), st, a);
+    return TL_OK;
+}
+
 // The direct-load kernel for one activation row.  All of K in one group when `share` workgroups of that
 // size fit a compute unit, else two alternating buffers of TG tiles.
 template <bool XF16, int NT, int PRO = kProNone>
@@ -2424,6 +2722,22 @@ int launch_small(KernelArgs a, const tl_layout_header* h, int x_dtype, void* wor
     a.x_sm = a.x_kmajor ? 1 : a.ldx;
     a.x_sk = a.x_kmajor ? a.ldx : 1;
     bool aligned = (a.ldx * es) % 16 == 0 && reinterpret_cast<uintptr_t>(a.X) % 16 == 0;
+    const bool chain_out = a.chain_res || a.chain_image;
+    // which kernel, and whether it has the epilogue that was asked for: decided before anything is launched
+    bool octet = false, resident = false;
+    if (mt >= 8) {
+        // fp16, 16 rows: eight rows per lane and two blocks per workgroup where the workgroups still fill the chip
+        octet = mt == 16 && a.x_f16 && knob(TL_OCTET, ceil_div(a.NB, 2) * ceil_div(a.M, 16) >= 2 * (int64_t)compute_units() ? 1 : 0) != 0;
+        // ... or, up to 16 rows and where it fits, the whole image resident in LDS and one workgroup per compute unit
+        // (it pays where a compute unit has more than one block to work through; TL_RES16=1 takes it wherever it fits, 0 never)
+        resident = mt == 16 && a.x_f16 && a.M <= 16 && (a.y_f16 || !(a.gated || chain_out || a.chain_sq_in)) && res16_fits(a, h) &&
+                   knob(TL_RES16, a.NB > compute_units() ? 1 : 0) != 0;
+        if ((chain_out || a.chain_sq_in) && (mt != 16 || !a.x_f16 || !a.y_f16 || a.M > 16))
+            return fail(TL_ERR_UNSUPPORTED, "chained products are for 9 to 16 fp16 rows");
+        if (a.gated && !octet && !resident)
+            return fail(TL_ERR_UNSUPPORTED, "no gated epilogue in the kernel for M=%d, N=%d (tl_spmm, then tl_silu_mul_pairs)", a.M, a.N);
+        if (chain_out && octet && !resident) return fail(TL_ERR_UNSUPPORTED, "no residual / image epilogue in the kernel for N=%d", a.N);
+    }
     // Slots of 8 and 16 rows are copied into LDS as 16-byte pieces of an aligned K-major image; activations
     // that are not one already are brought into that form in the workspace first.
     if (mt >= 8 && !(a.x_kmajor && aligned && a.ldx >= round_up(a.M, mt))) {
@@ -2447,24 +2761,18 @@ int launch_small(KernelArgs a, const tl_layout_header* h, int x_dtype, void* wor
         aligned = true;
     }
     if (mt >= 8) {
-        // fp16, 16 rows: eight rows per lane and two blocks per workgroup where the workgroups still fill the chip
-        const bool octet = mt == 16 && a.x_f16 && knob(TL_OCTET, ceil_div(a.NB, 2) * ceil_div(a.M, 16) >= 2 * (int64_t)compute_units() ? 1 : 0) != 0;
-        if (a.gated && !octet) return fail(TL_ERR_UNSUPPORTED, "no gated epilogue in the kernel for M=%d, N=%d (tl_spmm, then tl_silu_mul_pairs)", a.M, a.N);
-        const bool chain_out = a.chain_res || a.chain_image;
-        if ((chain_out || a.chain_sq_in) && (mt != 16 || !a.x_f16 || !a.y_f16 || a.M > 16))
-            return fail(TL_ERR_UNSUPPORTED, "chained products are for 9 to 16 fp16 rows");
-        if (chain_out && octet) return fail(TL_ERR_UNSUPPORTED, "no residual / image epilogue in the kernel for N=%d", a.N);
         if (mt == 8) return a.x_f16 ? launch_quad_kernel<8, true>(a, h, st) : launch_quad_kernel<8, false>(a, h, st);
+        if (resident) return launch_res16_kernel(a, h, st);
         if (octet) return launch_octet_kernel(a, h, st);
         if (wide) return a.x_f16 ? launch_quad_kernel<16, true, 1024>(a, h, st) : launch_quad_kernel<16, false, 1024>(a, h, st);
         return a.x_f16 ? launch_quad_kernel<16, true>(a, h, st) : launch_quad_kernel<16, false>(a, h, st);
     }
+    if (chain_out || a.chain_sq_in) return fail(TL_ERR_UNSUPPORTED, "chained products are for 9 to 16 fp16 rows");
     // one contiguous aligned row whose tiles are whole 16-byte pieces: straight copies into LDS
     if (mt == 1 && a.x_sk == 1 && reinterpret_cast<uintptr_t>(a.X) % 16 == 0 && h->tile_rows % (16 / es) == 0 && a.K % (16 / es) == 0 &&
         knob(TL_SPMV_DIRECT, 1))
         return a.x_f16 ? launch_spmv_direct<true>(a, h, st) : launch_spmv_direct<false>(a, h, st);
     if (a.gated) return fail(TL_ERR_UNSUPPORTED, "no gated epilogue in the kernel for M=%d and this activation layout (tl_spmm, then tl_silu_mul_pairs)", a.M);
-    if (a.chain_res || a.chain_image || a.chain_sq_in) return fail(TL_ERR_UNSUPPORTED, "chained products are for 9 to 16 fp16 rows");
     // Column blocks per workgroup.  A compute unit works through ceil(workgroups / 256) workgroups of
     // `set` blocks each: the narrowest set that keeps that product smallest.
     int set = 1;
@@ -2699,7 +3007,7 @@ int spmm_call(const tl_layout_header* header, const void* blob_dev, const void* 
         if (out && !(chain->next_norm_weight && chain->image_out && chain->squares_out))
             return fail(TL_ERR_ARG, "next_norm_weight, image_out and squares_out come together");
         if ((out || chain->residual) && gated) return fail(TL_ERR_ARG, "a gated product has no residual or image epilogue");
-        if (M > 16) return fail(TL_ERR_UNSUPPORTED, "chained products are for 9 to 16 fp16 rows");
+        if (M < 9 || M > 16) return fail(TL_ERR_UNSUPPORTED, "chained products are for 9 to 16 fp16 rows");
         if (chain->residual && chain->residual_ld < (int64_t)header->columns) return fail(TL_ERR_SHAPE, "residual_ld=%lld smaller than N", (long long)chain->residual_ld);
         if (out && (chain->image_ld < M || chain->image_ld > 16))  // the epilogue writes (and zeroes) 16 rows of the image at most
             return fail(TL_ERR_SHAPE, "image_ld=%lld outside M=%lld .. 16", (long long)chain->image_ld, (long long)M);

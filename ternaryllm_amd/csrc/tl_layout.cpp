@@ -114,13 +114,14 @@ struct RunRef {
 };
 
 constexpr int kLanesPerRun = 4;
+constexpr int kWeight16 = 4;  // a shared class of the 16-row kernel against a shared bank of the single-row kernel, in the deal
 constexpr int kSpreadSweeps = 2;
 
 // LDS bank of a row's activation in the single-row kernel: fp16 values, two to a bank word; the image of
 // tile t starts kSpmvImageSkew bytes further round the banks than that of tile t - 1 (tl_common.h).
 inline int bank_of(uint8_t row, int tile) { return ((row >> 1) + tile * (kSpmvImageSkew / 4)) & 31; }
 
-void spread_over_banks(const RunRef* runs, int n_runs, int sweeps)
+void spread_over_banks(const RunRef* runs, int n_runs, int sweeps, int tile_rows)
 {
     // read q = pass * 4 + byte; run r, lane l holds dword pass * 4 + l of the combined run
     int longest = 0;
@@ -128,7 +129,25 @@ void spread_over_banks(const RunRef* runs, int n_runs, int sweeps)
     if (longest == 0) return;
     const int passes = (longest + kLanesPerRun - 1) / kLanesPerRun, reads = passes * 4;
     std::vector<int> load((size_t)reads * 32, 0);
+    // 16-row kernel: at position e of the runs of one sign, the rows of the group's columns should differ modulo 8
+    std::vector<uint8_t> load16((size_t)2 * 256 * 8, 0);
     std::vector<uint8_t> pool[2];
+    {
+        // Behind the end of its run a lane of the 16-row kernel gathers from a zero slot: slot 248 + (column % 8) when
+        // the tile leaves all of 248 .. 255 free, else slot 255; the other columns' rows at those positions keep
+        // out of that class.
+        int longest16[2] = {0, 0};
+        for (int r = 0; r < n_runs; ++r) {
+            longest16[0] = std::max(longest16[0], (runs[r].n_pos + 3) / 4 * 4);
+            longest16[1] = std::max(longest16[1], (runs[r].n_neg + 3) / 4 * 4);
+        }
+        for (int r = 0; r < n_runs; ++r)
+            for (int sign = 0; sign < 2; ++sign) {
+                const int n = sign ? runs[r].n_neg : runs[r].n_pos;
+                const int zero_class = tile_rows <= kMaxTileRows - 7 ? (r & 7) : (kSentinel & 7);
+                for (int e = (n + 3) / 4 * 4; e < longest16[sign]; ++e) ++load16[((size_t)sign * 256 + e) * 8 + zero_class];
+            }
+    }
     auto position = [&](const RunRef& run, int q, int l, bool* neg, int* e) {
         const int pd = (run.n_pos + 3) / 4;
         const int i = (q >> 2) * kLanesPerRun + l;
@@ -144,8 +163,10 @@ void spread_over_banks(const RunRef* runs, int n_runs, int sweeps)
         // the padding bytes of the two last dwords read the tile's zero slot: loads that are there whatever the order
         for (int sign = 0; sign < 2; ++sign) {
             const int n = sign ? run.n_neg : run.n_pos;
-            for (int e = n; e < (n + 3) / 4 * 4; ++e)
+            for (int e = n; e < (n + 3) / 4 * 4; ++e) {
                 ++load[(size_t)((((sign ? pd : 0) + e / 4) / kLanesPerRun) * 4 + (e & 3)) * 32 + bank_of(kSentinel, run.tile)];
+                ++load16[((size_t)sign * 256 + e) * 8 + (kSentinel & 7)];
+            }
         }
         for (int q = 0; q < reads; ++q)
             for (int l = 0; l < kLanesPerRun; ++l) {
@@ -154,15 +175,19 @@ void spread_over_banks(const RunRef* runs, int n_runs, int sweeps)
                 if (!position(run, q, l, &neg, &e)) continue;
                 std::vector<uint8_t>& left = pool[neg ? 1 : 0];
                 const int* ld = &load[(size_t)q * 32];
+                uint8_t* l16 = &load16[((size_t)(neg ? 1 : 0) * 256 + e) * 8];
+                auto key = [&](uint8_t row) { return (kWeight16 * l16[row & 7] + ld[bank_of(row, run.tile)]) * 256 + row; };
                 size_t best = 0;
+                int best_key = key(left[0]);
                 for (size_t c = 1; c < left.size(); ++c) {
-                    const int lb = ld[bank_of(left[best], run.tile)], lc = ld[bank_of(left[c], run.tile)];
-                    if (lc < lb || (lc == lb && left[c] < left[best])) best = c;
+                    const int k = key(left[c]);
+                    if (k < best_key) { best = c; best_key = k; }
                 }
                 const uint8_t row = left[best];
                 left[best] = left.back();
                 left.pop_back();
                 ++load[(size_t)q * 32 + bank_of(row, run.tile)];
+                ++l16[row & 7];
                 run.bytes[(neg ? 4 * pd : 0) + e] = row;
             }
     }
@@ -202,6 +227,27 @@ void spread_over_banks(const RunRef* runs, int n_runs, int sweeps)
         const int pd = (run.n_pos + 3) / 4, nd = (run.n_neg + 3) / 4;
         for (int e = 0; e < 4 * (pd + nd); ++e) add(((e / 4) / kLanesPerRun) * 4 + (e & 3), run.bytes[e] >> 1, run.tile);
     }
+    // The 16-row kernel's side of a swap: what the positions e1 and e2 of one sign cost it before and after their rows
+    // (classes c1, c2) change places.  A position costs the largest number of the group's rows in one class (its LDS
+    // cycles), plus a little for every row beyond the first in a class.
+    auto cost16 = [&](const uint8_t* cnt) {
+        int most = 0, extra = 0;
+        for (int c = 0; c < 8; ++c) {
+            most = std::max(most, (int)cnt[c]);
+            extra += cnt[c] > 1 ? cnt[c] - 1 : 0;
+        }
+        return (float)most + 0.25f * (float)extra;
+    };
+    auto swap16 = [&](int sign, int e1, int e2, int c1, int c2, bool apply) {
+        if (c1 == c2) return 0.0f;
+        uint8_t* a = &load16[((size_t)sign * 256 + e1) * 8];
+        uint8_t* b = &load16[((size_t)sign * 256 + e2) * 8];
+        const float before = cost16(a) + cost16(b);
+        --a[c1]; ++a[c2]; --b[c2]; ++b[c1];
+        const float after = cost16(a) + cost16(b);
+        if (!apply) { ++a[c1]; --a[c2]; ++b[c2]; --b[c1]; }
+        return before - after;  // what the swap gains
+    };
     for (int sweep = 0; sweep < sweeps; ++sweep) {
         bool any = false;
         for (int r = 0; r < n_runs; ++r) {
@@ -213,26 +259,31 @@ void spread_over_banks(const RunRef* runs, int n_runs, int sweeps)
                 const int first_dword = sign ? pd : 0;
                 auto read_of = [&](int e) { return ((first_dword + e / 4) / kLanesPerRun) * 4 + (e & 3); };
                 for (int e1 = 0; e1 < n; ++e1) {
-                    const int q1 = read_of(e1), w1 = rows[e1] >> 1, b1 = bank_of(rows[e1], tile);
-                    // only a row that is alone on its word, on a bank that delivers another word too, is worth moving
-                    if (state[(size_t)q1].words[w1] != 1 || state[(size_t)q1].per_bank[b1] < 2) continue;
+                    const int q1 = read_of(e1), w1 = rows[e1] >> 1, b1 = bank_of(rows[e1], tile), c1 = rows[e1] & 7;
+                    // a row is worth moving when it is alone on its word, on a bank that delivers another word too
+                    // (single-row kernel), or shares its class with a row of another column (16-row kernel)
+                    const bool shared1 = state[(size_t)q1].words[w1] == 1 && state[(size_t)q1].per_bank[b1] >= 2;
+                    const bool shared16 = load16[((size_t)sign * 256 + e1) * 8 + c1] >= 2;
+                    if (!shared1 && !shared16) continue;
                     int best = -1;
                     float best_gain = 1e-6f;
                     for (int e2 = 0; e2 < n; ++e2) {
-                        const int q2 = read_of(e2);
-                        if (q2 == q1) continue;
-                        const int w2 = rows[e2] >> 1, b2 = bank_of(rows[e2], tile);
-                        // the row that comes must not bring a shared bank of its own
-                        if (b2 == b1 || (state[(size_t)q1].words[w2] == 0 && state[(size_t)q1].per_bank[b2] != 0)) continue;
-                        const float before = potential(q1) + potential(q2);
-                        drop(q1, w1, tile); add(q1, w2, tile); drop(q2, w2, tile); add(q2, w1, tile);
-                        const float gain = before - potential(q1) - potential(q2);
-                        drop(q2, w1, tile); add(q2, w2, tile); drop(q1, w2, tile); add(q1, w1, tile);
+                        if (e2 == e1) continue;
+                        const int q2 = read_of(e2), w2 = rows[e2] >> 1, c2 = rows[e2] & 7;
+                        float gain = (float)kWeight16 * swap16(sign, e1, e2, c1, c2, false);
+                        if (q2 != q1) {  // (inside one read of the single-row kernel nothing changes for it)
+                            if (!shared1 && gain <= 0.f) continue;
+                            const float before = potential(q1) + potential(q2);
+                            drop(q1, w1, tile); add(q1, w2, tile); drop(q2, w2, tile); add(q2, w1, tile);
+                            gain += before - potential(q1) - potential(q2);
+                            drop(q2, w1, tile); add(q2, w2, tile); drop(q1, w2, tile); add(q1, w1, tile);
+                        }
                         if (gain > best_gain) { best_gain = gain; best = e2; }
                     }
                     if (best >= 0) {
                         const int q2 = read_of(best), w2 = rows[best] >> 1;
-                        drop(q1, w1, tile); add(q1, w2, tile); drop(q2, w2, tile); add(q2, w1, tile);
+                        if (q2 != q1) { drop(q1, w1, tile); add(q1, w2, tile); drop(q2, w2, tile); add(q2, w1, tile); }
+                        swap16(sign, e1, best, c1, rows[best] & 7, true);
                         std::swap(rows[e1], rows[best]);
                         any = true;
                     }
@@ -375,7 +426,7 @@ extern "C" int tl_layout_build(const int32_t* neg_row, const int32_t* neg_off_ti
                         const uint32_t d = stream[c0 + j0 + i];
                         runs[i] = RunRef{bytes + (c0 + (d >> 16)) * 4, (int)(d & 0xff), (int)((d >> 8) & 0xff), t};
                     }
-                    spread_over_banks(runs.data(), gsz, kSpreadSweeps);
+                    spread_over_banks(runs.data(), gsz, kSpreadSweeps, g.tile_rows);
                 }
             }
     }

@@ -247,9 +247,62 @@ def test_small_m_kernels_in_every_mode(cuda, oracle, dtype):
                  {"TL_SPMV_TILES": "1"}, {"TL_SPMV_TILES": "1", "TL_SPMV_WIDE": "0"}, {"TL_SPMV_TILES": "0"}] if M == 1 else [{"TL_SMALL_MT": "8"}, {"TL_SMALL_MT": "16"}, {"TL_SMALL_MT": "16", "TL_TILE_GROUP": "2"},
                                    {"TL_SMALL_MT": "16", "TL_OCTET": "1"}, {"TL_SMALL_MT": "16", "TL_OCTET": "1", "TL_TILE_GROUP": "1"},
                                    {"TL_SMALL_MT": "16", "TL_OCTET": "1", "TL_LW": "1", "TL_TILE_GROUP": "8"},
-                                   {"TL_QUAD_WIDE": "0"}, {"TL_QUAD_WIDE": "1", "TL_LW": "2"}, {"TL_QUAD_WIDE": "1", "TL_TILE_GROUP": "1"}]
+                                   {"TL_QUAD_WIDE": "0"}, {"TL_QUAD_WIDE": "1", "TL_LW": "2"}, {"TL_QUAD_WIDE": "1", "TL_TILE_GROUP": "1"},
+                                   {"TL_RES16": "1"}, {"TL_RES16": "0"}]
         for env in settings + extra:
             print(f"case M={M} dtype={dtype} env={env}", flush=True)
             with knobs(**env):
                 y = ops.spmm(dw, x.to(cuda), out_dtype=torch.float32).cpu().numpy()
             assert np.array_equal(y.astype(np.float64), ref), (M, env)
+
+
+def test_resident_16_row_kernel_and_its_epilogues(cuda, oracle):
+    """9 to 16 fp16 rows with the activation image resident in LDS (tl_spmm_res16, TL_RES16=1): exact on integer
+    activations against the oracle -- one and several blocks per workgroup, ragged K and N, dense and sparse
+    weights (runs longer than a lane's registers hold), a tile height with a single zero slot -- and every epilogue
+    (scale, fp32 output, SiLU gate row-major and K-major, residual, next-norm image and squares, row factors)
+    bit for bit against the kernels it stands in for (TL_RES16=0)."""
+    from ternaryllm_amd import ops, _lib
+    from ternaryllm_amd.packing import PackedWeight
+    for K, N, M, s, tile_rows in ((2100, 200, 16, 0.7, 0), (4096, 4720, 13, 0.66, 0), (1000, 40, 9, 0.2, 0), (4000, 4400, 16, 0.9, 0),
+                                  (1530, 336, 16, 0.62, 255), (300, 16, 11, 0.05, 0)):
+        w = ternary_weight(K, N, s, 90 + M)
+        dw = ops.DeviceWeight(PackedWeight.from_dense(w, tile_rows), cuda)
+        x = activations(M, K, 91 + M, torch.float16, integer=True)
+        ref = oracle.fast_product(x.double().numpy(), w)
+        g = torch.Generator().manual_seed(92 + M)
+        scale = (0.5 + torch.rand(N, generator=g)).half().to(cuda) / 32
+        res = torch.randn((M, N), generator=g).half().to(cuda)
+        nw = (0.5 + torch.rand(N, generator=g)).half().to(cuda)
+        xd = x.to(cuda)
+        ximg, _ = ops._kmajor_image(M, K, xd)
+        ximg[:, :M] = xd.t()
+        xk = ximg[:, :M]
+        sq = torch.rand(((K + 15) // 16, 16), generator=g).to(cuda) * 50
+        outs = {}
+        for tag, env in (("old", {"TL_RES16": "0"}), ("new", {"TL_RES16": "1"})):
+            print(f"case K={K} N={N} M={M} s={s} tile_rows={tile_rows} {tag}", flush=True)
+            with knobs(**env):
+                o = {"plain32": ops.spmm(dw, xd, out_dtype=torch.float32), "plain": ops.spmm(dw, xd, scale),
+                     "kmajor": ops.spmm(dw, xk, scale, x_layout=_lib.TL_X_K_MAJOR),
+                     "res": ops.spmm_chain(dw, xk, scale, x_layout=_lib.TL_X_K_MAJOR, residual=res),
+                     "factors": ops.spmm_chain(dw, xk, scale, x_layout=_lib.TL_X_K_MAJOR, squares_in=sq, eps=1e-5)}
+                if tag == "new" or N < 16384:  # (the kernel for wide outputs has no image epilogue)
+                    o["image"] = ops.spmm_chain(dw, xk, scale, x_layout=_lib.TL_X_K_MAJOR, residual=res, next_norm_weight=nw, squares_in=sq, eps=1e-5)
+                if N % 2 == 0:
+                    o["gated"] = ops.spmm_gated(dw, xd, scale)
+                    o["gated_k"] = ops.spmm_gated(dw, xk, scale, x_layout=_lib.TL_X_K_MAJOR, kmajor=True)
+                    o["gated_factors"] = ops.spmm_chain(dw, xk, scale, x_layout=_lib.TL_X_K_MAJOR, squares_in=sq, eps=1e-5, gated=True, kmajor=True)
+            torch.cuda.synchronize()
+            outs[tag] = o
+        assert np.array_equal(outs["new"]["plain32"].cpu().numpy().astype(np.float64), ref), (K, N, M)
+        for name, got in outs["new"].items():
+            want = outs["old"].get(name)
+            if want is None:
+                continue
+            pairs = zip(got, want) if isinstance(got, tuple) else ((got, want),)
+            for a, b in pairs:
+                assert torch.equal(a, b), (K, N, M, name)
+        if "gated_k" in outs["new"]:  # the padding rows of a K-major image are zeros
+            img = outs["new"]["gated_k"]
+            assert not img.as_strided((N // 2, 16), (16, 1))[:, M:].any()

@@ -276,6 +276,12 @@ def test_compute_entry_points_reject_bad_arguments_before_any_launch():
     assert L.tl_spmm(hdr, fake, fake, 0, 0, 64, 1, fake, 0, 8, None, 0, None, 0, None) < 0             # ldy < N
     assert L.tl_spmm(hdr, fake, fake, 0, 2, 64, 1, fake, 0, 32, None, 0, None, 0, None) < 0            # unknown layout
     assert L.tl_spmm(hdr, ctypes.c_void_p(257), fake, 0, 0, 64, 1, fake, 0, 32, None, 0, None, 0, None) < 0  # unaligned blob
+    # a chained product outside 9 .. 16 rows is refused, one row or eight included (no launch, nothing ignored)
+    chain = _lib.Chain()
+    chain.residual, chain.residual_ld = fake.value, 32
+    for rows in (1, 8, 17):
+        assert L.tl_spmm_chain(hdr, fake, fake, _lib.TL_F16, 0, 64, rows, fake, _lib.TL_F16, 32, -1, None, 0, ctypes.byref(chain), fake, 1 << 20, None) \
+            == _lib.TL_ERR_UNSUPPORTED, rows
     pos = ctypes.c_void_p(4096)
     assert L.tl_rope_cache_update(fake, 5, 1, 2, 64, fake, fake, pos, fake, fake, fake, 16, None) < 0  # dtype
     assert L.tl_rope_cache_update(fake, 1, 1, 2, 63, fake, fake, pos, fake, fake, fake, 16, None) < 0  # odd head_dim
