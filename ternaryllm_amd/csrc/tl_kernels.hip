@@ -1010,27 +1010,35 @@ __global__ __launch_bounds__(kBlockThreads) void tl_spmm_octet(KernelArgs a)
 }
 
 // ---------------------------------------------------------------------------
-// Up to 16 fp16 rows: the whole activation image resident in LDS, the index stream straight into registers.
+// 16 fp16 rows or 8 fp32 rows: the whole activation image resident in LDS, the index stream straight into registers.
 // ---------------------------------------------------------------------------
-// One workgroup of 16 waves per compute unit.  The 16-row image of ALL of K ([tile][256 slots][16 rows], 8 KB a
-// tile) is loaded once per workgroup and stays; from then on only weights move, and they never touch LDS: a lane
+// One workgroup of 16 waves per compute unit.  The image of ALL of K ([tile][256 slots][32 bytes]: 16 fp16 or 8 fp32
+// rows, 8 KB a tile) is loaded once per workgroup and stays; from then on only weights move, and they never touch LDS: a lane
 // loads the dwords of its own run from the stream into registers, one (block, tile) unit ahead of their use, its
 // descriptor two units ahead, the chunk offset three.  A workgroup owns a range of whole column blocks; its
 // (block, tile) units, in block-major order (= the order of the stream), are cut into 16 contiguous pieces, one per
 // wave, so that after the barrier behind the image no wave waits for another until the column sums meet at the end.
-// In a unit the 64 lanes are 2 signs x 16 columns x 2 row octets: a lane walks ONE run (the +1 or the -1 rows of
-// its column) from start to end for eight rows -- one 16-byte LDS read and eight accumulates per index, the sign a
-// constant of the lane.  Where a wave's units pass from one block to the next it leaves its sums for the block in
+// In a unit the 64 lanes are 2 signs x 16 columns x 2 halves of a slot: a lane walks ONE run (the +1 or the -1 rows
+// of its column) from start to end for eight fp16 or four fp32 rows -- one 16-byte LDS read and eight (four)
+// accumulates per index, the sign a constant of the lane.  More rows than a slot holds are further workgroups
+// (blockIdx.y) with an image of their own.  Where a wave's units pass from one block to the next it leaves its sums for the block in
 // an LDS slot; slot (wave + block) is unique because both only grow along the unit order.  After the one barrier
 // at the end the slots of a block are added in wave order (the same order every time) and the sums go out.
 constexpr int kResWaves = 16;
-constexpr int kResSlotFloats = TL_BLOCK_COLUMNS * 16;  // sums of one block: [column][row]
 
-template <int NP>  // 16-byte pieces of a run that a lane holds in registers (longer runs: the rest dword by dword)
-__global__ __launch_bounds__(kResWaves * 64) void tl_spmm_res16(KernelArgs a)
+// ROWS_IN: the activations come as row-major rows of whole, aligned 16-byte pieces (else: an aligned K-major image, whose
+// slots are copied straight into LDS) and the workgroup turns them into its image itself: a thread takes the same
+// 16-byte piece of four rows, transposes the 4 x 4 (fp32) or 4 x 8 (fp16) values in registers and writes one slot
+// quarter per value of k.  Threads of a wave would all write slots that are equal modulo 8 -- the same banks -- so
+// each rotates its values by its piece number first and writes them in the rotated order.
+template <bool XF16, int NP, bool ROWS_IN>  // NP: 16-byte pieces of a run that a lane holds in registers (longer runs: the rest dword by dword)
+__global__ __launch_bounds__(kResWaves * 64) void tl_spmm_res(KernelArgs a)
 {
     extern __shared__ __align__(16) unsigned char lds[];
-    constexpr int NT = kResWaves * 64, W = kResWaves, MT = 16, ES = 2, VPS = MT * ES / 16;
+    constexpr int NT = kResWaves * 64, W = kResWaves, MT = XF16 ? 16 : 8, ES = XF16 ? 2 : 4, VPS = MT * ES / 16;
+    constexpr int NA = MT / 2;                              // rows (accumulators) of a lane
+    constexpr int kResSlotFloats = TL_BLOCK_COLUMNS * MT;   // sums of one block: [column][row]
+    static_assert(MT * ES == 32 && VPS == 2, "a slot is two 16-byte pieces");
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int G = (int)gridDim.x, g = (int)blockIdx.x;
@@ -1038,7 +1046,8 @@ __global__ __launch_bounds__(kResWaves * 64) void tl_spmm_res16(KernelArgs a)
     const int T = a.T;
     const int U = nblk * T;                                    // units of this workgroup, unit u = (block u / T, tile u % T)
     const int u0 = wave * U / W, u1 = (wave + 1) * U / W;      // this wave's
-    unsigned char* image = lds;                                // [T][256 slots][16 rows]
+    const int m0 = (int)blockIdx.y * MT;                       // first row of this workgroup's slot
+    unsigned char* image = lds;                                // [T][256 slots][MT rows]
     float* slots = reinterpret_cast<float*>(lds + a.xs_bytes); // [W + nblk - 1][column][row]
     using global_ptr = const __attribute__((address_space(1))) void*;
     using lds_ptr = __attribute__((address_space(3))) void*;
@@ -1048,20 +1057,6 @@ __global__ __launch_bounds__(kResWaves * 64) void tl_spmm_res16(KernelArgs a)
     const_u32_ptr cs = as_const(a.w0.chunkstart) + (size_t)b0 * T;
     const int last = max(u1 - 1, u0);  // units past the wave's last stand for it (loaded again, never used)
     const uint32_t cs_a = cs[u0], cs_b = cs[u0 + 1], cs_c = cs[u0 + 2];
-
-    {   // the image: rows of the K-major activations, zeros behind a tile's rows and behind K
-        const unsigned char* Xb = static_cast<const unsigned char*>(a.X);
-        const size_t row_bytes = (size_t)a.ldx * ES;
-        const int pieces = T * kTileSlots * VPS;  // a multiple of 64: whole waves
-        for (int first = wave * 64; first < pieces; first += NT) {
-            const int p = first + lane, slot = p / VPS, v = p % VPS;
-            const int r = slot & (kTileSlots - 1), k = (slot >> 8) * a.tile_rows + r;
-            if (r < a.tile_rows && k < a.K)
-                __builtin_amdgcn_global_load_lds((global_ptr)(Xb + (size_t)k * row_bytes + v * 16), (lds_ptr)(image + (size_t)first * 16), 16, 0, 0);
-            else
-                *reinterpret_cast<u32x4*>(image + (size_t)p * 16) = u32x4{0u, 0u, 0u, 0u};
-        }
-    }
 
     // The LDS serves a 16-byte read of a wave in four passes of 16 lanes: lanes 0-3, 12-15, 20-27 / 4-11, 16-19, 28-31 and
     // the same of lanes 32-63 (measured: two lanes of a pass on one bank cost a cycle more, lanes of different passes
@@ -1087,34 +1082,148 @@ __global__ __launch_bounds__(kResWaves * 64) void tl_spmm_res16(KernelArgs a)
         for (int j = 0; j < NP; ++j)  // dword-aligned 16-byte loads; what lies past the run is never used
             p[j] = *reinterpret_cast<const u32x4_a4*>(stream + start + 4 * j);
     };
-    uint32_t c_cur = cs_a, c_nxt = u0 + 1 <= last ? cs_b : cs_a, c_nx2 = u0 + 2 <= last ? cs_c : c_nxt, d_cur = 0, d_nxt = 0;
-    uint32_t touched = 0;  // every 64th byte of the first two chunks, so that the runs behind the descriptors come from the cache
+    uint32_t c_cur = cs_a, c_nxt = u0 + 1 <= last ? cs_b : cs_a, c_nx2 = u0 + 2 <= last ? cs_c : c_nxt, d_cur, d_nxt;
     u32x4 p_cur[NP], p_nxt[NP];
-    if (u0 < u1) {
-        d_cur = stream[c_cur + c16];
-        d_nxt = stream[c_nxt + c16];
-        if ((uint32_t)lane * 16u < cs_b - cs_a) touched = stream[cs_a + lane * 16];
-        if (u0 + 1 <= last && (uint32_t)lane * 16u < cs_c - cs_b) touched ^= stream[cs_b + lane * 16];
-    }
-    // the blocks this wave sends out at the end (b = wave, wave + 16, ...): what their chained epilogue needs, asked for now
-    float4 row_factors = make_float4(1.f, 1.f, 1.f, 1.f);
-    ChainOperands early = {{0.f, 0.f, 0.f, 0.f}, 0.f};
-    if (wave < nblk) {
-        if (a.chain_sq_in) row_factors = chain_row_factors(a, lane);
-        early = chain_operands(a, (b0 + wave) * TL_BLOCK_COLUMNS + (lane >> 2), lane & 3);
-    }
-    if (u0 < u1) {
+    // (straight-line code, every load unconditional: a wave without units reads what a neighbour reads; the waits are
+    // then counted exactly, and nothing below waits for more than it needs)
+    d_cur = stream[c_cur + c16];
+    d_nxt = stream[c_nxt + c16];
+    // every 64th byte of the first two chunks, so that the runs behind their descriptors come from the cache (a chunk
+    // that is not this wave's has length 0 here: cs_b and cs_c are table entries only as far as the wave's units go)
+    const uint32_t len_a = u0 < u1 ? cs_b - cs_a : 0u, len_b = u0 + 1 <= last ? cs_c - cs_b : 0u;
+    const uint32_t touched = stream[c_cur + min((uint32_t)lane * 16u, max(len_a, 1u) - 1u)];
+    const uint32_t touched2 = stream[c_nxt + min((uint32_t)lane * 16u, max(len_b, 1u) - 1u)];
+    // the first unit's runs: asked for behind the image's loads, as soon as its descriptor is here
+    auto first_pieces = [&]() {
         uint32_t start;
         int len;
         run_of(d_cur, c_cur, start, len);
         load_pieces(p_nxt, start);
+    };
+    if constexpr (!ROWS_IN) {   // the image: rows of the K-major activations, zeros behind a tile's rows and behind K
+        // (the workgroup's 1024 pieces a turn are two whole tiles: a thread's slot and piece of the slot never change,
+        // a turn moves its address two tiles on)
+        static_assert(NT == 2 * kTileSlots * VPS, "a turn of the image loop covers two tiles");
+        const size_t row_bytes = (size_t)a.ldx * ES;
+        const int r = (tid >> 1) & (kTileSlots - 1), v = tid & 1, tsub = wave >> 3;
+        const unsigned char* src = static_cast<const unsigned char*>(a.X) + (size_t)m0 * ES + ((size_t)tsub * a.tile_rows + r) * row_bytes + v * 16;
+        const size_t step = (size_t)2 * a.tile_rows * row_bytes;
+        for (int tile = tsub; tile < T; tile += 2, src += step) {
+            if (r < a.tile_rows && tile * a.tile_rows + r < a.K)
+                __builtin_amdgcn_global_load_lds((global_ptr)src, (lds_ptr)(image + ((size_t)tile * kTileSlots * VPS + (wave & 7) * 64) * 16), 16, 0, 0);
+            else
+                *reinterpret_cast<u32x4*>(image + ((size_t)tile * kTileSlots * VPS + (tid & (kTileSlots * VPS - 1))) * 16) = u32x4{0u, 0u, 0u, 0u};
+        }
+        first_pieces();
+    } else {
+        constexpr int KV = 16 / ES;  // values of k in a 16-byte piece of a row
+        constexpr int RQ = MT / 4;   // row quads of the slot
+        constexpr int QB = 32 / RQ;  // bytes of a row quad in a slot
+        constexpr int KSTEP = NT / RQ;  // pieces along k from one task of a thread to its next
+        static_assert(NT % RQ == 0, "a thread keeps its row quad from task to task");
+        // task t: row quad t % RQ, piece t / RQ of the rows; a thread's tasks are t = tid, tid + NT, ...: same four rows, KSTEP pieces on
+        const int tasks = (a.K / KV) * RQ, rq = tid % RQ;
+        const int row0 = m0 + 4 * rq;
+        const bool whole = m0 + MT <= a.M;  // (wave-uniform: the slot has all its rows)
+        const size_t row_bytes = (size_t)a.ldx * ES;
+        const unsigned char* rp[4];  // the thread's piece of its four rows (rows that do not exist: the last one, zeroed below)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)  // (a thread without a task reads the last piece: dropped below)
+            rp[i] = static_cast<const unsigned char*>(a.X) + (size_t)min(row0 + i, a.M - 1) * row_bytes + (size_t)min(tid / RQ, a.K / KV - 1) * 16;
+        u32x4 in[2][4];  // two tasks of a thread in flight
+        auto load_task = [&](u32x4 (&v)[4], int turn) {  // (a task past the last reads the thread's first again: dropped below)
+            const size_t off = (size_t)(tid + turn * NT < tasks ? turn : 0) * KSTEP * 16;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) v[i] = *reinterpret_cast<const u32x4*>(rp[i] + off);
+        };
+        auto store_task = [&](u32x4 (&v)[4], int turn) {
+            if (tid + turn * NT >= tasks) return;
+            const int kp = tid / RQ + turn * KSTEP, k = kp * KV;
+            const int tile = (int)(((unsigned long long)(unsigned)k * a.tile_magic) >> 32);  // k / tile_rows; a piece never straddles tiles
+            unsigned char* base = image + (size_t)tile * kTileSlots * 32 + (size_t)(k - tile * a.tile_rows) * 32 + rq * QB;
+            if (!whole) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (row0 + i >= a.M) v[i] = u32x4{0u, 0u, 0u, 0u};
+            }
+            // Written in k order every thread of a wave would hit the same banks (slots equal modulo 8), 16 to a bank: each
+            // thread rotates its values by its piece number first and writes them in the rotated order.
+            const int rot = kp & (KV - 1);
+            if constexpr (XF16) {
+                uint2 out[8];  // out[j]: the four rows' values of k + j
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const uint32_t a0 = v[0][j / 2], a1 = v[1][j / 2], a2 = v[2][j / 2], a3 = v[3][j / 2];
+                    // (low halves / high halves of two dwords side by side: one byte permute each)
+                    out[j] = (j & 1) ? make_uint2(__builtin_amdgcn_perm(a1, a0, 0x07060302u), __builtin_amdgcn_perm(a3, a2, 0x07060302u))
+                                     : make_uint2(__builtin_amdgcn_perm(a1, a0, 0x05040100u), __builtin_amdgcn_perm(a3, a2, 0x05040100u));
+                }
+#pragma unroll
+                for (int sh = 1; sh < 8; sh <<= 1) {
+                    uint2 t[8];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) t[j] = (rot & sh) ? out[(j + sh) & 7] : out[j];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) out[j] = t[j];
+                }
+#pragma unroll
+                for (int j = 0; j < 8; ++j) *reinterpret_cast<uint2*>(base + (size_t)((j + rot) & 7) * 32) = out[j];
+            } else {
+                u32x4 out[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) out[j] = u32x4{v[0][j], v[1][j], v[2][j], v[3][j]};
+#pragma unroll
+                for (int sh = 1; sh < 4; sh <<= 1) {
+                    u32x4 t[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) t[j] = (rot & sh) ? out[(j + sh) & 3] : out[j];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) out[j] = t[j];
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) *reinterpret_cast<u32x4*>(base + (size_t)((j + rot) & 3) * 32) = out[j];
+            }
+        };
+        load_task(in[0], 0);
+        load_task(in[1], 1);
+        // zeros behind a tile's rows and behind K, while the rows are on their way: the slots behind the full height of
+        // every tile but the last, and those behind the rows that the last tile has
+        {
+            const int behind = (kTileSlots - a.tile_rows) * VPS, full = (T - 1) * behind;
+            const int rows_last = a.K - (T - 1) * a.tile_rows, count = full + (kTileSlots - rows_last) * VPS;
+            for (int i = tid; i < count; i += NT) {
+                const int p = i < full ? (i / behind) * kTileSlots * VPS + a.tile_rows * VPS + i % behind
+                                       : (T - 1) * kTileSlots * VPS + rows_last * VPS + (i - full);
+                *reinterpret_cast<u32x4*>(image + (size_t)p * 16) = u32x4{0u, 0u, 0u, 0u};
+            }
+        }
+        first_pieces();  // (the descriptors were asked for before the rows: they are here first)
+        for (int turn = 0; tid + turn * NT < tasks; turn += 2) {
+            store_task(in[0], turn);
+            if (wave * 64 + (turn + 2) * NT < tasks) load_task(in[0], turn + 2);  // (wave-uniform)
+            store_task(in[1], turn + 1);
+            if (wave * 64 + (turn + 3) * NT < tasks) load_task(in[1], turn + 3);
+        }
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of the image (and its first loads)
+    // the blocks this wave sends out at the end (b = wave, wave + 16, ...): what their chained epilogue needs, asked for now
+    float4 row_factors = make_float4(1.f, 1.f, 1.f, 1.f);
+    ChainOperands early = {{0.f, 0.f, 0.f, 0.f}, 0.f};
+    if (XF16 && wave < nblk) {
+        if (a.chain_sq_in) row_factors = chain_row_factors(a, lane);
+        early = chain_operands(a, (b0 + wave) * TL_BLOCK_COLUMNS + (lane >> 2), lane & 3);
+    }
+    // this wave's share of the image has landed when only the NP loads of its first runs, asked for behind it, are
+    // outstanding (the row-major path wrote the image with ordinary stores, which the barrier itself waits for)
+    if constexpr (!ROWS_IN) {
+        if constexpr (NP == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+        static_assert(NP == 4 || NP == 6, "the wait counts the loads of the first runs");
+    }
     __syncthreads();
 
-    float acc[8];
+    float acc[NA];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+    for (int e = 0; e < NA; ++e) acc[e] = 0.f;
     auto issue4 = [](u32x4 (&v)[4], const unsigned char* xq, uint32_t word) {
         using lds_cptr = const __attribute__((address_space(3))) void*;
 #pragma unroll
@@ -1129,8 +1238,12 @@ __global__ __launch_bounds__(kResWaves * 64) void tl_spmm_res16(KernelArgs a)
         for (int b = 0; b < 4; ++b)
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                acc[2 * e] = fmaf(__half2float(__ushort_as_half((unsigned short)(v[b][e] & 0xffffu))), sign, acc[2 * e]);
-                acc[2 * e + 1] = fmaf(__half2float(__ushort_as_half((unsigned short)(v[b][e] >> 16))), sign, acc[2 * e + 1]);
+                if constexpr (XF16) {
+                    acc[2 * e] = fmaf(__half2float(__ushort_as_half((unsigned short)(v[b][e] & 0xffffu))), sign, acc[2 * e]);
+                    acc[2 * e + 1] = fmaf(__half2float(__ushort_as_half((unsigned short)(v[b][e] >> 16))), sign, acc[2 * e + 1]);
+                } else {
+                    acc[e] = fmaf(__uint_as_float(v[b][e]), sign, acc[e]);
+                }
             }
     };
 
@@ -1186,19 +1299,19 @@ __global__ __launch_bounds__(kResWaves * 64) void tl_spmm_res16(KernelArgs a)
         if (u + 1 == u1 || (u + 1) / T != b) {
             // last unit of this wave in block b: fold the two signs of a column, leave the sums in slot (wave + b)
 #pragma unroll
-            for (int e = 0; e < 8; ++e) acc[e] += __shfl_xor(acc[e], 32, 64);
+            for (int e = 0; e < NA; ++e) acc[e] += __shfl_xor(acc[e], 32, 64);
             if (sgn == 0) {
-                float4* out = reinterpret_cast<float4*>(slots + (size_t)(wave + b) * kResSlotFloats + c16 * 16 + h * 8);
+                float4* out = reinterpret_cast<float4*>(slots + (size_t)(wave + b) * kResSlotFloats + c16 * MT + h * NA);
                 out[0] = make_float4(acc[0], acc[1], acc[2], acc[3]);
-                out[1] = make_float4(acc[4], acc[5], acc[6], acc[7]);
+                if constexpr (NA == 8) out[1] = make_float4(acc[4], acc[5], acc[6], acc[7]);
             }
 #pragma unroll
-            for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+            for (int e = 0; e < NA; ++e) acc[e] = 0.f;
         }
         c_cur = c_nxt; c_nxt = c_nx2; c_nx2 = c_nx3;
         d_cur = d_nxt; d_nxt = d_nx2;
     }
-    if (touched == 0x5a5aa5a5u && a.M < 0) slots[0] = 0.f;  // (never: keeps the cache-warming loads in the program)
+    if ((touched ^ touched2) == 0x5a5aa5a5u && a.M < 0) slots[0] = 0.f;  // (never: keeps the cache-warming loads in the program)
     __syncthreads();
     // Block b goes out through wave b % 16: lane = column lane / 4, rows 4 * (lane % 4) .. + 3, the slots of the waves
     // that had units in the block added in wave order.
@@ -1206,14 +1319,28 @@ __global__ __launch_bounds__(kResWaves * 64) void tl_spmm_res16(KernelArgs a)
         const int col = lane >> 2, q = lane & 3;
         // the waves with units in block b, in order: unit x belongs to wave ((x + 1) * W - 1) / U
         const int w_first = ((b * T + 1) * W - 1) / U, w_last = ((b + 1) * T * W - 1) / U;
+        const int nb = b0 + b, n = nb * TL_BLOCK_COLUMNS + col;
+        const float sc = n < a.N ? load_scale(a.w0.scale, a.scale_f16, n) : 0.f;
+        if constexpr (!XF16) {
+            // eight fp32 rows: two per lane; the plain product only
+            float2 pair = make_float2(0.f, 0.f);
+            for (int w = w_first; w <= w_last; ++w)
+                if (w * U / W < (w + 1) * U / W) {  // (a wave without units left nothing)
+                    const float2 o = *reinterpret_cast<const float2*>(slots + (size_t)(w + b) * kResSlotFloats + col * MT + q * 2);
+                    pair.x += o.x; pair.y += o.y;
+                }
+            if (n < a.N) {
+                if (m0 + q * 2 < a.M) store_out(a.Y, a.y_f16, (long long)(m0 + q * 2) * a.ldy + n, pair.x * sc);
+                if (m0 + q * 2 + 1 < a.M) store_out(a.Y, a.y_f16, (long long)(m0 + q * 2 + 1) * a.ldy + n, pair.y * sc);
+            }
+            continue;
+        }
         float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
         for (int w = w_first; w <= w_last; ++w)
             if (w * U / W < (w + 1) * U / W) {  // (a wave without units left nothing)
-                const float4 o = *reinterpret_cast<const float4*>(slots + (size_t)(w + b) * kResSlotFloats + col * 16 + q * 4);
+                const float4 o = *reinterpret_cast<const float4*>(slots + (size_t)(w + b) * kResSlotFloats + col * MT + q * 4);
                 sum.x += o.x; sum.y += o.y; sum.z += o.z; sum.w += o.w;
             }
-        const int nb = b0 + b, n = nb * TL_BLOCK_COLUMNS + col;
-        const float sc = n < a.N ? load_scale(a.w0.scale, a.scale_f16, n) : 0.f;
         if (b >= W) {  // (more than 16 blocks per workgroup: asked for late)
             if (a.chain_sq_in) row_factors = chain_row_factors(a, lane);
             early = chain_operands(a, n, q);
@@ -2580,34 +2707,66 @@ int launch_octet_kernel(KernelArgs a, const tl_layout_header* h, hipStream_t st)
     return TL_OK;
 }
 
-// tl_spmm_res16: one workgroup per compute unit, each with a range of whole blocks.  It fits when the image of all of
-// K and the slots of the block sums fit the LDS, and the runs are short enough for a lane's registers.
-inline int res16_workgroups(const KernelArgs& a) { return std::min(compute_units(), a.NB); }
+// tl_spmm_res: one workgroup per compute unit, each with a range of whole blocks of one slot of rows (16 fp16 or 8
+// fp32 rows; the slots of a taller input share the compute units out among themselves).  It fits when the image of
+// all of K and the slots of the block sums fit the LDS, and the runs are short enough for a lane's registers.
+struct ResShape {
+    int parts;       // slots of rows
+    int groups;      // workgroups per slot
+    int pieces;      // 16-byte pieces of a run in a lane's registers (4 or 6), 0: does not fit
+    size_t lds;
+};
 
-inline size_t res16_lds(const KernelArgs& a)
+inline ResShape res_shape(const KernelArgs& a, const tl_layout_header* h)
 {
-    const int nblk_max = (int)ceil_div(a.NB, res16_workgroups(a));
-    return (size_t)a.T * kTileSlots * 16 * 2 + (size_t)(kResWaves + nblk_max - 1) * kResSlotFloats * 4;
+    ResShape r;
+    const int rows = a.x_f16 ? 16 : 8;
+    r.parts = (int)ceil_div(a.M, rows);
+    r.groups = std::max(1, std::min(compute_units() / r.parts, a.NB));
+    const int nblk_max = (int)ceil_div(a.NB, r.groups);
+    r.lds = (size_t)a.T * kTileSlots * 32 + (size_t)(kResWaves + nblk_max - 1) * TL_BLOCK_COLUMNS * rows * 4;
+    // a lane keeps 16 or 24 dwords (64 or 96 rows) of a run in registers and fetches the rest one by one: the mean
+    // run of one sign (half of the header's figure, which counts both) should stay well below that
+    r.pieces = h->mean_run_dwords_x16 <= 16 * 26 ? 4 : (h->mean_run_dwords_x16 <= 16 * 40 ? 6 : 0);
+    if (r.lds > 160 * 1024 || r.parts > 3 || r.parts > compute_units()) r.pieces = 0;
+    return r;
 }
 
-inline bool res16_fits(const KernelArgs& a, const tl_layout_header* h)
+template <bool XF16, int NP, bool ROWS_IN>
+int launch_res_np(KernelArgs a, const ResShape& shape, hipStream_t st)
 {
-    // a lane keeps 16 dwords (64 rows) of a run in registers and fetches the rest one by one: for sparse weights only
-    return res16_lds(a) <= 160 * 1024 && h->mean_run_dwords_x16 <= 16 * 26;
-}
-
-int launch_res16_kernel(KernelArgs a, const tl_layout_header* h, hipStream_t st)
-{
-    (void)h;
-    a.xs_bytes = a.T * kTileSlots * 16 * 2;
-    auto kernel = tl_spmm_res16<4>;
-    static bool raised = false;  // a repeated or racing call is harmless
+    a.xs_bytes = a.T * kTileSlots * 32;
+    a.tile_magic = (unsigned)(((1ull << 32) + a.tile_rows - 1) / a.tile_rows);
+    auto kernel = tl_spmm_res<XF16, NP, ROWS_IN>;
+    static bool raised = false;  // per instantiation; a repeated or racing call is harmless
     if (!raised) {
         if (int rc = raise_lds_limit(kernel, 160 * 1024)) return rc;
         raised = true;
     }
-    hipLaunchKernelGGL(kernel, dim3((unsigned)res16_workgroups(a)), dim3(kResWaves * 64), res16_lds(a), st, a);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)shape.groups, (unsigned)shape.parts), dim3(kResWaves * 64), shape.lds, st, a);
     return TL_OK;
+}
+
+// Row-major activations that tl_spmm_res turns into its image itself: rows of whole 16-byte pieces, aligned, and tiles
+// of whole pieces (no piece of a row straddles two tiles).
+inline bool res_takes_rows(const KernelArgs& a)
+{
+    const int es = a.x_f16 ? 2 : 4, kv = 16 / es;
+    return !a.x_kmajor && (a.ldx * es) % 16 == 0 && reinterpret_cast<uintptr_t>(a.X) % 16 == 0 && a.K % kv == 0 && a.tile_rows % kv == 0 &&
+           a.K < (1 << 24);
+}
+
+template <bool XF16, bool ROWS_IN>
+int launch_res_in(const KernelArgs& a, const ResShape& shape, hipStream_t st)
+{
+    return shape.pieces == 4 ? launch_res_np<XF16, 4, ROWS_IN>(a, shape, st) : launch_res_np<XF16, 6, ROWS_IN>(a, shape, st);
+}
+
+int launch_res_kernel(const KernelArgs& a, const tl_layout_header* h, hipStream_t st)
+{
+    const ResShape shape = res_shape(a, h);
+    if (!a.x_kmajor) return a.x_f16 ? launch_res_in<true, true>(a, shape, st) : launch_res_in<false, true>(a, shape, st);
+    return a.x_f16 ? launch_res_in<true, false>(a, shape, st) : launch_res_in<false, false>(a, shape, st);
 }
 
 // The direct-load kernel for one activation row.  All of K in one group when `share` workgroups of that
@@ -2730,8 +2889,10 @@ int launch_small(KernelArgs a, const tl_layout_header* h, int x_dtype, void* wor
         octet = mt == 16 && a.x_f16 && knob(TL_OCTET, ceil_div(a.NB, 2) * ceil_div(a.M, 16) >= 2 * (int64_t)compute_units() ? 1 : 0) != 0;
         // ... or, up to 16 rows and where it fits, the whole image resident in LDS and one workgroup per compute unit
         // (it pays where a compute unit has more than one block to work through; TL_RES16=1 takes it wherever it fits, 0 never)
-        resident = mt == 16 && a.x_f16 && a.M <= 16 && (a.y_f16 || !(a.gated || chain_out || a.chain_sq_in)) && res16_fits(a, h) &&
-                   knob(TL_RES16, a.NB > compute_units() ? 1 : 0) != 0;
+        if (mt == 16 && a.M <= 16 && (a.x_f16 ? (a.y_f16 || !(a.gated || chain_out || a.chain_sq_in)) : !(a.gated || chain_out || a.chain_sq_in))) {
+            const ResShape shape = res_shape(a, h);
+            resident = shape.pieces != 0 && knob(TL_RES16, (int64_t)a.NB * shape.parts > compute_units() ? 1 : 0) != 0;
+        }
         if ((chain_out || a.chain_sq_in) && (mt != 16 || !a.x_f16 || !a.y_f16 || a.M > 16))
             return fail(TL_ERR_UNSUPPORTED, "chained products are for 9 to 16 fp16 rows");
         if (a.gated && !octet && !resident)
@@ -2740,7 +2901,7 @@ int launch_small(KernelArgs a, const tl_layout_header* h, int x_dtype, void* wor
     }
     // Slots of 8 and 16 rows are copied into LDS as 16-byte pieces of an aligned K-major image; activations
     // that are not one already are brought into that form in the workspace first.
-    if (mt >= 8 && !(a.x_kmajor && aligned && a.ldx >= round_up(a.M, mt))) {
+    if (mt >= 8 && !(a.x_kmajor && aligned && a.ldx >= round_up(a.M, mt)) && !(resident && res_takes_rows(a))) {
         const int64_t need = small_kmajor_bytes(h, a.M, x_dtype);
         if (!workspace || workspace_bytes < need)
             return fail(TL_ERR_SIZE, "workspace has %lld bytes, %lld needed", (long long)workspace_bytes, (long long)need);
@@ -2762,7 +2923,7 @@ int launch_small(KernelArgs a, const tl_layout_header* h, int x_dtype, void* wor
     }
     if (mt >= 8) {
         if (mt == 8) return a.x_f16 ? launch_quad_kernel<8, true>(a, h, st) : launch_quad_kernel<8, false>(a, h, st);
-        if (resident) return launch_res16_kernel(a, h, st);
+        if (resident) return launch_res_kernel(a, h, st);
         if (octet) return launch_octet_kernel(a, h, st);
         if (wide) return a.x_f16 ? launch_quad_kernel<16, true, 1024>(a, h, st) : launch_quad_kernel<16, false, 1024>(a, h, st);
         return a.x_f16 ? launch_quad_kernel<16, true>(a, h, st) : launch_quad_kernel<16, false>(a, h, st);

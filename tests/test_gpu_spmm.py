@@ -257,7 +257,7 @@ def test_small_m_kernels_in_every_mode(cuda, oracle, dtype):
 
 
 def test_resident_16_row_kernel_and_its_epilogues(cuda, oracle):
-    """9 to 16 fp16 rows with the activation image resident in LDS (tl_spmm_res16, TL_RES16=1): exact on integer
+    """9 to 16 rows with the activation image resident in LDS (tl_spmm_res, TL_RES16=1): exact on integer
     activations against the oracle -- one and several blocks per workgroup, ragged K and N, dense and sparse
     weights (runs longer than a lane's registers hold), a tile height with a single zero slot -- and every epilogue
     (scale, fp32 output, SiLU gate row-major and K-major, residual, next-norm image and squares, row factors)
@@ -306,3 +306,16 @@ def test_resident_16_row_kernel_and_its_epilogues(cuda, oracle):
         if "gated_k" in outs["new"]:  # the padding rows of a K-major image are zeros
             img = outs["new"]["gated_k"]
             assert not img.as_strided((N // 2, 16), (16, 1))[:, M:].any()
+        # fp32 rows: slots of eight, two workgroups side by side; row-major rows (turned inside the kernel) and a K-major image
+        x32 = x.float().to(cuda)
+        scale32 = scale.float()
+        for tag, env in (("old", {"TL_RES16": "0"}), ("new", {"TL_RES16": "1"})):
+            print(f"case K={K} N={N} M={M} s={s} tile_rows={tile_rows} fp32 {tag}", flush=True)
+            with knobs(**env):
+                outs[tag] = {"plain": ops.spmm(dw, x32), "scaled": ops.spmm(dw, x32, scale32),
+                             "kmajor": ops.spmm(dw, x32.t().contiguous(), scale32, x_layout=_lib.TL_X_K_MAJOR),
+                             "strided": ops.spmm(dw, torch.cat([x32, x32], 1)[:, :K], scale32)}
+            torch.cuda.synchronize()
+        assert np.array_equal(outs["new"]["plain"].cpu().numpy().astype(np.float64), ref), (K, N, M)
+        for name in outs["new"]:
+            assert torch.equal(outs["new"][name], outs["old"][name]), (K, N, M, name)
