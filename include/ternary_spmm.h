@@ -162,9 +162,8 @@ typedef struct tl_layout_header {
     uint64_t total_bytes;    /* bytes of the blob that are in use, multiple of 256                        */
     uint32_t max_run_dwords; /* largest (+1 run dwords + -1 run dwords) of any (column, tile)             */
     uint32_t mean_run_dwords_x16; /* mean of the same, times 16, rounded up                               */
-    uint64_t checksum;       /* FNV-1a (64-bit, one step per dword) over chunk table, run order and stream */
-    uint64_t off_runorder;   /* byte offset of uint16 runorder[NB][T * 16], or 0 when T * 16 >= 65536       */
-    uint32_t reserved[38];
+    uint64_t checksum;       /* FNV-1a (64-bit, one step per dword) over the chunk table, then the stream */
+    uint32_t reserved[40];   /* zero */
 } tl_layout_header;
 
 /* Bytes of the blob that tl_layout_build will write for these tiled-CSC arrays
@@ -173,7 +172,9 @@ typedef struct tl_layout_header {
 int tl_layout_size(const int32_t* neg_off_tiled, const int32_t* pos_off_tiled,
                    int columns, int inners, int tile_k, int tile_rows, int64_t* blob_bytes);
 
-/* Builds the blob into host memory `blob` (blob_bytes as returned above). */
+/* Builds the blob into host memory `blob` (blob_bytes as returned above).  The pass that orders the rows of each
+ * tile runs on worker threads (environment variable TL_PACK_THREADS, read at every call; default: the hardware
+ * threads, 8 at most, divided among the calls in that pass at the moment); the blob does not depend on their number. */
 int tl_layout_build(const int32_t* neg_row, const int32_t* neg_off_tiled,
                     const int32_t* pos_row, const int32_t* pos_off_tiled,
                     int columns, int inners, int tile_k, int tile_rows,
@@ -267,6 +268,14 @@ int tl_spmm_time(const tl_layout_header* header, const void* blob_dev,
                  const void* scale, int scale_dtype,
                  void* workspace, int64_t workspace_bytes, void* stream,
                  int iters, float* mean_ms);
+
+/* Measurement helper with no counterpart in the reference: one launch that only READS `bytes` bytes
+ * (a multiple of 16, 16-byte aligned) of device memory, every lane 16 bytes at a time, and leaves one
+ * folded dword per workgroup in out[0 .. tl_read_probe_workgroups() - 1].  The benchmark runs it under
+ * the same HIP-graph replay as the single-row products: the box's own floor for a launch that must
+ * stream a weight of that size once. */
+int tl_read_probe_workgroups(void);
+int tl_stream_read_probe(const void* src, int64_t bytes, void* out, void* stream);
 
 /* ======================================================================== */
 /* Around the products of a single-token decode step.                       */

@@ -6,9 +6,19 @@ Two providers with one interface:
     checkout into oracle/_ref/libref_cpu.so by oracle/Makefile, behind oracle/ref_cpu_shim.cpp;
   * "port": this repository's restatement of the same kernels (oracle/cpu_port.cpp).
 The reference build uses AVX-512 in every function, so it is only offered on hosts with avx512f/bw/vl/dq.
+
+Timing follows the plan the reference's driver implies (ternaryLLM_CPU/src/main.cpp:1014,1069-1099: 10 runs)
+with the threads held still: one OpenMP thread per PHYSICAL core of the process's CPU set, bound
+(OMP_PROC_BIND=close, OMP_PLACES=cores).  The OpenMP runtime reads those variables once, when it starts, and
+a process that has imported torch has started it long before: the timed kernels therefore run in a child
+process (`python -m oracle.cpu_baseline ...`) whose environment is set before anything loads OpenMP.
 """
 import ctypes
+import json
 import os
+import subprocess
+import sys
+import tempfile
 import time
 
 import numpy as np
@@ -28,6 +38,7 @@ def _cpu_flags():
 
 
 def cpu_model():
+    """The full `model name` line of /proc/cpuinfo."""
     try:
         with open("/proc/cpuinfo") as f:
             for line in f:
@@ -38,6 +49,39 @@ def cpu_model():
     return "unknown"
 
 
+def physical_cores():
+    """Distinct (package, core) pairs among the CPUs this process may run on; the logical CPU count of that set
+    when /proc/cpuinfo does not say."""
+    try:
+        allowed = os.sched_getaffinity(0)
+    except AttributeError:
+        allowed = set(range(os.cpu_count() or 1))
+    cores, cpu, pkg = set(), None, 0
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                key, _, val = line.partition(":")
+                key = key.strip()
+                if key == "processor":
+                    cpu = int(val)
+                elif key == "physical id":
+                    pkg = int(val)
+                elif key == "core id" and cpu in allowed:
+                    cores.add((pkg, int(val)))
+    except (OSError, ValueError):
+        cores = set()
+    return len(cores) if cores else len(allowed)
+
+
+def threads():
+    """Threads of a timed run: one per physical core, no more than OMP_NUM_THREADS when the host sets it."""
+    n = physical_cores()
+    cap = os.environ.get("OMP_NUM_THREADS")
+    if cap and cap.isdigit() and int(cap) > 0:
+        n = min(n, int(cap))
+    return max(1, n)
+
+
 def _aligned(shape, dtype=np.float32, align=64):
     n = int(np.prod(shape))
     raw = np.zeros(n * np.dtype(dtype).itemsize + align, np.uint8)
@@ -45,17 +89,12 @@ def _aligned(shape, dtype=np.float32, align=64):
     return raw[off:off + n * np.dtype(dtype).itemsize].view(dtype).reshape(shape)
 
 
-class _Provider:
-    kind = None
-
-    def gemm(self, x_km, w_i8, M, N, K):
-        raise NotImplementedError
-
-
-class ReferenceProvider(_Provider):
+class ReferenceProvider:
+    """The reference's own kernels; `which` is "avx2" (32 rows x 8 columns, the reference's headline choice
+    "MergedMin_32G8_AVX2", main.cpp:1018,1088) or "avx512" (32 x 16, GEMM_CPU_FP32.cpp:8365)."""
     kind = "reference"
 
-    def __init__(self):
+    def __init__(self, which="avx2"):
         path = os.path.join(_HERE, "_ref", "libref_cpu.so")
         need = {"avx2", "fma", "avx512f", "avx512bw", "avx512vl", "avx512dq"}
         if not os.path.exists(path):
@@ -69,20 +108,24 @@ class ReferenceProvider(_Provider):
         for fn in (L.ref_gemm_32xg8_avx2, L.ref_gemm_32xg16_avx512):
             fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int]
         self.L = L
-        self.kernel_name = "GEMM_CPU_FP32_colMajor_TCSC_Merged_GroupMin_32xG16_AVX512_OpenMP"
+        self.group = 8 if which == "avx2" else 16
+        self.fn = L.ref_gemm_32xg8_avx2 if which == "avx2" else L.ref_gemm_32xg16_avx512
+        self.kernel_name = ("GEMM_CPU_FP32_colMajor_TCSC_Merged_GroupMin_32xG8_AVX2_OpenMP" if which == "avx2"
+                            else "GEMM_CPU_FP32_colMajor_TCSC_Merged_GroupMin_32xG16_AVX512_OpenMP")
 
     def build(self, w_i8, K, N):
-        return self.L.ref_group_build(w_i8.ctypes.data, K, N, 16)
+        return self.L.ref_group_build(w_i8.ctypes.data, K, N, self.group)
 
     def free(self, h):
         self.L.ref_group_free(h)
 
     def run(self, h, x_km, y_nm, M, N, K):
-        self.L.ref_gemm_32xg16_avx512(x_km.ctypes.data, h, y_nm.ctypes.data, M, N, K)
+        self.fn(x_km.ctypes.data, h, y_nm.ctypes.data, M, N, K)
 
 
-class PortProvider(_Provider):
+class PortProvider:
     kind = "port"
+    group = 8
 
     def __init__(self):
         path = os.path.join(_HERE, "libcpu_port.so")
@@ -93,7 +136,8 @@ class PortProvider(_Provider):
         L.port_group_build.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]
         L.port_group_free.argtypes = [ctypes.c_void_p]
         L.port_gemm_32xg8_avx2.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int]
-        L.port_gemv_g64_avx2.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int]
+        for fn in (L.port_gemv_g64_avx2, L.port_gemv_g64_avx512):
+            fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int]
         self.L = L
         self.kernel_name = "port of GEMM_CPU_FP32_colMajor_TCSC_Merged_GroupMin_32xG8_AVX2_OpenMP"
 
@@ -106,35 +150,34 @@ class PortProvider(_Provider):
     def run(self, h, x_km, y_nm, M, N, K):
         self.L.port_gemm_32xg8_avx2(x_km.ctypes.data, h, y_nm.ctypes.data, M, N, K)
 
-    def gemv(self, w_i8, x, N, K):
+    def gemv(self, w_i8, x, N, K, wide=False):
         h = self.L.port_group_build(w_i8.ctypes.data, K, N, 64, 0)
         y = np.zeros(N, np.float32)
-        self.L.port_gemv_g64_avx2(np.ascontiguousarray(x, np.float32).ctypes.data, h, y.ctypes.data, N, K)
+        (self.L.port_gemv_g64_avx512 if wide else self.L.port_gemv_g64_avx2)(np.ascontiguousarray(x, np.float32).ctypes.data, h, y.ctypes.data, N, K)
         self.L.port_group_free(h)
         return y
 
 
-def provider(prefer_reference=True):
+def _stats(samples):
+    s = sorted(samples)
+    return {"min": s[0], "median": s[len(s) // 2], "mean": sum(s) / len(s), "max": s[-1]}
+
+
+def _gemm_providers(prefer_reference):
+    out = []
     if prefer_reference:
-        try:
-            return ReferenceProvider()
-        except (RuntimeError, OSError):
-            pass
-    return PortProvider()
+        for which in ("avx2", "avx512"):
+            try:
+                out.append(ReferenceProvider(which))
+            except (RuntimeError, OSError):
+                pass
+    if not out:
+        out.append(PortProvider())
+    return out
 
 
-def threads():
-    return int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-
-
-def time_gemm(w, x, runs=10, prefer_reference=True, check=True):
-    """Times Y = X @ W on the CPU with the reference's headline kernel.
-
-    w: int [K, N] ternary, x: float [M, K] (M % 32 == 0, N % 16 == 0).  Converts to the kernel's
-    layouts (X as [K][M], result [N][M], 64-byte aligned), checks the result against the float64
-    product, then reports the mean of `runs` calls, like the reference's driver
-    (ternaryLLM_CPU/src/main.cpp:1014,1069-1099)."""
-    p = provider(prefer_reference)
+def _time_gemm_here(w, x, runs, prefer_reference, check):
+    """Runs in the process whose OpenMP environment is already what it should be."""
     K, N = w.shape
     M = x.shape[0]
     assert M % 32 == 0 and N % 16 == 0 and K < 32768
@@ -142,47 +185,115 @@ def time_gemm(w, x, runs=10, prefer_reference=True, check=True):
     x_km = _aligned((K, M))
     x_km[:] = np.asarray(x, np.float32).T
     y_nm = _aligned((N, M))
-    h = p.build(w8, K, N)
-    p.run(h, x_km, y_nm, M, N, K)
-    max_err = None
-    if check:
-        ref = (np.asarray(x, np.float64) @ w.astype(np.float64)).T
-        scale = np.maximum(np.abs(ref), np.linalg.norm(x, axis=1)[None, :] * np.sqrt(np.count_nonzero(w) / w.size))
-        max_err = float(np.max(np.abs(y_nm - ref) / scale))
-        if max_err > 1e-4:
-            p.free(h)
-            raise RuntimeError(f"CPU baseline kernel disagrees with the exact product (max rel err {max_err})")
-    t0 = time.perf_counter()
-    for _ in range(runs):
+    results = []
+    for p in _gemm_providers(prefer_reference):
+        h = p.build(w8, K, N)
         p.run(h, x_km, y_nm, M, N, K)
-    dt = (time.perf_counter() - t0) / runs
-    p.free(h)
-    return {"seconds": dt, "kind": p.kind, "kernel": p.kernel_name, "threads": threads(), "max_rel_err": max_err,
-            "cpu": cpu_model()}
+        max_err = None
+        if check:
+            ref = (np.asarray(x, np.float64) @ w.astype(np.float64)).T
+            scale = np.maximum(np.abs(ref), np.linalg.norm(x, axis=1)[None, :] * np.sqrt(np.count_nonzero(w) / w.size))
+            max_err = float(np.max(np.abs(y_nm - ref) / scale))
+            if max_err > 1e-4:
+                p.free(h)
+                raise RuntimeError(f"CPU baseline kernel disagrees with the exact product (max rel err {max_err})")
+        samples = []
+        for _ in range(runs):
+            t0 = time.perf_counter()
+            p.run(h, x_km, y_nm, M, N, K)
+            samples.append(time.perf_counter() - t0)
+        p.free(h)
+        st = _stats(samples)
+        results.append({"seconds": st["mean"], "seconds_min": st["min"], "seconds_median": st["median"], "seconds_max": st["max"],
+                        "runs": runs, "kind": p.kind, "kernel": p.kernel_name, "group": p.group, "max_rel_err": max_err})
+    return results
 
 
-def time_gemv(w, x, runs=20):
-    """Times y = x @ W (one row) on the CPU with this repository's port of the reference's decode kernel
-    GEMV_CPU_FP32_rowMajor_TCSC_Merged_GroupMin_G64_AVX2_OpenMP (ternaryLLM_CPU/src/GEMM_CPU_FP32.cpp:15008-15081;
-    the reference's own file holds it behind aligned loads that fault under GCC, so the port is what runs).
-    w: int [K, N] ternary (N % 64 == 0), x: float [K].  Checked against the float64 product first."""
+def _time_gemv_here(w, x, runs):
     p = PortProvider()
     K, N = w.shape
     assert N % 64 == 0 and K < 32768
     w8 = np.ascontiguousarray(w, dtype=np.int8)
     xv = np.ascontiguousarray(x, np.float32)
-    y = np.zeros(N, np.float32)
-    h = p.L.port_group_build(w8.ctypes.data, K, N, 64, 0)
-    p.L.port_gemv_g64_avx2(xv.ctypes.data, h, y.ctypes.data, N, K)
     ref = xv.astype(np.float64) @ w.astype(np.float64)
-    max_err = float(np.max(np.abs(y - ref)) / max(1e-9, np.abs(ref).max()))
-    if max_err > 1e-4:
-        p.L.port_group_free(h)
-        raise RuntimeError(f"CPU GEMV port disagrees with the exact product (max err / max {max_err})")
-    t0 = time.perf_counter()
-    for _ in range(runs):
-        p.L.port_gemv_g64_avx2(xv.ctypes.data, h, y.ctypes.data, N, K)
-    dt = (time.perf_counter() - t0) / runs
+    h = p.L.port_group_build(w8.ctypes.data, K, N, 64, 0)
+    results = []
+    kernels = [("port of GEMV_CPU_FP32_rowMajor_TCSC_Merged_GroupMin_G64_AVX2_OpenMP", p.L.port_gemv_g64_avx2)]
+    if "avx512f" in _cpu_flags():
+        kernels.append(("port of GEMV_CPU_FP32_rowMajor_TCSC_Merged_GroupMin_G64_AVX512_OpenMP", p.L.port_gemv_g64_avx512))
+    for name, fn in kernels:
+        y = np.zeros(N, np.float32)
+        fn(xv.ctypes.data, h, y.ctypes.data, N, K)
+        max_err = float(np.max(np.abs(y - ref)) / max(1e-9, np.abs(ref).max()))
+        if max_err > 1e-4:
+            p.L.port_group_free(h)
+            raise RuntimeError(f"CPU GEMV port disagrees with the exact product (max err / max {max_err})")
+        samples = []
+        for _ in range(runs):
+            t0 = time.perf_counter()
+            fn(xv.ctypes.data, h, y.ctypes.data, N, K)
+            samples.append(time.perf_counter() - t0)
+        st = _stats(samples)
+        results.append({"seconds": st["mean"], "seconds_min": st["min"], "seconds_median": st["median"], "seconds_max": st["max"],
+                        "runs": runs, "kind": "port", "kernel": name, "max_err_over_max": max_err})
     p.L.port_group_free(h)
-    return {"seconds": dt, "kind": "port", "kernel": "port of GEMV_CPU_FP32_rowMajor_TCSC_Merged_GroupMin_G64_AVX2_OpenMP",
-            "threads": threads(), "max_err_over_max": max_err, "cpu": cpu_model()}
+    return results
+
+
+def _in_child(mode, w, x, runs, prefer_reference=True, check=True):
+    """Writes the operands where a child process finds them, runs `python -m oracle.cpu_baseline` there with the
+    OpenMP variables set, and returns what it printed."""
+    n = threads()
+    env = dict(os.environ, OMP_NUM_THREADS=str(n), OMP_PROC_BIND="close", OMP_PLACES="cores", OMP_DYNAMIC="false")
+    with tempfile.TemporaryDirectory(prefix="tl_cpu_baseline_") as tmp:
+        path = os.path.join(tmp, "operands.npz")
+        np.savez(path, w=np.ascontiguousarray(w, dtype=np.int8), x=np.asarray(x, np.float32))
+        cmd = [sys.executable, "-m", "oracle.cpu_baseline", mode, path, str(runs), "1" if prefer_reference else "0", "1" if check else "0"]
+        done = subprocess.run(cmd, cwd=os.path.dirname(_HERE), env=env, capture_output=True, text=True, timeout=600)
+    if done.returncode != 0:
+        raise RuntimeError("CPU baseline child failed: " + (done.stderr.strip().splitlines() or ["?"])[-1])
+    results = json.loads(done.stdout.strip().splitlines()[-1])
+    for r in results:
+        r.update({"threads": n, "cpu": cpu_model(), "binding": "OMP_PROC_BIND=close OMP_PLACES=cores, one thread per physical core"})
+    return results
+
+
+def time_gemm_all(w, x, runs=10, prefer_reference=True, check=True):
+    """Times Y = X @ W on the CPU with the reference's GEMM kernels, every one this host can run: the AVX2
+    32 x 8 kernel (the reference's own headline choice) first, its AVX-512 32 x 16 sibling second; this
+    repository's port of the first where the reference build is absent.
+
+    w: int [K, N] ternary, x: float [M, K] (M % 32 == 0, N % 16 == 0).  Operands are converted to the kernels'
+    layouts (X as [K][M], result [N][M], 64-byte aligned), the result is checked against the float64 product,
+    then each kernel is called `runs` times; `seconds` is the mean (the reference driver's statistic), minimum,
+    median and maximum beside it."""
+    return _in_child("gemm", w, x, runs, prefer_reference, check)
+
+
+def time_gemm(w, x, runs=10, prefer_reference=True, check=True):
+    """The first entry of time_gemm_all: the reference's headline kernel."""
+    return time_gemm_all(w, x, runs, prefer_reference, check)[0]
+
+
+def time_gemv_all(w, x, runs=20):
+    """Times y = x @ W (one row) on the CPU with this repository's ports of the reference's decode kernels
+    GEMV_CPU_FP32_rowMajor_TCSC_Merged_GroupMin_G64_AVX2_OpenMP (ternaryLLM_CPU/src/GEMM_CPU_FP32.cpp:15008-15081)
+    and ..._G64_AVX512_OpenMP (:15684-15729); the reference's own file holds them behind aligned loads that fault
+    under GCC, so the ports are what runs.  w: int [K, N] ternary (N % 64 == 0), x: float [K].  Checked against
+    the float64 product first."""
+    return _in_child("gemv", w, np.asarray(x, np.float32)[None, :], runs)
+
+
+def time_gemv(w, x, runs=20):
+    return time_gemv_all(w, x, runs)[0]
+
+
+if __name__ == "__main__":
+    mode, path, runs = sys.argv[1], sys.argv[2], int(sys.argv[3])
+    with np.load(path) as z:
+        w_, x_ = z["w"].astype(np.int32), z["x"]
+    if mode == "gemm":
+        res = _time_gemm_here(w_, x_, runs, sys.argv[4] == "1", sys.argv[5] == "1")
+    else:
+        res = _time_gemv_here(w_, x_[0], runs)
+    print(json.dumps(res))

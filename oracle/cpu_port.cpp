@@ -16,7 +16,8 @@
 //   GEMM  32 rows x 8 columns, AVX2, OpenMP over column groups
 //         (GEMM_CPU_FP32.cpp:2956-3221); X is [K][M], result is [N][M].
 //   GEMV  64 columns per group, AVX2 i32 gathers on the paired part, scalar
-//         leftovers (GEMM_CPU_FP32.cpp:15008-15081); x row-major, int32 indices.
+//         leftovers (GEMM_CPU_FP32.cpp:15008-15081); x row-major, int32 indices;
+//         and its AVX-512 sibling (:15684-15729).
 #include <immintrin.h>
 #include <omp.h>
 
@@ -187,6 +188,36 @@ void port_gemv_g64_avx2(const float* x, void* h, float* result, int N, int K)
         }
         float* y = result + (size_t)j * 64;
         for (int q = 0; q < 8; ++q) _mm256_storeu_ps(y + 8 * q, acc[q]);
+        for (int c = 0; c < 64; ++c) {
+            float s = y[c];
+            for (int k = gd[1 + 2 * c]; k < gd[2 + 2 * c]; ++k) s += x[idx[k]];
+            for (int k = gd[2 + 2 * c]; k < gd[3 + 2 * c]; ++k) s -= x[idx[k]];
+            y[c] = s;
+        }
+    }
+}
+
+// The same with 16-lane gathers (GEMM_CPU_FP32.cpp:15684-15729): four accumulators of 16 columns.
+__attribute__((target("avx512f"))) void port_gemv_g64_avx512(const float* x, void* h, float* result, int N, int K)
+{
+    (void)K;
+    const Grouped* g = static_cast<const Grouped*>(h);
+    const int32_t* idx = g->idx32.data();
+    const int32_t* meta = g->meta.data();
+#pragma omp parallel for schedule(static)
+    for (int j = 0; j < N / 64; ++j) {
+        const int32_t* gd = meta + (size_t)j * 130;
+        __m512 acc[4];
+        for (int q = 0; q < 4; ++q) acc[q] = _mm512_setzero_ps();
+        for (int k = gd[0]; k < gd[1]; k += 128) {
+            for (int q = 0; q < 4; ++q) {
+                __m512i ip = _mm512_loadu_si512(idx + k + 16 * q);
+                __m512i in = _mm512_loadu_si512(idx + k + 64 + 16 * q);
+                acc[q] = _mm512_add_ps(acc[q], _mm512_sub_ps(_mm512_i32gather_ps(ip, x, 4), _mm512_i32gather_ps(in, x, 4)));
+            }
+        }
+        float* y = result + (size_t)j * 64;
+        for (int q = 0; q < 4; ++q) _mm512_storeu_ps(y + 16 * q, acc[q]);
         for (int c = 0; c < 64; ++c) {
             float s = y[c];
             for (int k = gd[1 + 2 * c]; k < gd[2 + 2 * c]; ++k) s += x[idx[k]];

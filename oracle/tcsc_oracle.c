@@ -14,16 +14,18 @@
  *                         brute force on tiny W, round trip to dense.
  *   orc_tiled_csc      -- closed form (row % TILE_K, exclusive cumsum of the
  *                         per-(column, tile) counts), invariants, round trip.
- *   orc_tiled_mcsc     -- six hand-worked cases (tests/golden/mcsc_hand_cases.json:
+ *   orc_tiled_mcsc     -- eight hand-worked cases (tests/golden/mcsc_hand_cases.json:
  *                         odd pair counts on either side, padding with
- *                         overwrite, the cursor overwrite across two tiles,
- *                         padded arrays), the p == n / even case that
+ *                         overwrite at padding sizes 4 and 8, the cursor
+ *                         overwrite across two tiles, padded arrays, four
+ *                         tiles of which three tie), the p == n / even case that
  *                         reduces to a plain interleave of orc_tiled_csc, the
  *                         alignment invariants of the offsets.  The reference
  *                         holds no fixture for it and its only other
  *                         implementation computes a different (untruncated)
  *                         format, so beyond those checks: parity unpinned.
- *   orc_tile_swizzle   -- numpy.argsort(kind="stable") per column; equals the
+ *   orc_tile_swizzle   -- numpy.argsort(kind="stable") per column and the hand case
+ *                         with three tied tiles; equals the
  *                         reference's std::sort only while a column has at
  *                         most 16 tiles (libstdc++ then runs a pure insertion
  *                         sort); above that the tie order of the reference is

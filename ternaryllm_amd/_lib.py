@@ -84,6 +84,8 @@ SIGNATURES = {
                               _VP, _I64, _VP]),
     "tl_spmm_time": (_INT, [_HDRP, _VP, _VP, _INT, _INT, _I64, _I64, _VP, _INT, _I64, _VP, _INT, _VP, _I64, _VP, _INT,
                             ctypes.POINTER(ctypes.c_float)]),
+    "tl_read_probe_workgroups": (_INT, []),
+    "tl_stream_read_probe": (_INT, [_VP, _I64, _VP, _VP]),
     "tl_rope_cache_update": (_INT, [_VP, _INT, _I64, _INT, _INT, _VP, _VP, _VP, _VP, _VP, _VP, _I64, _VP]),
     "tl_decode_attention": (_INT, [_VP, _VP, _VP, _INT, _I64, _INT, _INT, _I64, _VP, _VP, _I64, _VP]),
     "tl_decode_attention_split": (_INT, [_VP, _VP, _VP, _INT, _I64, _INT, _INT, _I64, _VP, _VP, _I64, _INT, _VP, _I64, _VP]),

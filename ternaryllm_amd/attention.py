@@ -9,7 +9,19 @@ import math
 import torch
 from torch import nn
 
+from . import ops
 from .linear import TernaryLinear
+from .packing import PackedWeight
+
+
+def side_by_side_key(device, projections):
+    """What a weight built from several projections depends on: the device, each projection's packed buffer and
+    scale (address and version, so that an assignment, an in-place edit or a state_dict load all count)."""
+    key = [device]
+    for p in projections:
+        key += [p.w_packed.data_ptr(), p.w_packed._version]
+        key += [None, None] if p.w_scale is None else [p.w_scale.data_ptr(), p.w_scale._version]
+    return tuple(key)
 
 
 def rope_tables(positions, head_dim, theta, dtype, device):
@@ -30,9 +42,15 @@ def apply_rope(x, cos, sin):
 
 
 class LlamaTernaryAttention(nn.Module):
-    def __init__(self, config, layer_idx=None, *, generator=None, reference_buffers=True):
+    def __init__(self, config, layer_idx=None, *, generator=None, reference_buffers=True, fused_qkv=True):
+        """fused_qkv: multiply the hidden states by ONE packed weight that holds the columns of q_proj, k_proj and
+        v_proj side by side (built from the three at the first forward on a device, and again when one of them
+        changes; a fourth blob as large as the three together): one pass over the activations, one re-layout and one
+        fix-up launch instead of three of each.  q_proj, k_proj and v_proj stay what the reference has there."""
         super().__init__()
         self.config = config
+        self.fused_qkv = fused_qkv
+        self._qkv = None  # (DeviceWeight, scale or None, key) of the side-by-side weight
         self.layer_idx = layer_idx
         self.hidden_size = config.hidden_size
         self.num_heads = config.num_attention_heads
@@ -58,6 +76,20 @@ class LlamaTernaryAttention(nn.Module):
         self.v_proj = make(self.hidden_size, self.num_key_value_heads * self.head_dim)
         self.o_proj = make(self.num_heads * self.head_dim, self.hidden_size)
 
+    def _qkv_weight(self, device):
+        """q | k | v side by side as one packed weight on `device`."""
+        projections = (self.q_proj, self.k_proj, self.v_proj)
+        key = side_by_side_key(device, projections)
+        if self._qkv is None or self._qkv[2] != key:
+            both = torch.cat([p.ternary_weight for p in projections], dim=1).contiguous()
+            scale = None
+            given = [p.w_scale for p in projections if p.w_scale is not None]
+            if given:  # a projection without a scale counts as one of ones, in the type of the first that has one
+                scale = torch.cat([(p.w_scale if p.w_scale is not None else torch.ones(p.out_features, device=device)).to(device, given[0].dtype)
+                                   for p in projections]).contiguous()
+            self._qkv = (ops.DeviceWeight(PackedWeight.from_dense(both.numpy()), device), scale, key)
+        return self._qkv[:2]
+
     def _rotary(self, position_ids, position_embeddings, q_len, past_len, dtype, device):
         if position_embeddings is not None:   # computed by the model, as newer `transformers` do
             cos, sin = position_embeddings
@@ -77,7 +109,7 @@ class LlamaTernaryAttention(nn.Module):
         attention_mask: additive, broadcastable to [batch, heads, q_len, kv_len]; longer masks are cut to
         the key length as in the reference (:103-105).  position_embeddings: (cos, sin) of
         [batch or 1, q_len, head_dim], else they are computed from position_ids ([q_len] or
-        [batch, q_len]), else from the cache length.  past_key_value: a `transformers` Cache (updated in
+        [batch, q_len]), else from cache_position, else from the cache's length.  past_key_value: a `transformers` Cache (updated in
         place with `layer_idx`; newer versions pass it as `past_key_values`) or a (k, v) tuple of
         [batch, kv_heads, past, head_dim]; with a tuple, or with use_cache and no cache, the third
         result is the new (k, v) tuple.  position_offset: position of the first token when neither
@@ -85,13 +117,26 @@ class LlamaTernaryAttention(nn.Module):
         if past_key_value is None:
             past_key_value = kwargs.pop("past_key_values", None)
         bsz, q_len, _ = hidden_states.shape
-        q = self.q_proj(hidden_states).view(bsz, q_len, -1, self.head_dim).transpose(1, 2)
-        k = self.k_proj(hidden_states).view(bsz, q_len, -1, self.head_dim).transpose(1, 2)
-        v = self.v_proj(hidden_states).view(bsz, q_len, -1, self.head_dim).transpose(1, 2)
+        if self.fused_qkv and hidden_states.is_cuda:
+            weight, scale = self._qkv_weight(hidden_states.device)
+            nq, nkv = self.q_proj.out_features, self.k_proj.out_features
+            qkv = ops.spmm(weight, hidden_states.reshape(bsz * q_len, -1), scale).view(bsz, q_len, nq + 2 * nkv)
+            q, k, v = (t.reshape(bsz, q_len, -1, self.head_dim).transpose(1, 2) for t in qkv.split((nq, nkv, nkv), dim=-1))
+        else:
+            q = self.q_proj(hidden_states).view(bsz, q_len, -1, self.head_dim).transpose(1, 2)
+            k = self.k_proj(hidden_states).view(bsz, q_len, -1, self.head_dim).transpose(1, 2)
+            v = self.v_proj(hidden_states).view(bsz, q_len, -1, self.head_dim).transpose(1, 2)
         is_tuple = isinstance(past_key_value, (tuple, list))
         past_len = position_offset
         if past_len is None:
-            past_len = past_key_value[0].shape[2] if is_tuple else 0
+            if is_tuple:
+                past_len = past_key_value[0].shape[2]
+            elif cache_position is not None and torch.is_tensor(cache_position) and cache_position.numel() > 0:
+                past_len = int(cache_position.reshape(-1)[0])   # the position of the first new token
+            elif past_key_value is not None and hasattr(past_key_value, "get_seq_length"):
+                past_len = int(past_key_value.get_seq_length(self.layer_idx))
+            else:
+                past_len = 0
         cos, sin = self._rotary(position_ids, position_embeddings, q_len, past_len, q.dtype, q.device)
         q, k = apply_rope(q, cos, sin), apply_rope(k, cos, sin)
         if is_tuple:

@@ -3430,6 +3430,42 @@ extern "C" int tl_mlp_gate_up(const tl_layout_header* gate_header, const void* g
     return finish_launch();
 }
 
+// Reads `pieces` 16-byte pieces and folds them: what streaming that much memory costs a launch that writes next to
+// nothing.  256 threads a workgroup, eight pieces of a thread in flight per turn.
+__global__ __launch_bounds__(256) void tl_read_probe(const u32x4* __restrict__ src, long long pieces, uint32_t* __restrict__ out)
+{
+    constexpr int U = 8;
+    const long long stride = (long long)gridDim.x * 256;
+    uint32_t fold = 0;
+    for (long long first = (long long)blockIdx.x * 256 + threadIdx.x; first < pieces; first += stride * U) {
+        u32x4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = first + u * stride < pieces ? src[first + u * stride] : u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int u = 0; u < U; ++u) fold ^= v[u][0] ^ v[u][1] ^ v[u][2] ^ v[u][3];
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) fold ^= __shfl_xor(fold, off, 64);
+    __shared__ uint32_t part[4];
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = fold;
+    __syncthreads();
+    if (threadIdx.x == 0) out[blockIdx.x] = part[0] ^ part[1] ^ part[2] ^ part[3];
+}
+
+extern "C" int tl_read_probe_workgroups(void) { return 8 * compute_units(); }
+
+extern "C" int tl_stream_read_probe(const void* src, int64_t bytes, void* out, void* stream)
+{
+    if (!src || !out) return fail(TL_ERR_ARG, "device pointer is null");
+    if (bytes <= 0 || bytes % 16) return fail(TL_ERR_SIZE, "bytes=%lld must be a positive multiple of 16", (long long)bytes);
+    if (reinterpret_cast<uintptr_t>(src) % 16 || reinterpret_cast<uintptr_t>(out) % 4) return fail(TL_ERR_ALIGN, "src must be 16-byte, out 4-byte aligned");
+    const long long pieces = bytes / 16;
+    const int groups = (int)std::min<long long>(tl_read_probe_workgroups(), ceil_div(pieces, 256));
+    hipLaunchKernelGGL(tl_read_probe, dim3((unsigned)groups), dim3(256), 0, static_cast<hipStream_t>(stream), static_cast<const u32x4*>(src), pieces,
+                       static_cast<uint32_t*>(out));
+    return finish_launch();
+}
+
 extern "C" int tl_spmm_time(const tl_layout_header* header, const void* blob_dev,
                             const void* X, int x_dtype, int x_layout, int64_t ldx, int64_t M,
                             void* Y, int y_dtype, int64_t ldy,

@@ -15,6 +15,9 @@
 #include <cmath>
 #include <cstring>
 #include <algorithm>
+#include <atomic>
+#include <cstdlib>
+#include <thread>
 #include <vector>
 
 #include "tl_common.h"
@@ -303,6 +306,20 @@ uint64_t content_checksum(const uint32_t* chunkstart, size_t n_table, const uint
     return h;
 }
 
+// Threads for the row-ordering pass of one tl_layout_build call: TL_PACK_THREADS if set, else the machine's hardware
+// threads up to 8, shared among the calls that are in that pass at the moment (callers that pack many weights on
+// threads of their own then get one each).  The caller gives its count back when its pass is over.
+std::atomic<int> g_builds_running{0};
+
+int pack_workers(int n_blocks)
+{
+    int cap = 0;
+    if (const char* e = std::getenv("TL_PACK_THREADS")) cap = std::atoi(e);
+    if (cap <= 0) cap = (int)std::min(8u, std::max(1u, std::thread::hardware_concurrency()));
+    const int running = g_builds_running.fetch_add(1) + 1;
+    return std::max(1, std::min(cap / running, n_blocks));
+}
+
 // Last "end" entry of a tiled-CSC offset array = number of stored rows of that sign.
 int64_t stream_length(const int32_t* off_tiled, int columns, int inners, int tile_k)
 {
@@ -396,7 +413,6 @@ extern "C" int tl_layout_build(const int32_t* neg_row, const int32_t* neg_off_ti
         }
     std::vector<uint64_t> cursor((size_t)T * 2);
     uint8_t* bytes = reinterpret_cast<uint8_t*>(stream);
-    std::vector<RunRef> runs(8);
     for (int y = 0; y < columns; ++y) {
         const int nb = y / kBlock, j = y % kBlock;
         for (int t = 0; t < T; ++t) {
@@ -415,20 +431,38 @@ extern "C" int tl_layout_build(const int32_t* neg_row, const int32_t* neg_off_ti
                     bytes[cursor[2 * (k / g.tile_rows) + sign]++] = (uint8_t)(k % g.tile_rows);
                 }
         }
-        // the block is complete: order the rows inside every group of 8 neighbouring columns of a tile (the single-row
-        // kernel puts 32 lanes, half a wave, on them: four per column, and the LDS serves half a wave at a time)
-        if (j == kBlock - 1 || y == columns - 1)
-            for (int t = 0; t < T; ++t) {
-                const uint64_t c0 = chunkstart[(size_t)nb * T + t];
-                for (int j0 = 0; j0 <= j; j0 += 8) {
-                    const int gsz = std::min(8, j + 1 - j0);
-                    for (int i = 0; i < gsz; ++i) {
-                        const uint32_t d = stream[c0 + j0 + i];
-                        runs[i] = RunRef{bytes + (c0 + (d >> 16)) * 4, (int)(d & 0xff), (int)((d >> 8) & 0xff), t};
-                    }
-                    spread_over_banks(runs.data(), gsz, kSpreadSweeps, g.tile_rows);
+    }
+
+    // Pass 3: order the rows inside every group of 8 neighbouring columns of a tile (the single-row kernel puts 32
+    // lanes, half a wave, on them: four per column, and the LDS serves half a wave at a time).  Blocks are
+    // independent of each other and the order found depends on the block alone, so worker threads take blocks in
+    // turn: the blob does not depend on how many there are.
+    auto order_block = [&](int nb) {
+        RunRef runs[8];
+        const int cols = std::min(kBlock, columns - nb * kBlock);
+        for (int t = 0; t < T; ++t) {
+            const uint64_t c0 = chunkstart[(size_t)nb * T + t];
+            for (int j0 = 0; j0 < cols; j0 += 8) {
+                const int gsz = std::min(8, cols - j0);
+                for (int i = 0; i < gsz; ++i) {
+                    const uint32_t d = stream[c0 + j0 + i];
+                    runs[i] = RunRef{bytes + (c0 + (d >> 16)) * 4, (int)(d & 0xff), (int)((d >> 8) & 0xff), t};
                 }
+                spread_over_banks(runs, gsz, kSpreadSweeps, g.tile_rows);
             }
+        }
+    };
+    {
+        const int workers = pack_workers(NB);
+        std::atomic<int> next{0};
+        auto work = [&]() {
+            for (int nb = next.fetch_add(1); nb < NB; nb = next.fetch_add(1)) order_block(nb);
+        };
+        std::vector<std::thread> pool;
+        for (int i = 1; i < workers; ++i) pool.emplace_back(work);
+        work();
+        for (auto& th : pool) th.join();
+        g_builds_running.fetch_sub(1);
     }
 
     tl_layout_header h;

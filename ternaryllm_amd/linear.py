@@ -239,10 +239,7 @@ class TernaryLinear(nn.Module):
         if input.dim() >= 2 and input.shape[-2] == K:  # K-major activations
             if input.dim() == 2:
                 return ops.spmm(w, input, self.w_scale, x_layout=1)
-            out = torch.empty((input.shape[0], input.shape[2], N), dtype=input.dtype, device=input.device)
-            for b in range(input.shape[0]):
-                ops.spmm(w, input[b], self.w_scale, x_layout=1, out=out[b])
-            return out
+            return ops.spmm_kmajor_batch(w, input, self.w_scale)
         raise ValueError(f"input of shape {tuple(input.shape)} does not match in_features={K}")
 
     def extra_repr(self):

@@ -343,6 +343,7 @@ class TernaryLlamaDecoder(nn.Module):
 
     def _advance(self, st):
         logits = self._decode_step(st["token"], st["pos"], st["mask"])
+        self.last_logits = logits  # (under a captured graph: the tensor every replay writes)
         st["token"].copy_(logits.argmax(-1))
         # positions stay inside the cache even if a caller steps past its end (the results are then
         # meaningless, but nothing is written out of bounds; generate() checks the length up front)

@@ -6,8 +6,25 @@ import torch
 from torch import nn
 
 from . import ops
+from .attention import side_by_side_key
 from .linear import TernaryLinear
 from .packing import PackedWeight
+
+
+def activation_function(name):
+    """The activation the reference looks up in transformers' ACT2FN (TernaryMLP.py:30): that table when the package
+    is there, else the handful of torch functions Llama-style configurations name."""
+    try:
+        from transformers.activations import ACT2FN
+        return ACT2FN[name]
+    except (ImportError, KeyError):
+        table = {"silu": torch.nn.functional.silu, "swish": torch.nn.functional.silu, "gelu": torch.nn.functional.gelu,
+                 "relu": torch.nn.functional.relu, "gelu_new": lambda t: torch.nn.functional.gelu(t, approximate="tanh"),
+                 "gelu_pytorch_tanh": lambda t: torch.nn.functional.gelu(t, approximate="tanh"), "tanh": torch.tanh,
+                 "sigmoid": torch.sigmoid}
+        if name not in table:
+            raise ValueError(f"activation {name!r} unknown")
+        return table[name]
 
 
 class LlamaTernaryMLP(nn.Module):
@@ -24,8 +41,9 @@ class LlamaTernaryMLP(nn.Module):
         self._pairs = None  # (DeviceWeight, scale or None, what it was built from) of the paired weight
         self.hidden_size = config.hidden_size
         self.intermediate_size = config.intermediate_size
-        if config.hidden_act != "silu":
-            raise ValueError("only the SiLU gate of Llama is supported")
+        # the fused kernels gate with SiLU; any other activation of the reference's table (TernaryMLP.py:30,
+        # transformers' ACT2FN) runs as two products and the torch operator
+        self.hidden_act = getattr(config, "hidden_act", "silu")
         scales = scales or {}
 
         def make(k, n, name):
@@ -37,12 +55,13 @@ class LlamaTernaryMLP(nn.Module):
         self.gate_proj = make(self.hidden_size, self.intermediate_size, "gate")
         self.up_proj = make(self.hidden_size, self.intermediate_size, "up")
         self.down_proj = make(self.intermediate_size, self.hidden_size, "down")
-        self.act_fn = torch.nn.functional.silu
+        self.act_fn = activation_function(self.hidden_act)
 
     def _paired_weight(self, device):
         """The (gate, up) pair weight on `device`: column 2j the gate, column 2j + 1 the up projection of output j."""
-        # built again when the device or either projection's packed buffer changes (a move, a state_dict load)
-        key = (device, self.gate_proj.w_packed.data_ptr(), self.up_proj.w_packed.data_ptr())
+        # built again when the device, either projection's packed buffer or either scale changes (a move, an
+        # assignment, an edit in place, a state_dict load)
+        key = side_by_side_key(device, (self.gate_proj, self.up_proj))
         if self._pairs is None or self._pairs[2] != key:
             g, u = self.gate_proj.ternary_weight, self.up_proj.ternary_weight
             both = torch.empty((g.shape[0], 2 * g.shape[1]), dtype=torch.int32)
@@ -60,6 +79,9 @@ class LlamaTernaryMLP(nn.Module):
     def forward(self, x):
         lead = x.shape[:-1]
         x2 = x.reshape(-1, self.hidden_size)
+        if self.hidden_act not in ("silu", "swish"):
+            h = self.act_fn(self.gate_proj(x2)) * self.up_proj(x2)
+            return self.down_proj(h).reshape(*lead, self.hidden_size)
         if self.paired:
             weight, scale = self._paired_weight(x2.device)
             h = ops.spmm_gated(weight, x2, scale)

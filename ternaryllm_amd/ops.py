@@ -140,6 +140,14 @@ def spmm(weight, x, scale=None, out_dtype=None, x_layout=_lib.TL_X_ROW_MAJOR, ou
     return y
 
 
+def spmm_kmajor_batch(weight, x3, scale=None):
+    """[batch, K, rows] -> [batch, rows, N]: the batch's K-major matrices laid side by side as one [K, batch * rows]
+    matrix (one copy when batch > 1), then ONE product over all of them instead of one per batch entry."""
+    batch, K, rows = x3.shape
+    side_by_side = x3[0] if batch == 1 else x3.permute(1, 0, 2).reshape(K, batch * rows)
+    return spmm(weight, side_by_side, scale, x_layout=_lib.TL_X_K_MAJOR).view(batch, rows, weight.columns)
+
+
 def spmm_gated(weight, x, scale=None, x_layout=_lib.TL_X_ROW_MAJOR, kmajor=False):
     """h[M, N / 2] with h[:, j] = silu(y[:, 2j]) * y[:, 2j + 1], y = (x @ W) * scale, for a gate | up weight whose
     columns are (gate, up) pairs.  One launch (tl_spmm_gated) where the shape's kernel has the epilogue -- one
@@ -364,6 +372,19 @@ def spmm_time(weight, x, iters, scale=None, out_dtype=None, x_layout=_lib.TL_X_R
                                      ctypes.byref(ms))
     _lib.check(rc)
     return ms.value, y
+
+
+def stream_read_probe(buf, out=None):
+    """One launch that only reads the bytes of `buf` (a contiguous cuda tensor of a multiple of 16 bytes), folded into
+    one dword per workgroup of `out` (made when not given): the floor of a launch that streams that much memory."""
+    n = _lib.lib().tl_read_probe_workgroups()
+    if out is None:
+        out = torch.empty(n, dtype=torch.int32, device=buf.device)
+    if out.numel() < n or out.dtype != torch.int32 or not buf.is_contiguous():
+        raise ValueError("out must hold one int32 per probe workgroup, buf must be contiguous")
+    with torch.cuda.device(buf.device):
+        _lib.check(_lib.lib().tl_stream_read_probe(buf.data_ptr(), buf.numel() * buf.element_size(), out.data_ptr(), _stream_ptr(buf.device)))
+    return out
 
 
 def rope_cache_update(qkv, cos_table, sin_table, pos, q_out, k_cache, v_cache):

@@ -66,12 +66,15 @@ def _prepared(rows, offs, columns, inners, uniformed):
 
 
 def ter_spmm(X, w_tiled_merged_row_indice, w_tiled_merged_col_offset, w_col_tile_indices,
-             batch_size, rows, columns, inners, uniformed, padded):
+             batch_size, rows, columns, inners, uniformed, padded, *, x_layout=None):
     """-> new tensor [batch_size, rows, columns]  (ter_spmm_wrapper.cu:318-348).
 
     X is [batch, rows, inners] (what the reference's modules pass) or [batch, inners, rows]
     (what the reference kernel reads, ter_spmm_kernel.cuh:173); the two are told apart by
-    shape.  float32 as in the reference, float16 in addition.
+    shape.  When rows == inners the shape does not tell: X is then read as [batch, rows, inners]
+    unless x_layout says otherwise.  x_layout (not in the reference's signature): None (by shape),
+    "row_major" / 0 for [batch, rows, inners], "k_major" / 1 for [batch, inners, rows]; a layout
+    that the shape contradicts raises ValueError.  float32 as in the reference, float16 in addition.
     `uniformed`: the same-sign part of every tile is left out, as in the reference's kernels.
     `padded`: accepted; every pair of the arrays is walked.  (Under this flag the reference's M > 1
     kernel leaves out what remains of a tile's pair part after whole groups of 8 entries, 16 for
@@ -89,11 +92,15 @@ def ter_spmm(X, w_tiled_merged_row_indice, w_tiled_merged_col_offset, w_col_tile
     if X.numel() != batch_size * rows * inners:
         raise ValueError("X does not hold batch_size * rows * inners elements")
     x3 = X.reshape(batch_size, *X.shape[-2:]) if X.dim() >= 2 else X.reshape(batch_size, rows, inners)
-    if x3.shape[-1] == inners and x3.shape[-2] == rows:
+    layouts = {None: None, "row_major": _lib.TL_X_ROW_MAJOR, "k_major": _lib.TL_X_K_MAJOR,
+               _lib.TL_X_ROW_MAJOR: _lib.TL_X_ROW_MAJOR, _lib.TL_X_K_MAJOR: _lib.TL_X_K_MAJOR}
+    if x_layout not in layouts:
+        raise ValueError(f"x_layout={x_layout!r}: expected None, 'row_major' (0) or 'k_major' (1)")
+    asked = layouts[x_layout]
+    if asked != _lib.TL_X_K_MAJOR and x3.shape[-1] == inners and x3.shape[-2] == rows:
         return ops.spmm(weight, x3.reshape(batch_size * rows, inners)).reshape(batch_size, rows, columns)
-    if x3.shape[-2] == inners and x3.shape[-1] == rows:
-        out = torch.empty((batch_size, rows, columns), dtype=X.dtype, device=X.device)
-        for b in range(batch_size):
-            ops.spmm(weight, x3[b], x_layout=_lib.TL_X_K_MAJOR, out=out[b])
-        return out
+    if asked != _lib.TL_X_ROW_MAJOR and x3.shape[-2] == inners and x3.shape[-1] == rows:
+        return ops.spmm_kmajor_batch(weight, x3)
+    if asked is not None:
+        raise ValueError(f"X of shape {tuple(X.shape)} is not x_layout={x_layout!r} for rows={rows}, inners={inners}")
     raise ValueError(f"X of shape {tuple(X.shape)} is neither [batch, rows, inners] nor [batch, inners, rows]")

@@ -34,6 +34,34 @@ def test_ter_spmm_drop_in_on_merged_arrays(cuda, oracle):
     assert empty.shape == (0, 4, N)  # what the reference returns for a 2-D input (batch_size = 0)
 
 
+def test_ter_spmm_square_input_reads_row_major_unless_told(cuda, oracle):
+    """rows == inners: the shape of X does not tell [batch, rows, inners] from [batch, inners, rows].  Without
+    x_layout the shim reads it as the reference's modules pass it (row-major); x_layout="k_major" reads the same
+    buffer as the reference kernel does; a layout that the shape contradicts is refused."""
+    import ter_spmm
+    K, N, tk = 256, 48, 64
+    w = ternary_weight(K, N, 0.7, 44)
+    wt = torch.from_numpy(w)
+    tm = ter_spmm.convert_to_ter_tiled_mcsc(wt, N, K, (wt == 1).sum().item(), (wt == -1).sum().item(), tk, False, 4)
+    rows = torch.from_numpy(tm[0]).to(torch.int16).to(cuda)
+    offs = torch.from_numpy(tm[1]).to(cuda)
+    tiles = torch.from_numpy(tm[2]).to(torch.int16).to(cuda)
+    bs = 2
+    x = activations(bs * K, K, 45, torch.float32, integer=True).reshape(bs, K, K)
+    as_rows = np.stack([oracle.mcsc_product(x[b].numpy(), tm[0], tm[1], N, tk) for b in range(bs)])
+    as_kmajor = np.stack([oracle.mcsc_product(x[b].t().contiguous().numpy(), tm[0], tm[1], N, tk) for b in range(bs)])
+    assert not np.array_equal(as_rows, as_kmajor)
+    xd = x.to(cuda)
+    for layout, want in ((None, as_rows), ("row_major", as_rows), (0, as_rows), ("k_major", as_kmajor), (1, as_kmajor)):
+        y = ter_spmm.ter_spmm(xd, rows, offs, tiles, bs, K, N, K, False, False, x_layout=layout)
+        assert np.array_equal(y.cpu().numpy().astype(np.float64), want), layout
+    narrow = xd[:, :8].contiguous()   # [batch, 8, K]: only row-major fits
+    with pytest.raises(ValueError):
+        ter_spmm.ter_spmm(narrow, rows, offs, tiles, bs, 8, N, K, False, False, x_layout="k_major")
+    with pytest.raises(ValueError):
+        ter_spmm.ter_spmm(narrow, rows, offs, tiles, bs, 8, N, K, False, False, x_layout="columns")
+
+
 def _hand_cases():
     import json
     import os
@@ -241,6 +269,59 @@ def test_attention_block_against_torch(cuda):
     attn.is_causal = True
     ref4 = (torch.softmax((q @ k.transpose(-1, -2)) / 8.0, -1) @ v).transpose(1, 2).reshape(B, S, 256) @ wo
     assert torch.allclose(o4.cpu(), ref4, rtol=2e-4, atol=2e-4 * ref4.abs().max().item())
+
+
+def test_attention_with_one_weight_for_q_k_v(cuda):
+    """fused_qkv: q | k | v as one packed weight gives what the three projections give one by one (integer
+    activations: every sum is exact, so bit for bit), with and without scales, for 1, 12 and 200 tokens; the
+    side-by-side weight follows a projection that changes."""
+    from ternaryllm_amd import LlamaTernaryAttention, TernaryConfig
+    g = torch.Generator().manual_seed(14)
+    cfg = TernaryConfig(hidden_size=512, num_attention_heads=8, num_key_value_heads=2, sparsity=0.85)
+    attn = LlamaTernaryAttention(cfg, generator=g).to(cuda).half()
+    other = LlamaTernaryAttention(cfg, generator=g).to(cuda).half()
+
+    def both(x):
+        attn.fused_qkv = True
+        one = attn(x, use_cache=True)
+        attn.fused_qkv = False
+        three = attn(x, use_cache=True)
+        attn.fused_qkv = True
+        return one, three
+
+    for scaled in (False, True):
+        if scaled:
+            attn.q_proj.w_scale = (0.5 + torch.rand(512, generator=g)).half().to(cuda)
+            attn.v_proj.w_scale = (0.5 + torch.rand(128, generator=g)).half().to(cuda)   # k_proj stays without one
+        for tokens in (1, 12, 200):
+            x = activations(tokens, 512, 70 + tokens, torch.float16, integer=True).reshape(1, tokens, 512).to(cuda) / 64
+            one, three = both(x)
+            assert attn._qkv[0].columns == 512 + 2 * 128
+            assert torch.equal(one[2][0], three[2][0]) and torch.equal(one[2][1], three[2][1])   # keys and values
+            assert torch.equal(one[0], three[0])
+    before = attn._qkv[0]
+    attn.k_proj.load_state_dict(other.k_proj.state_dict())
+    x = activations(4, 512, 99, torch.float16, integer=True).reshape(1, 4, 512).to(cuda) / 64
+    one, three = both(x)
+    assert attn._qkv[0] is not before and torch.equal(one[0], three[0]) and torch.equal(one[2][0], three[2][0])
+
+
+def test_mlp_block_with_another_activation(cuda):
+    """hidden_act other than "silu" (TernaryMLP.py:30-34 looks the activation up by name): the block is two
+    products, the named activation in torch and the down product; against an fp64 restatement."""
+    from ternaryllm_amd import LlamaTernaryMLP, TernaryConfig
+    g = torch.Generator().manual_seed(15)
+    for act, fn in (("gelu", torch.nn.functional.gelu), ("relu", torch.relu)):
+        cfg = TernaryConfig(hidden_size=256, intermediate_size=768, sparsity=0.8, hidden_act=act)
+        for paired in (False, True):
+            mlp = LlamaTernaryMLP(cfg, generator=g, paired=paired).to(cuda)
+            for tokens in (1, 40):
+                x = 0.1 * torch.randn((tokens, 256), generator=g)
+                wg, wu, wd = (p.ternary_weight.double() for p in (mlp.gate_proj, mlp.up_proj, mlp.down_proj))
+                ref = (fn(x.double() @ wg) * (x.double() @ wu)) @ wd
+                y = mlp(x.to(cuda))
+                assert y.shape == (tokens, 256) and y.dtype == torch.float32
+                assert (y.double().cpu() - ref).abs().max().item() <= FP32_TOL * ref.abs().max().item()
 
 
 def test_full_size_properties(cuda):

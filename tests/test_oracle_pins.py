@@ -111,6 +111,7 @@ def test_mcsc_product_hand_worked(oracle, case):
     the same-sign part with its sign, the row offset of a second tile, dropped and mis-signed rows of the
     lossy tiles, a row named twice by padded arrays."""
     x = np.array(case["x"], np.float64)[None, :]
+    assert case["x"] == [3 ** (k % 11) + k for k in range(case["inners"])]   # the fixture's activation row, as its note defines it
     assert sum(s * case["x"][r] for s, r in case["product_terms"]) == case["product"]
     rows = np.array(case["merged_row_idx"], np.int32)
     off = np.array(case["merged_off"], np.int32)

@@ -256,6 +256,14 @@ def test_cpu_baselines_match_exact_product():
     p = cpu_baseline.PortProvider()
     xv = x[0]
     assert np.allclose(p.gemv(np.ascontiguousarray(w, np.int8), xv, 64, 1024), xv.astype(np.float64) @ w, atol=1e-3)
+    if "avx512f" in cpu_baseline._cpu_flags():
+        assert np.allclose(p.gemv(np.ascontiguousarray(w, np.int8), xv, 64, 1024, wide=True), xv.astype(np.float64) @ w, atol=1e-3)
+    # every kernel the host can run, one bound thread per physical core, run statistics beside the mean
+    both = cpu_baseline.time_gemm_all(w, x, runs=2)
+    assert both[0]["kernel"].endswith("32xG8_AVX2_OpenMP") and all(r["seconds_min"] <= r["seconds_median"] <= r["seconds_max"] for r in both)
+    assert both[0]["threads"] == cpu_baseline.threads() <= cpu_baseline.physical_cores()
+    for r in cpu_baseline.time_gemv_all(w, xv, runs=2):
+        assert r["max_err_over_max"] < 1e-5
 
 
 def test_compute_entry_points_reject_bad_arguments_before_any_launch():
