@@ -214,7 +214,7 @@ def sparsity_sweep_leg(dev, x, steps, sparsities=(0.70, 0.75, 0.80, 0.85, 0.90, 
     return rows
 
 
-def cold_decode_leg(dev, K=4096, N=4096, sparsity=0.66, copies=48, calls=1000, M=1):
+def cold_decode_leg(dev, K=4096, N=4096, sparsity=0.66, copies=48, calls=1000, M=1, kmajor=False):
     """Config 2 as the decoder meets it: `calls` SpMV calls, each with an x of its own, over `copies` distinct
     copies of the weight (about 300 MB, more than the last-level cache holds), captured as one HIP graph
     and replayed.  With M > 1: the same for a batch of M rows (row-major).  Beside it, under the same replay, the
@@ -232,7 +232,11 @@ def cold_decode_leg(dev, K=4096, N=4096, sparsity=0.66, copies=48, calls=1000, M
     g = torch.Generator().manual_seed(1245)
     xs = torch.randn((calls, M, K), generator=g).to(torch.float16).to(dev)  # a fresh x for every call of the graph
     ys = torch.empty((calls, M, N), dtype=torch.float16, device=dev)
-    t = graph_us_per_node(lambda i: ops.spmm(ws[i % copies], xs[i], out=ys[i]), calls, 12, full=True)
+    if kmajor:  # the activations as the decoder's kernels hand them from one product to the next: [K][M], M contiguous
+        xk = xs.transpose(1, 2).contiguous()
+        t = graph_us_per_node(lambda i: ops.spmm(ws[i % copies], xk[i], x_layout=ops._lib.TL_X_K_MAJOR, out=ys[i]), calls, 12, full=True)
+    else:
+        t = graph_us_per_node(lambda i: ops.spmm(ws[i % copies], xs[i], out=ys[i]), calls, 12, full=True)
     med = t["median"]
     # parity of the last replay: first and last call
     err = 0.0
@@ -246,8 +250,8 @@ def cold_decode_leg(dev, K=4096, N=4096, sparsity=0.66, copies=48, calls=1000, M
     whole = (dw.blob.numel() // 16) * 16
     read_t = graph_us_per_node(lambda i: ops.stream_read_probe(ws[i % copies].blob[:whole], folds), nodes, 12, full=True)
     B = pw.algorithmic_bytes(M, 2, 2)
-    out = {"M": M, "K": K, "N": N, "sparsity": sparsity, "weight_copies": copies, "distinct_x": calls,
-           "us_per_call_best10_mean": round(t["best10_mean"] * 1e6, 3),
+    out = {"M": M, "K": K, "N": N, "sparsity": sparsity, "x_layout": "K-major [K][M]" if kmajor else "row-major [M][K]", "weight_copies": copies,
+           "distinct_x": calls, "us_per_call_best10_mean": round(t["best10_mean"] * 1e6, 3),
            "GB_per_s": round(B / med / 1e9, 1), "pct_hbm_peak": round(100 * B / med / 1e9 / HBM_PEAK_GBS, 2),
            "tokens_per_s": round(M / med, 1), "max_err_over_max": err, "weight_bytes": int(dw.blob.numel()),
            "read_only_stream_of_one_weight_us": round(read_t["median"] * 1e6, 3),
@@ -297,6 +301,76 @@ def balanced_leg(dev, steps, warmup):
         row["balanced_over_iid"] = round(row["balanced_blocks_of_256"]["kernel_ms"] / row["iid"]["kernel_ms"], 4)
         out.append(row)
     return out
+
+
+def decode_nodes_leg(model, dev, pos_value):
+    """What bounds the single-row decode step, node by node: every kind of node of the captured step is replayed from a
+    graph of its 32 instances (one per layer, each with its own weights and cache: cold, as in the step), beside a
+    graph of read-only launches that stream the same bytes (the floor of a launch on this box).  The sum of the floors
+    is the step's bound here; the step's time over the sum of its nodes' is what the gaps between 162 nodes cost."""
+    import torch
+    from ternaryllm_amd import ops
+    c = model.config
+    eps, H, L = c.rms_norm_eps, c.hidden_size, model.layers
+    n_layers = len(L)
+    g = torch.Generator().manual_seed(1246)
+    x = (0.05 * torch.randn((1, H), generator=g)).to(model.dtype).to(dev)
+    pos = torch.full((1,), pos_value, dtype=torch.long, device=dev)
+    folds = torch.empty(ops._lib.lib().tl_read_probe_workgroups(), dtype=torch.int32, device=dev)
+    qkv_row = ops.spmv_fused(L[0].qkv_proj.device_weight(), "rmsnorm", x, None, L[0].input_layernorm.weight, eps, L[0].qkv_proj.w_scale)
+    att_row = model._attend(qkv_row, model._cache_of(L[0], 0), model._cache_of(L[0], 1), pos, False, splits=1)
+    gated_row = ops.spmv_fused(L[0].gate_up_proj.device_weight(), "rmsnorm", x, None, L[0].post_attention_layernorm.weight, eps,
+                               L[0].gate_up_proj.w_scale, gated=True)
+    kv_bytes = 2 * c.num_attention_heads * (pos_value + 1) * c.head_dim * x.element_size()
+    kv_bytes -= kv_bytes % 16
+
+    def blob(m):
+        b = m.device_weight().blob
+        return b[:(b.numel() // 16) * 16]
+
+    kinds = [
+        ("q|k|v product, RMSNorm on its input", lambda i: ops.spmv_fused(L[i].qkv_proj.device_weight(), "rmsnorm", x, None, L[i].input_layernorm.weight,
+                                                                        eps, L[i].qkv_proj.w_scale),
+         lambda i: ops.stream_read_probe(blob(L[i].qkv_proj), folds), blob(L[0].qkv_proj).numel()),
+        ("rotary + cache row + attention over %d rows" % (pos_value + 1),
+         lambda i: model._attend(qkv_row, model._cache_of(L[i], 0), model._cache_of(L[i], 1), pos, False, splits=1),
+         lambda i: ops.stream_read_probe(model._cache[i].reshape(-1).view(torch.uint8)[:kv_bytes], folds), kv_bytes),
+        ("o product + residual", lambda i: ops.spmv_add(L[i].o_proj.device_weight(), att_row, x, L[i].o_proj.w_scale),
+         lambda i: ops.stream_read_probe(blob(L[i].o_proj), folds), blob(L[0].o_proj).numel()),
+        ("gate|up product, RMSNorm on its input, SiLU gate in its epilogue",
+         lambda i: ops.spmv_fused(L[i].gate_up_proj.device_weight(), "rmsnorm", x, None, L[i].post_attention_layernorm.weight, eps,
+                                  L[i].gate_up_proj.w_scale, gated=True),
+         lambda i: ops.stream_read_probe(blob(L[i].gate_up_proj), folds), blob(L[0].gate_up_proj).numel()),
+        ("down product + residual", lambda i: ops.spmv_add(L[i].down_proj.device_weight(), gated_row, x, L[i].down_proj.w_scale),
+         lambda i: ops.stream_read_probe(blob(L[i].down_proj), folds), blob(L[0].down_proj).numel()),
+    ]
+    rows, sum_nodes, sum_floor = [], 0.0, 0.0
+    for name, node, probe, nbytes in kinds:
+        t = graph_us_per_node(node, n_layers, 12, full=True)
+        f = graph_us_per_node(probe, n_layers, 12, full=True)
+        rows.append({"node": name, "per_step": n_layers, "bytes": int(nbytes), "us": round(t["median"] * 1e6, 3), "us_min": round(t["min"] * 1e6, 3),
+                     "us_max": round(t["max"] * 1e6, 3), "read_floor_us": round(f["median"] * 1e6, 3),
+                     "time_over_read_floor": round(t["median"] / f["median"], 2)})
+        sum_nodes += n_layers * t["median"]
+        sum_floor += n_layers * f["median"]
+    # the head: once per step; timed behind the 32 q|k|v products of a graph (which push it out of the caches) as the
+    # difference to that graph without it
+    def with_head(i):
+        if i < n_layers:
+            return kinds[0][1](i)
+        return ops.spmv_fused(model.lm_head.device_weight(), "rmsnorm", x, None, model.norm.weight, eps, model.lm_head.w_scale)
+
+    def with_head_probe(i):
+        return kinds[0][2](i) if i < n_layers else ops.stream_read_probe(blob(model.lm_head), folds)
+
+    t_head = graph_us_per_node(with_head, n_layers + 1, 12, full=True)["median"] * (n_layers + 1) - rows[0]["us"] * 1e-6 * n_layers
+    f_head = graph_us_per_node(with_head_probe, n_layers + 1, 12, full=True)["median"] * (n_layers + 1) - rows[0]["read_floor_us"] * 1e-6 * n_layers
+    rows.append({"node": "head product, RMSNorm on its input", "per_step": 1, "bytes": int(blob(model.lm_head).numel()), "us": round(t_head * 1e6, 3),
+                 "read_floor_us": round(f_head * 1e6, 3), "time_over_read_floor": round(t_head / f_head, 2)})
+    sum_nodes += t_head
+    sum_floor += f_head
+    return {"nodes": rows, "sum_of_nodes_ms": round(sum_nodes * 1e3, 4), "sum_of_read_floors_ms": round(sum_floor * 1e3, 4),
+            "note": "each node kind replayed alone from a graph of its 32 per-layer instances; floors: read-only launches over the same bytes"}
 
 
 def decoder_leg(dev, prompt=512, new_tokens=128):
@@ -354,11 +428,20 @@ def decoder_leg(dev, prompt=512, new_tokens=128):
             print("bench.py: decoder check failed at batch %d (first replayed step equals eager: %s, tokens repeat: %s)"
                   % (B, first_step_equal, tokens_repeat), file=sys.stderr)
             sys.exit(1)
+        nodes = None
+        if B == 1 and model.fused_decode and model.native_decode:
+            nodes = decode_nodes_leg(model, dev, prompt + new_tokens // 2)
         res["batch_%d" % B] = {"prefill_ms": round(t_prefill * 1e3, 2), "prefill_tokens_per_s": round(B * prompt / t_prefill, 1),
                                "decode_ms_per_step": round(t_decode * 1e3 / new_tokens, 4),
                                "decode_tokens_per_s": round(B * new_tokens / t_decode, 1),
                                "end_to_end_tokens_per_s": round(B * (prompt + new_tokens) / (t_prefill + t_decode), 1),
                                "checked": "first replayed step == eager step bit for bit; %d greedy tokens repeat over two runs" % new_tokens}
+        if nodes is not None:
+            step_ms = res["batch_1"]["decode_ms_per_step"]
+            nodes["step_ms"] = step_ms
+            nodes["step_over_sum_of_nodes"] = round(step_ms / nodes["sum_of_nodes_ms"], 3)
+            nodes["step_over_sum_of_read_floors"] = round(step_ms / nodes["sum_of_read_floors_ms"], 3)
+            res["batch_1"]["per_node"] = nodes
     del model
     torch.cuda.empty_cache()
     return res
@@ -552,8 +635,8 @@ def main():
             except Exception as e:  # noqa: BLE001 - the baseline is optional, the GPU figures are not
                 extra["c2_cpu_baseline"] = {"value": None, "sample": "failed: %s" % e}
         # the decoder's other products, one row and sixteen, over 24 cold copies each
-        extra["decode_cold_shapes"] = [cold_decode_leg(dev, K, N, copies=24, calls=240, M=M)
-                                       for K, N in ((4096, 4096), (4096, 11008), (11008, 4096)) for M in (1, 16)]
+        extra["decode_cold_shapes"] = [cold_decode_leg(dev, K, N, copies=24, calls=240, M=M, kmajor=km)
+                                       for K, N in ((4096, 4096), (4096, 11008), (11008, 4096)) for M, km in ((1, False), (16, False), (16, True))]
     # ---- whole decoder: 32 layers, every linear ternary at 66 % sparsity -------
     if not args.no_extra and not args.no_decoder and not args.only_decode_shapes:
         extra["c5_decoder"] = decoder_leg(dev)

@@ -269,6 +269,31 @@ def test_decode_attention_over_a_long_cache(cuda):
         assert (out.double() - ref).abs().max().item() <= 3e-3 * max(1.0, ref.abs().max().item()), pos
 
 
+def test_decode_attention_ignores_what_lies_past_the_position(cuda):
+    """Cache rows behind the position are not part of the result whatever they hold (the kernel may ask for some of
+    them before it knows the position): NaN and infinities there change nothing, for 1 to 8 workgroups per head."""
+    from ternaryllm_amd import ops
+    g = torch.Generator().manual_seed(13)
+    B, H, hd, S = 2, 4, 128, 700
+    q = torch.randn((B, H, hd), generator=g).to(torch.float16).to(cuda)
+    kc = torch.randn((B, H, S, hd), generator=g).to(torch.float16).to(cuda)
+    vc = torch.randn((B, H, S, hd), generator=g).to(torch.float16).to(cuda)
+    for pos in (0, 5, 63, 64, 127, 128, 300, 698):
+        p = torch.tensor([pos], dtype=torch.long, device=cuda)
+        kz, vz, kn, vn = kc.clone(), vc.clone(), kc.clone(), vc.clone()
+        kz[:, :, pos + 1:] = 0
+        vz[:, :, pos + 1:] = 0
+        kn[:, :, pos + 1:] = float("nan")
+        vn[:, :, pos + 1:] = float("inf")
+        for splits in (1, 3, 8):
+            assert torch.equal(ops.decode_attention(q, kn, vn, p, splits=splits), ops.decode_attention(q, kz, vz, p, splits=splits)), (pos, splits)
+        n = pos + 1
+        sc = (q.double()[:, :, None, :] * kc.double()[:, :, :n]).sum(-1) / hd ** 0.5
+        ref = (sc.softmax(-1)[..., None] * vc.double()[:, :, :n]).sum(2).reshape(B, H * hd)
+        out = ops.decode_attention(q, kn, vn, p, splits=1)
+        assert (out.double() - ref).abs().max().item() <= 3e-3 * max(1.0, ref.abs().max().item()), pos
+
+
 def test_split_attention_and_its_fold_inside_the_output_projection(cuda, oracle):
     """tl_decode_attention_split: the cache rows of a head shared out among 1-8 workgroups, folded by the second
     launch, against the single-pass kernel and a float64 restatement (few rows, pieces without rows, a position
