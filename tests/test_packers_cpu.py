@@ -71,6 +71,22 @@ def test_device_blob_round_trip(K, N, tile_rows):
         assert np.array_equal(pw2.blob, pw.blob)
 
 
+def test_blob_does_not_depend_on_the_packing_threads(monkeypatch):
+    """The row-ordering pass of tl_layout_build runs on worker threads (TL_PACK_THREADS, read at every call): the
+    blob is the same byte for byte for 1, 3 and 8 of them, and when several calls pack at the same time."""
+    from concurrent.futures import ThreadPoolExecutor
+    w = ternary_weight(1000, 200, 0.66, 31)
+    blobs = []
+    for n in ("1", "3", "8"):
+        monkeypatch.setenv("TL_PACK_THREADS", n)
+        blobs.append(bytes(packing.PackedWeight.from_dense(w).blob))
+    assert blobs[0] == blobs[1] == blobs[2]
+    monkeypatch.delenv("TL_PACK_THREADS")
+    with ThreadPoolExecutor(max_workers=4) as pool:
+        together = list(pool.map(lambda _: bytes(packing.PackedWeight.from_dense(w).blob), range(6)))
+    assert all(b == blobs[0] for b in together)
+
+
 def test_blob_validation_catches_corruption():
     w = ternary_weight(512, 40, 0.6, 77)
     pw = packing.PackedWeight.from_dense(w)
