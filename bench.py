@@ -63,23 +63,12 @@ def weight_and_packed(K, N, sparsity, seed, device):
 
 def kernel_source_hash():
     """sha256 over the sources the headline's three kernels and their launcher are built from (the row-parallel
-    part of tl_kernels.hip, the blob builder, the shared constants): a traffic figure recorded for other sources
-    is not reported.  Edits to the other kernels of tl_kernels.hip leave it alone."""
+    kernels' translation unit, what it shares with the others, the blob builder, the shared constants): a traffic
+    figure recorded for other sources is not reported."""
     import hashlib
     h = hashlib.sha256()
     csrc = os.path.join(ROOT, "ternaryllm_amd", "csrc")
-    with open(os.path.join(csrc, "tl_kernels.hip"), "rb") as f:
-        text = f.read()
-    # [re-layout kernel ... end of the device code) and [row launcher ... the small-M workspace helper)
-    marks = ((b"// Activation re-layout for the row-parallel kernel", b"// Host side."),
-             (b"// Bytes of partial sums the row kernel may leave", b"// Runs the re-layout pre-pass into"))
-    for begin, end in marks:
-        i, j = text.find(begin), text.find(end)
-        if i < 0 or j < i:   # the file was reorganised: hash all of it
-            h.update(text)
-            break
-        h.update(text[i:j])
-    for name in ("tl_layout.cpp", "tl_common.h"):
+    for name in ("tl_rows.hip", "tl_device.h", "tl_layout.cpp", "tl_common.h"):
         with open(os.path.join(csrc, name), "rb") as f:
             h.update(f.read())
     return h.hexdigest()[:16]

@@ -38,15 +38,25 @@ def _cpu_flags():
 
 
 def cpu_model():
-    """The full `model name` line of /proc/cpuinfo."""
+    """The `model name` of /proc/cpuinfo with what identifies the part where that name is generic (a virtual machine
+    may report a bare family name): vendor, family, model and stepping numbers."""
+    want = {"vendor_id": None, "model name": None, "cpu family": None, "model": None, "stepping": None}
     try:
         with open("/proc/cpuinfo") as f:
             for line in f:
-                if line.startswith("model name"):
-                    return line.split(":", 1)[1].strip()
+                key, _, value = line.partition(":")
+                key = key.strip()
+                if key in want and want[key] is None:
+                    want[key] = value.strip()
+                if all(v is not None for v in want.values()):
+                    break
     except OSError:
         pass
-    return "unknown"
+    if want["model name"] is None:
+        return "unknown"
+    ids = ", ".join("%s %s" % (label, want[key]) for label, key in (("family", "cpu family"), ("model", "model"), ("stepping", "stepping"))
+                    if want[key] is not None)
+    return "%s (%s%s)" % (want["model name"], (want["vendor_id"] + ", ") if want["vendor_id"] else "", ids)
 
 
 def physical_cores():

@@ -6,7 +6,7 @@ import subprocess
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(PKG_DIR)
 LIB_PATH = os.path.join(PKG_DIR, "libternary_spmm.so")
-SOURCES = ["tl_pack.cpp", "tl_layout.cpp", "tl_kernels.hip", "tl_decode.hip"]
+SOURCES = ["tl_pack.cpp", "tl_layout.cpp", "tl_kernels.hip", "tl_small_m.hip", "tl_rows.hip", "tl_decode.hip"]
 
 
 def hipcc():
