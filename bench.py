@@ -618,7 +618,7 @@ def main():
                 rows = [{"value": round(B2 / r2["seconds"] / 1e9, 3), "unit": "GB/s", "cores": r2["threads"], "kind": r2["kind"], "kernel": r2["kernel"],
                          "us": round(r2["seconds"] * 1e6, 1), "us_min": round(r2["seconds_min"] * 1e6, 1), "us_median": round(r2["seconds_median"] * 1e6, 1),
                          "tokens_per_s": round(1 / r2["seconds"], 1), "max_err_over_max": r2["max_err_over_max"]}
-                        for r2 in cpu_baseline.time_gemv_all(w2.numpy(), torch.randn(4096, generator=g).numpy(), runs=20)]
+                        for r2 in cpu_baseline.time_gemv_all(w2.numpy(), torch.randn(4096, generator=g).numpy(), runs=50)]
                 extra["c2_cpu_baseline"] = rows[0]
                 extra["c2_cpu_baseline"]["also"] = rows[1:]
             except Exception as e:  # noqa: BLE001 - the baseline is optional, the GPU figures are not
