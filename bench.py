@@ -307,9 +307,27 @@ def decode_nodes_leg(model, dev, pos_value):
     pos = torch.full((1,), pos_value, dtype=torch.long, device=dev)
     folds = torch.empty(ops._lib.lib().tl_read_probe_workgroups(), dtype=torch.int32, device=dev)
     qkv_row = ops.spmv_fused(L[0].qkv_proj.device_weight(), "rmsnorm", x, None, L[0].input_layernorm.weight, eps, L[0].qkv_proj.w_scale)
-    att_row = model._attend(qkv_row, model._cache_of(L[0], 0), model._cache_of(L[0], 1), pos, False, splits=1)
+    att_row = model._attend(qkv_row, model._cache_of(L[0], 0), model._cache_of(L[0], 1), pos, False, splits=None if model.split_attention else 1)
     gated_row = ops.spmv_fused(L[0].gate_up_proj.device_weight(), "rmsnorm", x, None, L[0].post_attention_layernorm.weight, eps,
                                L[0].gate_up_proj.w_scale, gated=True)
+    # the step's own launches: with row_chain the o and down products leave the next norm's image and sums of squares,
+    # and the products behind a norm start from those
+    chain = model.row_chain
+    if chain:
+        _, image, squares = ops.spmv_add(L[0].o_proj.device_weight(), att_row, x, L[0].o_proj.w_scale, next_norm_weight=L[0].post_attention_layernorm.weight)
+
+    def behind_norm(m, norm, gated=False):
+        if chain:
+            return ops.spmv_fused(m.device_weight(), "rmsnorm_sums", image, squares, None, eps, m.w_scale, gated=gated)
+        return ops.spmv_fused(m.device_weight(), "rmsnorm", x, None, norm.weight, eps, m.w_scale, gated=gated)
+
+    def ends_block(m, row, next_norm):
+        if chain:
+            return ops.spmv_add(m.device_weight(), row, x, m.w_scale, next_norm_weight=next_norm.weight)
+        return ops.spmv_add(m.device_weight(), row, x, m.w_scale)
+
+    norm_note = "RMSNorm factor from the sums that came with its input" if chain else "RMSNorm on its input"
+    add_note = " + residual + next norm's image and sums" if chain else " + residual"
     kv_bytes = 2 * c.num_attention_heads * (pos_value + 1) * c.head_dim * x.element_size()
     kv_bytes -= kv_bytes % 16
 
@@ -318,19 +336,16 @@ def decode_nodes_leg(model, dev, pos_value):
         return b[:(b.numel() // 16) * 16]
 
     kinds = [
-        ("q|k|v product, RMSNorm on its input", lambda i: ops.spmv_fused(L[i].qkv_proj.device_weight(), "rmsnorm", x, None, L[i].input_layernorm.weight,
-                                                                        eps, L[i].qkv_proj.w_scale),
+        ("q|k|v product, " + norm_note, lambda i: behind_norm(L[i].qkv_proj, L[i].input_layernorm),
          lambda i: ops.stream_read_probe(blob(L[i].qkv_proj), folds), blob(L[0].qkv_proj).numel()),
         ("rotary + cache row + attention over %d rows" % (pos_value + 1),
-         lambda i: model._attend(qkv_row, model._cache_of(L[i], 0), model._cache_of(L[i], 1), pos, False, splits=1),
+         lambda i: model._attend(qkv_row, model._cache_of(L[i], 0), model._cache_of(L[i], 1), pos, False, splits=None if model.split_attention else 1),
          lambda i: ops.stream_read_probe(model._cache[i].reshape(-1).view(torch.uint8)[:kv_bytes], folds), kv_bytes),
-        ("o product + residual", lambda i: ops.spmv_add(L[i].o_proj.device_weight(), att_row, x, L[i].o_proj.w_scale),
+        ("o product" + add_note, lambda i: ends_block(L[i].o_proj, att_row, L[i].post_attention_layernorm),
          lambda i: ops.stream_read_probe(blob(L[i].o_proj), folds), blob(L[0].o_proj).numel()),
-        ("gate|up product, RMSNorm on its input, SiLU gate in its epilogue",
-         lambda i: ops.spmv_fused(L[i].gate_up_proj.device_weight(), "rmsnorm", x, None, L[i].post_attention_layernorm.weight, eps,
-                                  L[i].gate_up_proj.w_scale, gated=True),
+        ("gate|up product, " + norm_note + ", SiLU gate in its epilogue", lambda i: behind_norm(L[i].gate_up_proj, L[i].post_attention_layernorm, gated=True),
          lambda i: ops.stream_read_probe(blob(L[i].gate_up_proj), folds), blob(L[0].gate_up_proj).numel()),
-        ("down product + residual", lambda i: ops.spmv_add(L[i].down_proj.device_weight(), gated_row, x, L[i].down_proj.w_scale),
+        ("down product" + add_note, lambda i: ends_block(L[i].down_proj, gated_row, L[i].input_layernorm),
          lambda i: ops.stream_read_probe(blob(L[i].down_proj), folds), blob(L[0].down_proj).numel()),
     ]
     rows, sum_nodes, sum_floor = [], 0.0, 0.0
@@ -347,14 +362,14 @@ def decode_nodes_leg(model, dev, pos_value):
     def with_head(i):
         if i < n_layers:
             return kinds[0][1](i)
-        return ops.spmv_fused(model.lm_head.device_weight(), "rmsnorm", x, None, model.norm.weight, eps, model.lm_head.w_scale)
+        return behind_norm(model.lm_head, model.norm)
 
     def with_head_probe(i):
         return kinds[0][2](i) if i < n_layers else ops.stream_read_probe(blob(model.lm_head), folds)
 
     t_head = graph_us_per_node(with_head, n_layers + 1, 12, full=True)["median"] * (n_layers + 1) - rows[0]["us"] * 1e-6 * n_layers
     f_head = graph_us_per_node(with_head_probe, n_layers + 1, 12, full=True)["median"] * (n_layers + 1) - rows[0]["read_floor_us"] * 1e-6 * n_layers
-    rows.append({"node": "head product, RMSNorm on its input", "per_step": 1, "bytes": int(blob(model.lm_head).numel()), "us": round(t_head * 1e6, 3),
+    rows.append({"node": "head product, " + norm_note, "per_step": 1, "bytes": int(blob(model.lm_head).numel()), "us": round(t_head * 1e6, 3),
                  "read_floor_us": round(f_head * 1e6, 3), "time_over_read_floor": round(t_head / f_head, 2)})
     sum_nodes += t_head
     sum_floor += f_head

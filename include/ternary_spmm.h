@@ -55,6 +55,7 @@ extern "C" {
 #define TL_PRODUCER_SILU_GATE 1   /* tl_spmv_fused: x = silu(in[:K]) * in[K:]                  */
 #define TL_PRODUCER_ADD_RMSNORM 2 /* tl_spmv_fused: x = RMSNorm(in + in2) * norm_weight        */
 #define TL_PRODUCER_RMSNORM 3     /* tl_spmv_fused: x = RMSNorm(in) * norm_weight, factor applied to the sums */
+#define TL_PRODUCER_RMSNORM_SUMS 4 /* tl_spmv_fused: TL_PRODUCER_RMSNORM on what tl_spmv_add_norm left behind */
 
 #define TL_ACT_NONE 0
 #define TL_ACT_SILU_GATE 1 /* out = silu(gate) * up, for tl_mlp_gate_up */
@@ -333,6 +334,18 @@ int tl_decode_attention_rope(const void* qkv, const void* cos_table, const void*
                              const int64_t* pos_dev, void* out, int64_t out_kmajor_ld,
                              int splits, void* workspace, int64_t workspace_bytes, void* stream);
 
+/* tl_decode_attention_split (q given, qkv NULL) or tl_decode_attention_rope (qkv with its tables given, q NULL) for
+ * 2 to 8 splits without the second launch: each workgroup of a (batch row, head) counts itself in once its piece is
+ * in `workspace`, and the one that finds the others counted folds the pieces into `out` -- no workgroup waits for
+ * another.  arrivals: batch * heads 32-bit counters in device memory, zero before the first call; every call leaves
+ * them zero.  Calls that share `arrivals` or `workspace` must not overlap (work on one stream does not).  The
+ * result equals the two-launch form's bit for bit (same pieces, same fold).  Same reference lines. */
+int tl_decode_attention_fold(const void* q, const void* qkv, const void* cos_table, const void* sin_table,
+                             void* k_cache, void* v_cache, int dtype,
+                             int64_t batch, int heads, int head_dim, int64_t max_seq,
+                             const int64_t* pos_dev, void* out, int64_t out_kmajor_ld,
+                             int splits, void* workspace, int64_t workspace_bytes, uint32_t* arrivals, void* stream);
+
 /* Y[N] = (x * W) * scale for ONE activation row x that the call produces itself, so that a decode step
  * needs neither a launch nor a trip through memory for the producer (the reference leaves these steps to
  * separate torch operators, TernaryLLM/TernaryMLP.py:34 and the Hugging Face decoder layer it patches):
@@ -347,6 +360,11 @@ int tl_decode_attention_rope(const void* qkv, const void* cos_table, const void*
  *                            Equal to TL_PRODUCER_ADD_RMSNORM with in2 == NULL up to that rounding; in2 and
  *                            sum_out must be NULL.  (The residual add belongs to the product BEFORE the norm
  *                            then: tl_spmv_add, tl_spmv_attn_combine_add.)
+ *   TL_PRODUCER_RMSNORM_SUMS the same product, for a row that the product before it prepared (tl_spmv_add_norm):
+ *                            in = its image (row * norm_weight, x_dtype), in2 = its sums of squares, float32, one per
+ *                            16 values of the row (ceil(K / 16) numbers); norm_weight and sum_out must be NULL.  The
+ *                            kernel is then the plain single-row product with one factor at the end.
+ *                            TL_ERR_UNSUPPORTED where a column block's tiles do not fit the LDS of that kernel.
  * in, in2, norm_weight, sum_out are of x_dtype, K values each (2K for the gate | up row), 16-byte aligned.
  * Roundings are those of the separate kernels.  TL_ERR_UNSUPPORTED when K or the blob's tile height is not
  * a whole number of 16-byte pieces (use the separate kernels then). */
@@ -361,6 +379,18 @@ int tl_spmv_fused(const tl_layout_header* header, const void* blob_dev, int prod
  * single-row kernels do not apply (K or the tile height not whole 16-byte pieces). */
 int tl_spmv_add(const tl_layout_header* header, const void* blob_dev, const void* x, int x_dtype, const void* residual,
                 void* Y, int y_dtype, const void* scale, int scale_dtype, void* stream);
+
+/* tl_spmv_add for a row that goes on into an RMSNorm and a product (the post-attention norm and gate | up after the
+ * output projection, the next layer's input norm and q | k | v after the down projection, the final norm and the head:
+ * TernaryLLM/TernaryLlama.py:69-75 and the Hugging Face decoder layer behind it).  Beside Y the epilogue leaves
+ * image_out[n] = Y[n] * next_norm_weight[n] (y_dtype, N values) and squares_out[b] = sum of Y[n]^2 over column block b
+ * (float32, ceil(N / 16) numbers): what tl_spmv_fused with TL_PRODUCER_RMSNORM_SUMS starts from, so that the product
+ * after the norm neither multiplies the row nor sums its squares.  next_norm_weight: N values of y_dtype.  All three
+ * 16-byte aligned; image_out a row of its own.  TL_ERR_UNSUPPORTED where the single-row kernel with this epilogue
+ * does not take the weight (call tl_spmv_add and TL_PRODUCER_RMSNORM then). */
+int tl_spmv_add_norm(const tl_layout_header* header, const void* blob_dev, const void* x, int x_dtype, const void* residual,
+                     void* Y, int y_dtype, const void* scale, int scale_dtype, const void* next_norm_weight,
+                     void* image_out, float* squares_out, void* stream);
 
 /* A decoder layer at 9 to 16 fp16 rows without kernels of its own for the residual add and the RMSNorm (the Hugging
  * Face decoder layer the reference patches, TernaryLLM/TernaryLlama.py:69-75): the products on either side do them.

@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(_DIR, "libternary_spmm.so")
 TL_F32, TL_F16 = 0, 1
 TL_X_ROW_MAJOR, TL_X_K_MAJOR = 0, 1
 TL_ACT_SILU_GATE = 1
-TL_PRODUCER_NONE, TL_PRODUCER_SILU_GATE, TL_PRODUCER_ADD_RMSNORM, TL_PRODUCER_RMSNORM = 0, 1, 2, 3
+TL_PRODUCER_NONE, TL_PRODUCER_SILU_GATE, TL_PRODUCER_ADD_RMSNORM, TL_PRODUCER_RMSNORM, TL_PRODUCER_RMSNORM_SUMS = 0, 1, 2, 3, 4
 TL_LAYOUT_MAGIC = 0x35474C54
 TL_ERR_UNSUPPORTED = -5
 
@@ -89,10 +89,12 @@ SIGNATURES = {
     "tl_rope_cache_update": (_INT, [_VP, _INT, _I64, _INT, _INT, _VP, _VP, _VP, _VP, _VP, _VP, _I64, _VP]),
     "tl_decode_attention": (_INT, [_VP, _VP, _VP, _INT, _I64, _INT, _INT, _I64, _VP, _VP, _I64, _VP]),
     "tl_decode_attention_split": (_INT, [_VP, _VP, _VP, _INT, _I64, _INT, _INT, _I64, _VP, _VP, _I64, _INT, _VP, _I64, _VP]),
+    "tl_decode_attention_fold": (_INT, [_VP, _VP, _VP, _VP, _VP, _VP, _INT, _I64, _INT, _INT, _I64, _VP, _VP, _I64, _INT, _VP, _I64, _VP, _VP]),
     "tl_decode_attention_rope": (_INT, [_VP, _VP, _VP, _VP, _VP, _INT, _I64, _INT, _INT, _I64, _VP, _VP, _I64, _INT, _VP, _I64, _VP]),
     "tl_spmv_attn_combine": (_INT, [_HDRP, _VP, _VP, _INT, _INT, _INT, _VP, _INT, _VP, _INT, _VP]),
     "tl_spmv_attn_combine_add": (_INT, [_HDRP, _VP, _VP, _INT, _INT, _INT, _VP, _VP, _INT, _VP, _INT, _VP]),
     "tl_spmv_add": (_INT, [_HDRP, _VP, _VP, _INT, _VP, _VP, _INT, _VP, _INT, _VP]),
+    "tl_spmv_add_norm": (_INT, [_HDRP, _VP, _VP, _INT, _VP, _VP, _INT, _VP, _INT, _VP, _VP, _VP, _VP]),
     "tl_add_rmsnorm": (_INT, [_VP, _VP, _VP, _INT, _I64, _INT, ctypes.c_float, _VP, _VP, _I64, _VP]),
     "tl_silu_mul": (_INT, [_VP, _INT, _I64, _INT, _VP, _I64, _VP]),
     "tl_silu_mul_pairs": (_INT, [_VP, _INT, _I64, _INT, _VP, _I64, _VP]),

@@ -97,7 +97,8 @@ template <typename T, int HD>
 __global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restrict__ q, const T* __restrict__ k_cache,
                                                                const T* __restrict__ v_cache, const long long* __restrict__ pos_p,
                                                                T* __restrict__ out, long long out_kld, int heads, long long max_seq,
-                                                               float scale, int splits, float* __restrict__ pieces, FreshToken<T> fresh)
+                                                               float scale, int splits, float* __restrict__ pieces,
+                                                               unsigned* __restrict__ arrivals, FreshToken<T> fresh)
 {
     constexpr int VE = 16 / (int)sizeof(T);   // values per 16-byte piece
     constexpr int CPR = HD / VE;              // lanes per cache row
@@ -106,6 +107,7 @@ __global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restri
     static_assert(CPR <= 64 && (CPR & (CPR - 1)) == 0, "a row's lanes must sit in one wave");
     __shared__ float partial[RG][HD + 1];
     __shared__ float group_max[RG], group_sum[RG];
+    __shared__ int last_to_arrive;
     const int tid = threadIdx.x;
     const long long bh = blockIdx.x;
     const long long pos = *pos_p;
@@ -273,15 +275,56 @@ __global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restri
         }
         if (pieces) {
             float* mine = pieces + ((size_t)bh * splits + blockIdx.y) * (HD + 4);
-            mine[tid] = o;  // 0 when the workgroup had no rows (top = -inf, norm = 0)
-            if (tid == 0) {
-                mine[HD] = top;
-                mine[HD + 1] = norm;
+            // (o is 0 when the workgroup had no rows: top = -inf, norm = 0)
+            if (arrivals) {
+                // for another workgroup of this launch to read: stores that go through to memory past this chip
+                // part's own cache, complete before this thread reaches the barrier below
+                __hip_atomic_store(mine + tid, o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (tid == 0) {
+                    __hip_atomic_store(mine + HD, top, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_store(mine + HD + 1, norm, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            } else {
+                mine[tid] = o;
+                if (tid == 0) {
+                    mine[HD] = top;
+                    mine[HD + 1] = norm;
+                }
             }
-            return;
+        } else {
+            const long long b = bh / heads;
+            const size_t col = (size_t)(bh % heads) * HD + tid;  // of the [batch][heads * head_dim] output
+            out[out_kld ? col * out_kld + b : (size_t)b * heads * HD + col] = from_f<T>(o / norm);
+        }
+    }
+    if (!pieces || !arrivals) return;
+    // The workgroups of a (batch row, head) count themselves in once their pieces are out; the one that finds all the
+    // others counted folds the pieces (as tl_attn_combine does) and leaves the counter at zero for the next call.
+    // No workgroup waits for another.  Pieces and counter are written and read by accesses of device scope (they
+    // pass the caches that the parts of the chip do not share), so no cache is written back or emptied for them.
+    __syncthreads();
+    if (tid == 0) {
+        const unsigned before = __hip_atomic_fetch_add(arrivals + bh, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        last_to_arrive = before + 1u == (unsigned)splits;
+        if (last_to_arrive) __hip_atomic_store(arrivals + bh, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!last_to_arrive) return;
+    if (tid < HD) {
+        const float* all = pieces + (size_t)bh * splits * (HD + 4);
+        float top = -INFINITY;
+        for (int s = 0; s < splits; ++s) top = fmaxf(top, __hip_atomic_load(all + (size_t)s * (HD + 4) + HD, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+        float norm = 0.f, o = 0.f;
+        for (int s = 0; s < splits; ++s) {
+            const float* piece = all + (size_t)s * (HD + 4);
+            const float pm = __hip_atomic_load(piece + HD, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const float wgt = pm == -INFINITY ? 0.f : __expf(pm - top);
+            norm = fmaf(__hip_atomic_load(piece + HD + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT), wgt, norm);
+            o = fmaf(__hip_atomic_load(piece + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT), wgt, o);
         }
         const long long b = bh / heads;
-        const size_t col = (size_t)(bh % heads) * HD + tid;  // of the [batch][heads * head_dim] output
+        const size_t col = (size_t)(bh % heads) * HD + tid;
         out[out_kld ? col * out_kld + b : (size_t)b * heads * HD + col] = from_f<T>(o / norm);
     }
 }
@@ -474,14 +517,14 @@ struct FreshArgs {
 
 template <typename T, int HD>
 int attn_launch(dim3 grid, size_t lds, hipStream_t st, const void* q, const void* k, const void* v, const long long* pos, void* out,
-                long long out_kld, int heads, long long max_seq, float scale, int splits, float* partial, const FreshArgs& f)
+                long long out_kld, int heads, long long max_seq, float scale, int splits, float* partial, unsigned* arrivals, const FreshArgs& f)
 {
     auto kernel = tl_decode_attn<T, HD>;
     FreshToken<T> fresh{static_cast<const T*>(f.qkv), static_cast<const T*>(f.cos_table), static_cast<const T*>(f.sin_table),
                         f.qkv ? static_cast<T*>(const_cast<void*>(k)) : nullptr, f.qkv ? static_cast<T*>(const_cast<void*>(v)) : nullptr};
     hipLaunchKernelGGL(kernel, dim3(grid.x, (unsigned)splits), dim3(kAttnThreads), lds, st, static_cast<const T*>(q), static_cast<const T*>(k),
-                       static_cast<const T*>(v), pos, static_cast<T*>(out), out_kld, heads, max_seq, scale, splits, partial, fresh);
-    if (partial && out) {
+                       static_cast<const T*>(v), pos, static_cast<T*>(out), out_kld, heads, max_seq, scale, splits, partial, arrivals, fresh);
+    if (partial && out && !arrivals) {
         auto combine = tl_attn_combine<T, HD>;
         hipLaunchKernelGGL(combine, grid, dim3(HD), 0, st, partial, splits, static_cast<T*>(out), out_kld, heads);
     }
@@ -491,12 +534,12 @@ int attn_launch(dim3 grid, size_t lds, hipStream_t st, const void* q, const void
 template <typename T>
 int attn_dispatch(int head_dim, dim3 grid, size_t lds, hipStream_t st, const void* q, const void* k, const void* v,
                   const long long* pos, void* out, long long out_kld, int heads, long long max_seq, float scale, int splits, float* partial,
-                  const FreshArgs& f)
+                  unsigned* arrivals, const FreshArgs& f)
 {
     switch (head_dim) {
-        case 64: return attn_launch<T, 64>(grid, lds, st, q, k, v, pos, out, out_kld, heads, max_seq, scale, splits, partial, f);
-        case 128: return attn_launch<T, 128>(grid, lds, st, q, k, v, pos, out, out_kld, heads, max_seq, scale, splits, partial, f);
-        case 256: return attn_launch<T, 256>(grid, lds, st, q, k, v, pos, out, out_kld, heads, max_seq, scale, splits, partial, f);
+        case 64: return attn_launch<T, 64>(grid, lds, st, q, k, v, pos, out, out_kld, heads, max_seq, scale, splits, partial, arrivals, f);
+        case 128: return attn_launch<T, 128>(grid, lds, st, q, k, v, pos, out, out_kld, heads, max_seq, scale, splits, partial, arrivals, f);
+        case 256: return attn_launch<T, 256>(grid, lds, st, q, k, v, pos, out, out_kld, heads, max_seq, scale, splits, partial, arrivals, f);
         default: return fail(TL_ERR_UNSUPPORTED, "head_dim=%d (64, 128 or 256 supported)", head_dim);
     }
 }
@@ -532,7 +575,7 @@ constexpr int kAttnMaxSplits = 8;
 
 int attention(const void* q, const FreshArgs& fresh, const void* k_cache, const void* v_cache, int dtype, int64_t batch, int heads, int head_dim,
               int64_t max_seq, const int64_t* pos_dev, void* out, int64_t out_kmajor_ld, int splits, void* workspace, int64_t workspace_bytes,
-              void* stream)
+              void* stream, uint32_t* arrivals = nullptr)
 {
     if (int rc = check_common(dtype, batch, heads, head_dim, max_seq, pos_dev)) return rc;
     if (!(q || fresh.qkv) || !k_cache || !v_cache || (!out && !workspace)) return fail(TL_ERR_ARG, "device pointer is null");
@@ -555,11 +598,13 @@ int attention(const void* q, const FreshArgs& fresh, const void* k_cache, const 
     const long long* pos = reinterpret_cast<const long long*>(pos_dev);
     const float scale = 1.0f / sqrtf((float)head_dim);
     float* partial = leaves_pieces ? static_cast<float*>(workspace) : nullptr;
+    if (arrivals && (!out || splits < 2 || reinterpret_cast<uintptr_t>(arrivals) % 4))
+        return fail(TL_ERR_ARG, "the fold inside the kernel is for 2 or more splits, an output and 4-byte aligned counters");
     int rc;
     if (dtype == TL_F16) rc = attn_dispatch<__half>(head_dim, grid, lds, st, q, k_cache, v_cache, pos, out, (long long)out_kmajor_ld, heads,
-                                                    (long long)max_seq, scale, splits, partial, fresh);
+                                                    (long long)max_seq, scale, splits, partial, arrivals, fresh);
     else rc = attn_dispatch<float>(head_dim, grid, lds, st, q, k_cache, v_cache, pos, out, (long long)out_kmajor_ld, heads, (long long)max_seq,
-                                   scale, splits, partial, fresh);
+                                   scale, splits, partial, arrivals, fresh);
     if (rc) return rc;
     return launched();
 }
@@ -655,4 +700,15 @@ extern "C" int tl_silu_mul(const void* gate_up, int dtype, int64_t rows, int wid
 extern "C" int tl_silu_mul_pairs(const void* gate_up, int dtype, int64_t rows, int width, void* out, int64_t out_kmajor_ld, void* stream)
 {
     return silu_mul_call(gate_up, dtype, rows, width, out, out_kmajor_ld, stream, 1);
+}
+
+extern "C" int tl_decode_attention_fold(const void* q, const void* qkv, const void* cos_table, const void* sin_table, void* k_cache, void* v_cache,
+                                        int dtype, int64_t batch, int heads, int head_dim, int64_t max_seq, const int64_t* pos_dev, void* out,
+                                        int64_t out_kmajor_ld, int splits, void* workspace, int64_t workspace_bytes, uint32_t* arrivals,
+                                        void* stream)
+{
+    if (!arrivals) return fail(TL_ERR_ARG, "arrivals is null");
+    if ((q != nullptr) == (qkv != nullptr)) return fail(TL_ERR_ARG, "give q, or qkv with the rotary tables");
+    return attention(q, FreshArgs{qkv, qkv ? cos_table : nullptr, qkv ? sin_table : nullptr}, k_cache, v_cache, dtype, batch, heads, head_dim, max_seq,
+                     pos_dev, out, out_kmajor_ld, splits, workspace, workspace_bytes, stream, arrivals);
 }

@@ -1265,6 +1265,7 @@ __global__ __launch_bounds__(kResWaves * 64) void tl_spmm_res(KernelArgs a)
 // are rounded to the activation type.
 constexpr int kProNone = 0, kProSiluGate = 1, kProAddNorm = 2, kProAttnCombine = 3;
 constexpr int kProNormDeferred = 4;  // launcher only: RMSNorm whose factor multiplies the sums (tl_spmv_tiles), else kProAddNorm
+constexpr int kProNormSums = 5;      // launcher only: the row comes multiplied by the norm weight, its squares summed in pieces (tl_spmv_tiles alone)
 
 template <bool F16>
 __device__ __forceinline__ float round_to_x(float v)
@@ -1514,6 +1515,10 @@ __global__ __launch_bounds__(NT) void tl_spmv_direct(KernelArgs a)
 // for by count, so the chunks stay in flight), the waves add up in[k]^2 on the side, and rsqrt(mean + eps), one
 // number for the whole row, multiplies the column sums at the very end -- no wave waits for another before it
 // gathers.  (The row is thus rounded to the activation type as in * norm_w, not as in * factor * norm_w.)
+// NORM == 2 is the same product with the two steps in front of the gather taken away: the row arrives already
+// multiplied by the norm weight, with the sums of squares of its values in pieces beside it -- what the product
+// that made the row leaves in its epilogue (chain_w below) -- so this kernel is the plain one plus a factor at the
+// end, with one set of images and as many workgroups to a compute unit as the plain one.
 
 // Waits until at most `later` of this wave's vector-memory instructions are outstanding (they complete in
 // order): everything issued before the last `later` has then arrived.  Counts above 13 wait for a few more.
@@ -1539,7 +1544,9 @@ __device__ __forceinline__ void tiles_wait_vm(int later)
 
 constexpr int kTilesMaxOwn = 8;  // tiles a wave of tl_spmv_tiles may own
 
-template <bool XF16, int NT, bool NORM = false>
+constexpr int kNormNone = 0, kNormInside = 1, kNormSums = 2;
+
+template <bool XF16, int NT, int NORM = kNormNone>
 __global__ __launch_bounds__(NT) void tl_spmv_tiles(KernelArgs a)
 {
     extern __shared__ __align__(16) unsigned char lds[];
@@ -1562,7 +1569,17 @@ __global__ __launch_bounds__(NT) void tl_spmv_tiles(KernelArgs a)
     using lds_ptr = __attribute__((address_space(3))) void*;
     const uint32_t base = cs[0];
 
-    if constexpr (NORM) {
+    float squares = 0.f;  // this lane's share of sum(in^2): of the row itself (kNormInside), of the sums that came with it (kNormSums)
+    if constexpr (NORM == kNormSums) {
+        // One number per 16 values of the row, shared out over the threads: loads issued ahead of every load that
+        // is waited for by count, their values first used after the last tile (no wave waits for them here).
+        const int blocks = a.chain_sq_blocks;
+        const float s0 = tid < blocks ? a.chain_sq_in[tid] : 0.f;
+        const float s1 = tid + NT < blocks ? a.chain_sq_in[tid + NT] : 0.f;
+        squares = s0 + s1;
+        for (int i = tid + 2 * NT; i < blocks; i += NT) squares += a.chain_sq_in[i];  // (K above 16 * 2 * NT)
+    }
+    if constexpr (NORM == kNormInside) {
         // the row and the norm weight of this wave's tiles, ahead of every chunk
 #pragma unroll
         for (int j = 0; j < kMaxOwn; ++j) {
@@ -1594,7 +1611,7 @@ __global__ __launch_bounds__(NT) void tl_spmv_tiles(KernelArgs a)
             // slot among them) is zeroed
             const int rows_here = min(a.tile_rows, a.K - t * a.tile_rows);
             unsigned char* image = xs + (size_t)t * PITCH * ES;
-            if constexpr (!NORM) {
+            if constexpr (NORM != kNormInside) {
                 if (lane * VE < rows_here)
                     __builtin_amdgcn_global_load_lds((global_ptr)(Xb + ((size_t)t * a.tile_rows + (size_t)lane * VE) * ES), (lds_ptr)image, 16, 0, 0);
                 ++loads[j];
@@ -1603,8 +1620,7 @@ __global__ __launch_bounds__(NT) void tl_spmv_tiles(KernelArgs a)
         }
     }
 
-    float squares = 0.f;  // NORM: this lane's share of sum(in^2)
-    if constexpr (NORM) {
+    if constexpr (NORM == kNormInside) {
         int chunk_loads = 0;
 #pragma unroll
         for (int j = 0; j < kMaxOwn; ++j) chunk_loads += loads[j];
@@ -1649,7 +1665,7 @@ __global__ __launch_bounds__(NT) void tl_spmv_tiles(KernelArgs a)
     acc[0] += __shfl_xor(acc[0], 1, 64);
     acc[0] += __shfl_xor(acc[0], 2, 64);
     if (lw == 0) red[wave * TL_BLOCK_COLUMNS + c16] = acc[0];
-    if constexpr (NORM) {
+    if constexpr (NORM != kNormNone) {
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) squares += __shfl_xor(squares, off, 64);
         if (lane == 0) red[W * TL_BLOCK_COLUMNS + wave] = squares;
@@ -1659,7 +1675,7 @@ __global__ __launch_bounds__(NT) void tl_spmv_tiles(KernelArgs a)
         float sum = 0.f;
 #pragma unroll
         for (int w = 0; w < W; ++w) sum += red[w * TL_BLOCK_COLUMNS + tid];
-        if constexpr (NORM) {
+        if constexpr (NORM != kNormNone) {
             float total = 0.f;
 #pragma unroll
             for (int w = 0; w < W; ++w) total += red[W * TL_BLOCK_COLUMNS + w];
@@ -1670,6 +1686,24 @@ __global__ __launch_bounds__(NT) void tl_spmv_tiles(KernelArgs a)
             const float y = n < a.N ? as_output(sum * load_scale(a.w0.scale, a.scale_f16, n), a.y_f16) : 0.f;
             const float up = __shfl_xor(y, 1, 64);  // the odd neighbour's
             if (!(tid & 1) && n + 1 < a.N) store_out(a.Y, a.y_f16, n / 2, gate_pair(y, up, a.y_f16));
+            return;
+        }
+        if (a.chain_w) {
+            // The row goes on into an RMSNorm and a product: leave it multiplied by that norm's weight (rounded as the
+            // norm inside the next kernel would round it) and the block's share of the sum of its squares beside the
+            // row itself, so that the next product starts as a plain one (kNormSums).
+            float y = 0.f;
+            if (n < a.N) {
+                float v = sum * load_scale(a.w0.scale, a.scale_f16, n);
+                if (a.residual) v = as_output(v, a.y_f16) + load_scale(a.residual, a.y_f16, n);
+                y = as_output(v, a.y_f16);
+                store_out(a.Y, a.y_f16, n, v);
+                store_out(a.chain_image, a.y_f16, n, y * load_scale(a.chain_w, a.y_f16, n));
+            }
+            float q = y * y;
+#pragma unroll
+            for (int off = 1; off < TL_BLOCK_COLUMNS; off <<= 1) q += __shfl_xor(q, off, 64);
+            if (tid == 0) a.chain_sq_out[nb] = q;
             return;
         }
         if (n < a.N) store_result(a, n, sum * load_scale(a.w0.scale, a.scale_f16, n));
@@ -1927,7 +1961,7 @@ int launch_spmv_direct_nt(KernelArgs a, const tl_layout_header* h, hipStream_t s
 
 // tl_spmv_tiles: every tile of the block resident (a wave loads its own and waits for nobody else's).
 // Returns TL_ERR_UNSUPPORTED when that does not fit; the caller then takes tl_spmv_direct.
-template <bool XF16, int NT, bool NORM = false>
+template <bool XF16, int NT, int NORM = kNormNone>
 int launch_spmv_tiles_nt(KernelArgs a, const tl_layout_header* h, hipStream_t st)
 {
     constexpr int es = XF16 ? 2 : 4;
@@ -1936,9 +1970,9 @@ int launch_spmv_tiles_nt(KernelArgs a, const tl_layout_header* h, hipStream_t st
     if (a.T > (NT / 64) * kTilesMaxOwn) return TL_ERR_UNSUPPORTED;
     a.xs_bytes = a.T * tile_bytes;
     a.buf_bytes = (int)round_up((int64_t)a.T * chunk_bytes, 16);
-    const size_t lds = (size_t)a.xs_bytes * (NORM ? 2 : 1) + a.buf_bytes + (size_t)(((NT / 64) * (TL_BLOCK_COLUMNS + 1) + 3) & ~3) * 4;
+    const size_t lds = (size_t)a.xs_bytes * (NORM == kNormInside ? 2 : 1) + a.buf_bytes + (size_t)(((NT / 64) * (TL_BLOCK_COLUMNS + 1) + 3) & ~3) * 4;
     int share = std::max(1, std::min(knob(TL_SPMV_SHARE, 4), (int)ceil_div(a.NB, compute_units())));
-    if (NORM) share = std::min(share, 3);  // the second set of images: three workgroups of K = 4096 fit a compute unit, not four
+    if (NORM == kNormInside) share = std::min(share, 3);  // the second set of images: three workgroups of K = 4096 fit a compute unit, not four
     if (lds > (size_t)(160 * 1024 / share - 1024)) return TL_ERR_UNSUPPORTED;
     auto kernel = tl_spmv_tiles<XF16, NT, NORM>;
     static bool raised = false;  // per instantiation; a repeated or racing call is harmless
@@ -1956,19 +1990,24 @@ template <bool XF16, int PRO = kProNone>
 int launch_spmv_direct(const KernelArgs& a, const tl_layout_header* h, hipStream_t st)
 {
     const bool wide = knob(TL_SPMV_WIDE, a.NB <= compute_units() ? 1 : 0) != 0;
-    if constexpr (PRO == kProNormDeferred) {
+    if constexpr (PRO == kProNormSums) {
+        const int rc = wide ? launch_spmv_tiles_nt<XF16, 1024, kNormSums>(a, h, st) : launch_spmv_tiles_nt<XF16, kBlockThreads, kNormSums>(a, h, st);
+        if (rc == TL_ERR_UNSUPPORTED) return fail(TL_ERR_UNSUPPORTED, "the weight's blocks do not fit the kernel that takes a row with its sums of squares");
+        return rc;
+    } else if constexpr (PRO == kProNormDeferred) {
         if (knob(TL_SPMV_TILES, 1) != 0) {
-            const int rc = wide ? launch_spmv_tiles_nt<XF16, 1024, true>(a, h, st) : launch_spmv_tiles_nt<XF16, kBlockThreads, true>(a, h, st);
+            const int rc = wide ? launch_spmv_tiles_nt<XF16, 1024, kNormInside>(a, h, st) : launch_spmv_tiles_nt<XF16, kBlockThreads, kNormInside>(a, h, st);
             if (rc != TL_ERR_UNSUPPORTED) return rc;
         }
         return wide ? launch_spmv_direct_nt<XF16, 1024, kProAddNorm>(a, h, st) : launch_spmv_direct_nt<XF16, kBlockThreads, kProAddNorm>(a, h, st);
     } else {
         if constexpr (PRO == kProNone) {
             // the tile-per-wave kernel where the block fits it; with the other producers it is the slower of the two
-            if (knob(TL_SPMV_TILES, 1) != 0) {
+            if (knob(TL_SPMV_TILES, 1) != 0 || a.chain_w) {
                 const int rc = wide ? launch_spmv_tiles_nt<XF16, 1024>(a, h, st) : launch_spmv_tiles_nt<XF16, kBlockThreads>(a, h, st);
                 if (rc != TL_ERR_UNSUPPORTED) return rc;
             }
+            if (a.chain_w) return fail(TL_ERR_UNSUPPORTED, "the weight's blocks do not fit the kernel that leaves the row for the next norm");
         }
         return wide ? launch_spmv_direct_nt<XF16, 1024, PRO>(a, h, st) : launch_spmv_direct_nt<XF16, kBlockThreads, PRO>(a, h, st);
     }
@@ -2099,7 +2138,8 @@ int small_launch(KernelArgs a, const tl_layout_header* h, int x_dtype, void* wor
 namespace {
 int spmv_fused_call(const tl_layout_header* header, const void* blob_dev, int producer,
                     const void* in, const void* in2, const void* norm_weight, float eps, void* sum_out, int x_dtype,
-                    void* Y, int y_dtype, const void* scale, int scale_dtype, void* stream, bool gated, const void* residual = nullptr)
+                    void* Y, int y_dtype, const void* scale, int scale_dtype, void* stream, bool gated, const void* residual = nullptr,
+                    const void* next_norm_weight = nullptr, void* image_out = nullptr, float* squares_out = nullptr)
 {
     if (int rc = check_header(header)) return rc;
     if (gated && header->columns % 2) return fail(TL_ERR_SHAPE, "N=%u: gate and up columns come in pairs", header->columns);
@@ -2107,14 +2147,25 @@ int spmv_fused_call(const tl_layout_header* header, const void* blob_dev, int pr
     if (int rc = check_dtype(y_dtype, "y")) return rc;
     if (scale)
         if (int rc = check_dtype(scale_dtype, "scale")) return rc;
-    if (producer != TL_PRODUCER_NONE && producer != TL_PRODUCER_SILU_GATE && producer != TL_PRODUCER_ADD_RMSNORM && producer != TL_PRODUCER_RMSNORM)
+    if (producer != TL_PRODUCER_NONE && producer != TL_PRODUCER_SILU_GATE && producer != TL_PRODUCER_ADD_RMSNORM && producer != TL_PRODUCER_RMSNORM &&
+        producer != TL_PRODUCER_RMSNORM_SUMS)
         return fail(TL_ERR_ARG, "producer code %d unknown", producer);
     if (residual && gated) return fail(TL_ERR_ARG, "a gated product has no residual row of its width");
     if (reinterpret_cast<uintptr_t>(residual) % (y_dtype == TL_F16 ? 2 : 4)) return fail(TL_ERR_ALIGN, "residual is not aligned to its type");
     if (!blob_dev || !in || !Y) return fail(TL_ERR_ARG, "device pointer is null");
     if (reinterpret_cast<uintptr_t>(blob_dev) % 256) return fail(TL_ERR_ALIGN, "weight blob must be 256-byte aligned");
     if ((producer == TL_PRODUCER_ADD_RMSNORM || producer == TL_PRODUCER_RMSNORM) && !norm_weight) return fail(TL_ERR_ARG, "norm_weight is null");
-    if (producer != TL_PRODUCER_ADD_RMSNORM && (in2 || sum_out)) return fail(TL_ERR_ARG, "in2 and sum_out belong to TL_PRODUCER_ADD_RMSNORM");
+    if (producer == TL_PRODUCER_RMSNORM_SUMS) {
+        if (!in2 || norm_weight || sum_out) return fail(TL_ERR_ARG, "TL_PRODUCER_RMSNORM_SUMS takes the sums of squares in in2, and neither norm_weight nor sum_out");
+    } else if (producer != TL_PRODUCER_ADD_RMSNORM && (in2 || sum_out)) {
+        return fail(TL_ERR_ARG, "in2 and sum_out belong to TL_PRODUCER_ADD_RMSNORM");
+    }
+    if (next_norm_weight) {
+        if (!image_out || !squares_out) return fail(TL_ERR_ARG, "image_out or squares_out is null");
+        if (image_out == Y || image_out == in || image_out == residual) return fail(TL_ERR_ARG, "image_out must be a row of its own");
+        for (const void* p : {next_norm_weight, static_cast<const void*>(image_out), static_cast<const void*>(squares_out)})
+            if (reinterpret_cast<uintptr_t>(p) % 16) return fail(TL_ERR_ALIGN, "next_norm_weight, image_out and squares_out must be 16-byte aligned");
+    }
     if (sum_out && (sum_out == in || sum_out == in2)) return fail(TL_ERR_ARG, "sum_out must not be one of the inputs: other workgroups still read them");
     const int es = x_dtype == TL_F16 ? 2 : 4, ve = 16 / es;
     // what the direct-load kernel needs of a row: whole aligned 16-byte pieces per tile
@@ -2134,11 +2185,17 @@ int spmv_fused_call(const tl_layout_header* header, const void* blob_dev, int pr
     a.one = 1.0f;
     a.gated = gated;
     a.residual = residual;
+    a.chain_w = next_norm_weight; a.chain_image = image_out; a.chain_sq_out = squares_out;
     hipStream_t st = static_cast<hipStream_t>(stream);
     int rc;
     if (producer == TL_PRODUCER_NONE)
         rc = a.x_f16 ? launch_spmv_direct<true>(a, header, st) : launch_spmv_direct<false>(a, header, st);
-    else if (producer == TL_PRODUCER_RMSNORM)
+    else if (producer == TL_PRODUCER_RMSNORM_SUMS) {
+        a.X2 = nullptr;
+        a.chain_sq_in = static_cast<const float*>(in2);
+        a.chain_sq_blocks = (int)ceil_div(header->inners, TL_BLOCK_COLUMNS);
+        rc = a.x_f16 ? launch_spmv_direct<true, kProNormSums>(a, header, st) : launch_spmv_direct<false, kProNormSums>(a, header, st);
+    } else if (producer == TL_PRODUCER_RMSNORM)
         rc = a.x_f16 ? launch_spmv_direct<true, kProNormDeferred>(a, header, st) : launch_spmv_direct<false, kProNormDeferred>(a, header, st);
     else if (producer == TL_PRODUCER_SILU_GATE)
         rc = a.x_f16 ? launch_spmv_direct<true, kProSiluGate>(a, header, st) : launch_spmv_direct<false, kProSiluGate>(a, header, st);
@@ -2162,6 +2219,16 @@ extern "C" int tl_spmv_add(const tl_layout_header* header, const void* blob_dev,
     if (!residual) return fail(TL_ERR_ARG, "residual is null");
     return spmv_fused_call(header, blob_dev, TL_PRODUCER_NONE, x, nullptr, nullptr, 0.f, nullptr, x_dtype, Y, y_dtype, scale, scale_dtype, stream, false,
                            residual);
+}
+
+extern "C" int tl_spmv_add_norm(const tl_layout_header* header, const void* blob_dev, const void* x, int x_dtype, const void* residual,
+                                void* Y, int y_dtype, const void* scale, int scale_dtype, const void* next_norm_weight,
+                                void* image_out, float* squares_out, void* stream)
+{
+    if (!residual) return fail(TL_ERR_ARG, "residual is null");
+    if (!next_norm_weight) return fail(TL_ERR_ARG, "next_norm_weight is null");
+    return spmv_fused_call(header, blob_dev, TL_PRODUCER_NONE, x, nullptr, nullptr, 0.f, nullptr, x_dtype, Y, y_dtype, scale, scale_dtype, stream, false,
+                           residual, next_norm_weight, image_out, squares_out);
 }
 
 extern "C" int tl_spmv_fused_gated(const tl_layout_header* header, const void* blob_dev, int producer,

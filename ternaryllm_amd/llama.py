@@ -128,13 +128,16 @@ class TernaryLlamaDecoder(nn.Module):
             self.lm_head._header.tile_rows % 8 == 0 and H % 8 == 0
         # the attention kernel rotates q and k and writes the token's cache row itself; False runs the separate kernel first
         self.fused_rope = True
-        # single-row steps: share the cache rows of a head out among several workgroups and fold the pieces inside the
-        # output projection.  That pays once a head's rows are many: up to about a thousand rows one workgroup per
-        # head and a plain output projection (the faster single-row kernel) are quicker together.
+        # single-row steps: share the cache rows of a head out among several workgroups, the last of which to finish
+        # folds their pieces.  That pays once a head's rows are many: up to about a thousand rows one workgroup per
+        # head is as quick.
         self.split_attention = self.max_seq_len > 1024
         # steps of 9 to 16 fp16 rows: the products do the residual adds and the RMSNorms around them (tl_spmm_chain);
         # switched off by the first step whose shapes have no such kernel
         self.chain_decode = dtype == torch.float16
+        # single-row steps: the o and down projections prepare the row for the norm behind them (spmv_add with
+        # next_norm_weight); switched off by the first step whose shapes have no such kernel
+        self.row_chain = True
         self._layer_index = {id(layer): i for i, layer in enumerate(self.layers)}
 
     # -- pieces ------------------------------------------------------------------------------
@@ -223,6 +226,13 @@ class TernaryLlamaDecoder(nn.Module):
         # 5 to 48 rows: the products read a K-major image, so whatever feeds one writes it in that layout
         # (its transpose as a view) and no re-layout pass runs in front of the products
         if B == 1 and self.fused_decode:
+            if self.row_chain:
+                try:
+                    return self._decode_step_fused(x, pos)
+                except RuntimeError as e:
+                    if "TL_ERR_UNSUPPORTED" not in str(e) or torch.cuda.is_current_stream_capturing():
+                        raise
+                    self.row_chain = False
             return self._decode_step_fused(x, pos)
         km = 5 <= B <= 48 and c.hidden_size != B and c.intermediate_size != B
         if km and 9 <= B <= 16 and self.chain_decode:
@@ -274,25 +284,45 @@ class TernaryLlamaDecoder(nn.Module):
         normalise their input themselves (RMSNorm with the factor applied to the sums, tl_spmv_fused "rmsnorm"); the
         gate|up product applies the SiLU gate in its epilogue (columns packed as gate/up pairs); the attention rotates
         q and k and writes the cache row; with a long cache (split_attention) it shares the cache rows of a head out
-        among several workgroups (32 heads alone leave seven compute units in eight idle) and leaves its result in
-        pieces that the output projection folds while it stages its row (tl_spmv_attn_combine); the o and down
-        projections add their result to the residual stream in their epilogue."""
+        among several workgroups (32 heads alone leave seven compute units in eight idle), the last of which folds
+        their pieces (tl_decode_attention_fold); the o and down projections add their result to the residual stream
+        in their epilogue."""
         eps = self.config.rms_norm_eps
-        hd, dtype = self.config.head_dim, x.dtype
         # x is the residual stream: every product that ends a block adds its result to it in the epilogue, and the
-        # products that start one normalise it on the way in (the factor applied to their sums)
-        for layer in self.layers:
-            qkv = ops.spmv_fused(layer.qkv_proj.device_weight(), "rmsnorm", x, None, layer.input_layernorm.weight, eps, layer.qkv_proj.w_scale)
-            if self.split_attention:
-                pieces = self._attend(qkv, self._cache_of(layer, 0), self._cache_of(layer, 1), pos, False, pieces=True)
-                x = ops.spmv_attn_combine(layer.o_proj.device_weight(), pieces, hd, dtype, layer.o_proj.w_scale, residual=x)
+        # products that start one normalise it on the way in (the factor applied to their sums).  With row_chain the
+        # product that ends a block also leaves the row multiplied by the next norm's weight and the sums of its
+        # squares (spmv_add(..., next_norm_weight=)), and the product after the norm is the plain kernel with one
+        # factor at the end ("rmsnorm_sums"): it keeps one image of the row in LDS, not two.
+        chain = self.row_chain
+        image = squares = None
+        for li, layer in enumerate(self.layers):
+            if squares is None:
+                qkv = ops.spmv_fused(layer.qkv_proj.device_weight(), "rmsnorm", x, None, layer.input_layernorm.weight, eps, layer.qkv_proj.w_scale)
             else:
-                att = self._attend(qkv, self._cache_of(layer, 0), self._cache_of(layer, 1), pos, False, splits=1)
+                qkv = ops.spmv_fused(layer.qkv_proj.device_weight(), "rmsnorm_sums", image, squares, None, eps, layer.qkv_proj.w_scale)
+            squares = None
+            # a long cache: the rows of a head shared out among several workgroups, the last of which folds their pieces
+            att = self._attend(qkv, self._cache_of(layer, 0), self._cache_of(layer, 1), pos, False, splits=None if self.split_attention else 1)
+            if chain:
+                x, image, squares = ops.spmv_add(layer.o_proj.device_weight(), att, x, layer.o_proj.w_scale,
+                                                 next_norm_weight=layer.post_attention_layernorm.weight)
+            else:
                 x = ops.spmv_add(layer.o_proj.device_weight(), att, x, layer.o_proj.w_scale)
-            gated = ops.spmv_fused(layer.gate_up_proj.device_weight(), "rmsnorm", x, None, layer.post_attention_layernorm.weight, eps,
-                                   layer.gate_up_proj.w_scale, gated=True)
-            x = ops.spmv_add(layer.down_proj.device_weight(), gated, x, layer.down_proj.w_scale)
-        return ops.spmv_fused(self.lm_head.device_weight(), "rmsnorm", x, None, self.norm.weight, eps, self.lm_head.w_scale)
+            if squares is None:
+                gated = ops.spmv_fused(layer.gate_up_proj.device_weight(), "rmsnorm", x, None, layer.post_attention_layernorm.weight, eps,
+                                       layer.gate_up_proj.w_scale, gated=True)
+            else:
+                gated = ops.spmv_fused(layer.gate_up_proj.device_weight(), "rmsnorm_sums", image, squares, None, eps,
+                                       layer.gate_up_proj.w_scale, gated=True)
+            squares = None
+            if chain:
+                nxt = self.layers[li + 1].input_layernorm.weight if li + 1 < len(self.layers) else self.norm.weight
+                x, image, squares = ops.spmv_add(layer.down_proj.device_weight(), gated, x, layer.down_proj.w_scale, next_norm_weight=nxt)
+            else:
+                x = ops.spmv_add(layer.down_proj.device_weight(), gated, x, layer.down_proj.w_scale)
+        if squares is None:
+            return ops.spmv_fused(self.lm_head.device_weight(), "rmsnorm", x, None, self.norm.weight, eps, self.lm_head.w_scale)
+        return ops.spmv_fused(self.lm_head.device_weight(), "rmsnorm_sums", image, squares, None, eps, self.lm_head.w_scale)
 
     def _attend(self, qkv, k_cache, v_cache, pos, kmajor, pieces=False, splits=None):
         """Rotary embedding, cache update and attention for the token whose q | k | v the projection just wrote: one

@@ -271,7 +271,9 @@ def spmv_fused(weight, producer, inp, inp2=None, norm_weight=None, eps=0.0, scal
     producer "add_rmsnorm": s = inp + inp2 (inp2 may be None), x = rmsnorm(s) * norm_weight; with want_sum the
     call also returns s (a new tensor);
     producer "rmsnorm": x = rmsnorm(inp) * norm_weight with the normalisation factor applied to the column sums (the
-    row multiplied is inp * norm_weight in inp's dtype; no part of the kernel waits for the mean).
+    row multiplied is inp * norm_weight in inp's dtype; no part of the kernel waits for the mean);
+    producer "rmsnorm_sums": the same product for a row that spmv_add(..., next_norm_weight=) left behind: inp is its
+    image (row * norm weight), inp2 its float32 sums of squares, one per 16 values; norm_weight stays None.
     Returns y, or (y, s).  Raises RuntimeError (TL_ERR_UNSUPPORTED) where the
     fused kernel does not apply (K or the tile height not whole 16-byte pieces); callers then use the separate operators.
     gated: the weight's columns are (gate, up) pairs and y is [1, N / 2] with y[j] = silu(y'[2j]) * y'[2j + 1]
@@ -279,16 +281,22 @@ def spmv_fused(weight, producer, inp, inp2=None, norm_weight=None, eps=0.0, scal
     K, N = weight.inners, weight.columns
     if gated and N % 2:
         raise ValueError("gate and up columns come in pairs: N must be even")
-    code = {"silu_gate": _lib.TL_PRODUCER_SILU_GATE, "add_rmsnorm": _lib.TL_PRODUCER_ADD_RMSNORM, "rmsnorm": _lib.TL_PRODUCER_RMSNORM}[producer]
+    code = {"silu_gate": _lib.TL_PRODUCER_SILU_GATE, "add_rmsnorm": _lib.TL_PRODUCER_ADD_RMSNORM, "rmsnorm": _lib.TL_PRODUCER_RMSNORM,
+            "rmsnorm_sums": _lib.TL_PRODUCER_RMSNORM_SUMS}[producer]
+    if producer == "rmsnorm_sums":
+        if norm_weight is not None or want_sum:
+            raise ValueError("the image already holds the norm weight, and the sum is the row that came with it")
+        if inp2 is None or inp2.dtype != torch.float32 or inp2.numel() != (K + 15) // 16 or not inp2.is_contiguous() or inp2.device != weight.device:
+            raise ValueError("inp2 must hold one float32 sum of squares per 16 values of the row")
     if producer == "rmsnorm" and (inp2 is not None or want_sum):
         raise ValueError("the rmsnorm producer has no second summand: the residual add belongs to the product before it (spmv_add)")
     x_code = _code(inp.dtype, "inp")
     need = 2 * K if producer == "silu_gate" else K
-    tensors = [inp] + [t for t in (inp2, norm_weight) if t is not None]
+    tensors = [inp] + [t for t in (inp2 if producer != "rmsnorm_sums" else None, norm_weight) if t is not None]
     for t in tensors:
         if t.numel() != (need if t is inp else K) or not t.is_contiguous() or t.dtype != inp.dtype or t.device != weight.device:
             raise ValueError("inputs must be contiguous rows of the weight's K (2K for a gate | up row), one dtype, on the weight's device")
-    if producer != "silu_gate" and norm_weight is None:
+    if producer in ("add_rmsnorm", "rmsnorm") and norm_weight is None:
         raise ValueError(f"{producer} needs norm_weight")
     out_dtype = out_dtype or inp.dtype
     y = torch.empty((1, N // 2 if gated else N), dtype=out_dtype, device=inp.device)
@@ -305,10 +313,14 @@ def spmv_fused(weight, producer, inp, inp2=None, norm_weight=None, eps=0.0, scal
     return (y, s_out) if want_sum else y
 
 
-def spmv_add(weight, x, residual, scale=None):
+def spmv_add(weight, x, residual, scale=None, next_norm_weight=None):
     """residual + (x @ W) * scale for one contiguous row x [1, K] or [K] and a residual row of N values (tl_spmv_add):
     the residual add of a decoder layer in the epilogue of the product in front of it, rounded as the separate add of
-    the stored product would round.  Returns a new [1, N] tensor of residual's dtype."""
+    the stored product would round.  Returns a new [1, N] tensor of residual's dtype.
+    next_norm_weight [N]: the weight of the RMSNorm the new row goes into (tl_spmv_add_norm).  Returns (y, image,
+    squares) then: image = y * next_norm_weight in y's dtype and squares [ceil(N / 16)] float32, the sums of y^2 over
+    runs of 16 values -- the inputs of spmv_fused(..., "rmsnorm_sums", image, squares).  Raises RuntimeError
+    (TL_ERR_UNSUPPORTED) where the weight's shape leaves the product to a kernel without that epilogue."""
     K, N = weight.inners, weight.columns
     if x.numel() != K or residual.numel() != N or not x.is_contiguous() or not residual.is_contiguous():
         raise ValueError("x must be a contiguous row of K values and residual one of N")
@@ -316,6 +328,19 @@ def spmv_add(weight, x, residual, scale=None):
         raise RuntimeError("x and residual must be on the weight's device")
     y = torch.empty((1, N), dtype=residual.dtype, device=x.device)
     scale, s_code = _scale_args(scale, N, x.device)
+    if next_norm_weight is not None:
+        if next_norm_weight.numel() != N or next_norm_weight.dtype != residual.dtype or not next_norm_weight.is_contiguous() or \
+                next_norm_weight.device != weight.device:
+            raise ValueError("next_norm_weight must be a contiguous row of N values of the residual's dtype on the weight's device")
+        image = torch.empty((1, N), dtype=residual.dtype, device=x.device)
+        squares = torch.empty((N + 15) // 16, dtype=torch.float32, device=x.device)
+        with torch.cuda.device(x.device):
+            rc = _lib.lib().tl_spmv_add_norm(ctypes.byref(weight.header), weight.blob.data_ptr(), x.data_ptr(), _code(x.dtype, "x"),
+                                             residual.data_ptr(), y.data_ptr(), _code(residual.dtype, "residual"),
+                                             scale.data_ptr() if scale is not None else None, s_code, next_norm_weight.data_ptr(),
+                                             image.data_ptr(), squares.data_ptr(), _stream_ptr(x.device))
+        _lib.check(rc)
+        return y, image, squares
     with torch.cuda.device(x.device):
         rc = _lib.lib().tl_spmv_add(ctypes.byref(weight.header), weight.blob.data_ptr(), x.data_ptr(), _code(x.dtype, "x"), residual.data_ptr(),
                                     y.data_ptr(), _code(residual.dtype, "residual"), scale.data_ptr() if scale is not None else None, s_code,
@@ -417,6 +442,7 @@ def _kmajor_image(rows, width, like):
 
 
 _attn_workspaces = {}
+_attn_arrivals = {}
 _ATTN_MAX_SPLITS = 8
 
 
@@ -441,11 +467,17 @@ def _check_fresh(fresh, k_cache):
     return qkv, cos_table, sin_table
 
 
-def _attention_call(q, fresh, k_cache, v_cache, pos, out_ptr, ld, splits, ws_ptr, ws_bytes):
+def _attention_call(q, fresh, k_cache, v_cache, pos, out_ptr, ld, splits, ws_ptr, ws_bytes, arrivals_ptr=None):
     B, heads, max_seq, hd = k_cache.shape
     L = _lib.lib()
     with torch.cuda.device(k_cache.device):
-        if fresh is None:
+        if arrivals_ptr is not None:
+            qkv, cos_table, sin_table = fresh if fresh is not None else (None, None, None)
+            rc = L.tl_decode_attention_fold(q.data_ptr() if fresh is None else None, qkv.data_ptr() if qkv is not None else None,
+                                            cos_table.data_ptr() if qkv is not None else None, sin_table.data_ptr() if qkv is not None else None,
+                                            k_cache.data_ptr(), v_cache.data_ptr(), _code(k_cache.dtype, "cache"), B, heads, hd, max_seq,
+                                            pos.data_ptr(), out_ptr, ld, splits, ws_ptr, ws_bytes, arrivals_ptr, _stream_ptr(k_cache.device))
+        elif fresh is None:
             rc = L.tl_decode_attention_split(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), _code(q.dtype, "q"), B, heads, hd,
                                              max_seq, pos.data_ptr(), out_ptr, ld, splits, ws_ptr, ws_bytes, _stream_ptr(q.device))
         else:
@@ -456,12 +488,13 @@ def _attention_call(q, fresh, k_cache, v_cache, pos, out_ptr, ld, splits, ws_ptr
     _lib.check(rc)
 
 
-def decode_attention(q, k_cache, v_cache, pos, out=None, kmajor=False, splits=None, fresh=None):
+def decode_attention(q, k_cache, v_cache, pos, out=None, kmajor=False, splits=None, fresh=None, fold_inside=True):
     """Attention of one query per (batch row, head) over cache rows [0, pos].  q: [B, heads, head_dim];
     caches: [B, heads, max_seq, head_dim]; pos: one-element int64 device tensor.  Returns [B, heads * head_dim],
     or with kmajor its transpose [heads * head_dim, B] as a view of a K-major image (for spmm's x_layout=1).
     splits: workgroups that share the cache rows of a (batch row, head) (1 to 8; default: by the size of
-    the step, see _attention_splits).
+    the step, see _attention_splits).  Their pieces are folded by the last of them to finish (tl_decode_attention_fold),
+    or with fold_inside=False by a second launch (tl_decode_attention_split, tl_decode_attention_rope).
     fresh=(qkv, cos_table, sin_table) with q=None: the same kernel also does what rope_cache_update does --
     rotates q and k of the token and writes its k, v into cache row `pos` -- in the one launch."""
     B, heads, max_seq, hd = k_cache.shape
@@ -487,7 +520,7 @@ def decode_attention(q, k_cache, v_cache, pos, out=None, kmajor=False, splits=No
         raise ValueError("pos must be a one-element int64 tensor on the same device")
     if splits is None:
         splits = _attention_splits(B, heads, q.device)
-    ws_ptr, ws_bytes = None, 0
+    ws_ptr, ws_bytes, arrivals_ptr = None, 0, None
     if splits > 1:
         # scratch for the pieces: one buffer per (device, stream), like the products' (work on a stream is ordered)
         key = (q.device.index, torch.cuda.current_stream(q.device).cuda_stream)
@@ -497,7 +530,14 @@ def decode_attention(q, k_cache, v_cache, pos, out=None, kmajor=False, splits=No
             ws = torch.empty(need, dtype=torch.uint8, device=q.device)
             _attn_workspaces[key] = ws
         ws_ptr, ws_bytes = ws.data_ptr(), ws.numel()
-    _attention_call(None if fresh is not None else q, fresh, k_cache, v_cache, pos, out.data_ptr(), ld, splits, ws_ptr, ws_bytes)
+        if fold_inside:
+            # one counter per (batch row, head): zero between calls (the kernel leaves them so)
+            counters = _attn_arrivals.get(key)
+            if counters is None or counters.numel() < B * heads:
+                counters = torch.zeros(B * heads, dtype=torch.int32, device=q.device)
+                _attn_arrivals[key] = counters
+            arrivals_ptr = counters.data_ptr()
+    _attention_call(None if fresh is not None else q, fresh, k_cache, v_cache, pos, out.data_ptr(), ld, splits, ws_ptr, ws_bytes, arrivals_ptr)
     return out[:, :B] if kmajor else out
 
 

@@ -320,6 +320,10 @@ def test_split_attention_and_its_fold_inside_the_output_projection(cuda, oracle)
                     assert (out.double() - single.double()).abs().max().item() <= tol * max(1.0, ref.abs().max().item())
                     outk = ops.decode_attention(q, kc, vc, p, kmajor=True, splits=splits)
                     assert torch.equal(outk.t(), out)
+                    # the pieces folded by the last workgroup to finish (the default) and by a launch of their own;
+                    # the counters of the first form are left at zero: a call with another number of pieces follows at once
+                    assert torch.equal(out, ops.decode_attention(q, kc, vc, p, splits=splits, fold_inside=False)), (pos, splits)
+                assert all(int(c.abs().max()) == 0 for c in ops._attn_arrivals.values())
         # the output projection with the fold inside, batch 1
         H, hd, S, N = 32, 128, 700, 272
         K = H * hd
@@ -382,6 +386,8 @@ def test_attention_that_rotates_and_updates_the_cache_itself(cuda):
                     kc3, vc3 = kc0.clone(), vc0.clone()
                     assert torch.equal(ops.decode_attention(None, kc3, vc3, p, kmajor=True, splits=splits, fresh=(qkv, cos, sin)).t(), fused)
                     assert torch.equal(kc3, kc2)
+                    kc5, vc5 = kc0.clone(), vc0.clone()
+                    assert torch.equal(ops.decode_attention(None, kc5, vc5, p, splits=splits, fresh=(qkv, cos, sin), fold_inside=False), fused)
                     if pos < S:
                         kc4, vc4 = kc0.clone(), vc0.clone()
                         pieces = ops.decode_attention_pieces(None, kc4, vc4, p, splits=splits, fresh=(qkv, cos, sin))
@@ -473,6 +479,57 @@ def test_fused_producers_of_the_single_row_product(cuda, oracle, dtype, tol):
     with pytest.raises(RuntimeError, match="UNSUPPORTED"):   # a tile height that is not whole 16-byte pieces: the separate kernels are the way then
         odd = ops.DeviceWeight(PackedWeight.from_dense(ternary_weight(1000, 40, 0.7, 3), tile_rows=250), cuda)
         ops.spmv_fused(odd, "silu_gate", torch.zeros(2000, dtype=dtype, device=cuda))
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float16, 2e-3), (torch.float32, 1e-5)])
+def test_single_row_product_prepares_the_next_norm(cuda, dtype, tol):
+    """tl_spmv_add_norm and TL_PRODUCER_RMSNORM_SUMS: the product that ends a block leaves, beside the new residual
+    row, that row times the next norm's weight and the sums of its squares over runs of 16; the product behind the
+    norm starts from those.  The row bit for bit against tl_spmv_add, the image against the rounded product of row
+    and weight, the sums and the second product against float64 and against TL_PRODUCER_RMSNORM on the row."""
+    from tests.util import knobs, max_rel_err, ternary_weight
+    from ternaryllm_amd import ops
+    from ternaryllm_amd.packing import PackedWeight
+    g = torch.Generator().manual_seed(77)
+    eps = 1e-5
+    for K1, N1, N2 in ((4096, 1024, 272), (1000, 1000, 40), (11008, 4096, 96)):   # whole blocks; a ragged last block and tile; many tiles
+        w1, w2 = ternary_weight(K1, N1, 0.7, K1 + N1), ternary_weight(N1, N2, 0.66, N1 + N2)
+        d1, d2 = (ops.DeviceWeight(PackedWeight.from_dense(w), cuda) for w in (w1, w2))
+        s1 = (0.01 + 0.01 * torch.rand(N1, generator=g)).to(dtype).to(cuda)
+        s2 = (0.5 + torch.rand(N2, generator=g)).to(dtype).to(cuda)
+        act = torch.randn((1, K1), generator=g).to(dtype).to(cuda)
+        res = torch.randn(N1, generator=g).to(dtype).to(cuda)
+        nw = (1 + 0.1 * torch.randn(N1, generator=g)).to(dtype).to(cuda)
+        for setting in ({}, {"TL_SPMV_WIDE": "1"}) if K1 == 11008 else ({}, {"TL_SPMV_WIDE": "0"}):
+            with knobs(**setting):
+                y, image, squares = ops.spmv_add(d1, act, res, s1, next_norm_weight=nw)
+                assert torch.equal(y, ops.spmv_add(d1, act, res, s1)), (K1, N1, setting)
+                assert torch.equal(image, (y.float() * nw.float()[None]).to(dtype)) if dtype == torch.float16 else torch.equal(image, y * nw[None])
+                blocks = (N1 + 15) // 16
+                padded = torch.zeros(blocks * 16, dtype=torch.float64, device=cuda)
+                padded[:N1] = y[0].double()
+                want = padded.view(blocks, 16).pow(2).sum(1)
+                assert squares.shape == (blocks,) and (squares.double() - want).abs().max().item() <= 1e-6 * want.max().item()
+                h64 = y[0].double() * torch.rsqrt(y[0].double().pow(2).mean() + eps) * nw.double()
+                ref = (h64.cpu().numpy()[None, :] @ w2.astype("float64")) * s2.double().cpu().numpy()[None, :]
+                out = ops.spmv_fused(d2, "rmsnorm_sums", image, squares, None, eps, s2)
+                assert max_rel_err(out.double().cpu().numpy(), ref, h64.cpu().numpy()[None, :], w2) <= 2 * tol, (K1, N1, N2, setting)
+                other = ops.spmv_fused(d2, "rmsnorm", y, None, nw, eps, s2)
+                assert max_rel_err(out.double().cpu().numpy(), other.double().cpu().numpy(), h64.cpu().numpy()[None, :], w2) <= tol
+                assert torch.equal(ops.spmv_fused(d2, "rmsnorm_sums", image, squares, None, eps, s2, gated=True), ops.silu_mul(out, pairs=True))
+        with pytest.raises(ValueError, match="one float32 sum"):
+            ops.spmv_fused(d2, "rmsnorm_sums", image, squares[:-1].contiguous(), None, eps, s2)
+        with pytest.raises(ValueError, match="already holds"):
+            ops.spmv_fused(d2, "rmsnorm_sums", image, squares, nw, eps, s2)
+    # 86 tiles are more than the eight waves of the tile-per-wave kernel own at 512 threads, and the other kernel has no such epilogue
+    low = ops.DeviceWeight(PackedWeight.from_dense(ternary_weight(4096, 64, 0.7, 3), tile_rows=48), cuda)
+    act, res, nw = (torch.ones(n, dtype=dtype, device=cuda) for n in (4096, 64, 64))
+    with knobs(TL_SPMV_WIDE="0"):
+        assert torch.equal(ops.spmv_add(low, act, res), ops.spmm(low, act[None]) + res[None])
+        with pytest.raises(RuntimeError, match="UNSUPPORTED"):
+            ops.spmv_add(low, act, res, next_norm_weight=nw)
+        with pytest.raises(RuntimeError, match="UNSUPPORTED"):
+            ops.spmv_fused(low, "rmsnorm_sums", act, torch.ones(256, dtype=torch.float32, device=cuda), None, eps)
 
 
 def test_silu_gate_in_the_epilogue_of_the_gate_up_product(cuda):
@@ -578,9 +635,11 @@ def test_fused_single_row_step_equals_the_unfused_one(tiny, cuda):
     assert tiny.fused_decode
     outs = {}
     assert not tiny.split_attention   # a short cache: one workgroup per head; the split form is forced below
-    for fused in (False, True, "split"):
+    assert tiny.row_chain
+    for fused in (False, True, "split", "plain"):   # "plain": the products behind a norm multiply the row and sum its squares themselves
         tiny.fused_decode = bool(fused)
         tiny.split_attention = fused == "split"
+        tiny.row_chain = fused != "plain"
         tiny._graph = None
         tiny.prefill(tokens[:, :28])
         st = tiny._decode_state(1)
@@ -591,11 +650,14 @@ def test_fused_single_row_step_equals_the_unfused_one(tiny, cuda):
             st["mask"].copy_((torch.arange(tiny.max_seq_len, device=cuda) <= 28 + j)[None, None, None])
             logits.append(tiny._decode_step(st["token"], st["pos"], st["mask"]).float())
         outs[fused] = torch.stack(logits)
+        assert tiny.row_chain == (fused != "plain")   # no step fell back
     tiny.fused_decode = True
     tiny.split_attention = False
+    tiny.row_chain = True
     tiny._state = None
     tiny._graph = None
     assert (outs[True] - outs[False]).abs().max().item() <= 2e-3 * outs[False].abs().max().item()
+    assert (outs["plain"] - outs[False]).abs().max().item() <= 2e-3 * outs[False].abs().max().item()
     assert (outs["split"] - outs[False]).abs().max().item() <= 2e-3 * outs[False].abs().max().item()
     eager = tiny.generate(tokens, 10, use_graph=False)
     graphed = tiny.generate(tokens, 10, use_graph=True)
