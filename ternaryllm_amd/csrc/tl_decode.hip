@@ -76,7 +76,15 @@ __global__ __launch_bounds__(256) void tl_rope_cache(const T* __restrict__ qkv, 
 // when the maximum moves), so nothing waits for memory a second time; the RG running results are
 // combined through LDS at the end.
 constexpr int kAttnThreads = 1024;
-constexpr int kAttnBatch = 4;  // rows of a row group whose loads are in flight together
+constexpr int kAttnBatch = 5;  // rows of a row group whose loads are in flight together
+
+
+// The value another lane of the same row of 16 holds, by a data-parallel-primitive code
+template <int CTRL>
+__device__ __forceinline__ float lane_permuted(float v)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
 
 //
 // With `fresh` (q|k|v of the token as the projection wrote them, [batch][3][heads][HD], plus the rotary tables)
@@ -106,7 +114,10 @@ __global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restri
     constexpr int NB = kAttnBatch;
     static_assert(CPR <= 64 && (CPR & (CPR - 1)) == 0, "a row's lanes must sit in one wave");
     __shared__ float partial[RG][HD + 1];
+    constexpr int SG = kAttnThreads / HD;     // threads that share the fold of one output value
+    static_assert(RG % SG == 0, "the row groups are dealt out evenly to the threads of an output value");
     __shared__ float group_max[RG], group_sum[RG];
+    __shared__ float fold_o[SG][HD], fold_norm[SG], fold_top;
     __shared__ int last_to_arrive;
     const int tid = threadIdx.x;
     const long long bh = blockIdx.x;
@@ -142,22 +153,29 @@ __global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restri
     };
 
     // A row group's rows come NB at a time; the first batch is asked for before q is ready.  (Asking for the next
-    // batch before the current one is worked on, two register sets alternating, was slower: 128 registers.)
-    auto load_batch = [&](long long j0, uint4 (&kk)[NB], uint4 (&vv)[NB]) {
+    // batch before the current one is worked on, two register sets alternating, was no faster at 3 rows per batch
+    // and slower at 4, where it needs more than the 128 registers a thread of 1024 may have.)
+    // Every slot of a batch is loaded, without a branch: a slot past the group's last row takes the batch's first row
+    // again (its score is masked below, so it adds exactly nothing), and the cache row the token will take is loaded
+    // like any other and replaced by the token's own key and value before use.  Row numbers and offsets are 32-bit
+    // (the launcher holds a head's cache under 2 GiB).
+    const int n_rows = (int)n, fresh_row = has_fresh ? (int)pos : -1;
+    auto row_of = [&](int j0, int u) {
+        const int j = j0 + u * RG;
+        return j < n_rows ? j : j0;
+    };
+    auto load_batch = [&](int j0, uint4 (&kk)[NB], uint4 (&vv)[NB]) {
 #pragma unroll
         for (int u = 0; u < NB; ++u) {
-            const long long j = j0 + (long long)u * RG;
-            kk[u] = vv[u] = make_uint4(0u, 0u, 0u, 0u);
-            if (j < n && !(has_fresh && j == pos)) {  // rows past the end are not fetched, nor the row the token will take
-                kk[u] = *reinterpret_cast<const uint4*>(kc + (size_t)j * HD + c * VE);
-                vv[u] = *reinterpret_cast<const uint4*>(vc + (size_t)j * HD + c * VE);
-            }
+            const uint32_t off = (uint32_t)row_of(j0, u) * HD + c * VE;
+            kk[u] = *reinterpret_cast<const uint4*>(kc + off);
+            vv[u] = *reinterpret_cast<const uint4*>(vc + off);
         }
     };
     uint4 ka[NB], va[NB];
-    const long long step = (long long)RG * NB;
-    long long j0 = lo + rg;
-    if (j0 < n) load_batch(j0, ka, va);
+    constexpr int step = RG * NB;
+    int j0 = (int)lo + rg;
+    if (j0 < n_rows) load_batch(j0, ka, va);
 
     float qv[VE];
     uint4 k_new = make_uint4(0u, 0u, 0u, 0u), v_new = make_uint4(0u, 0u, 0u, 0u);  // this lane's piece of the token's key and value
@@ -196,11 +214,11 @@ __global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restri
     float acc[VE];
 #pragma unroll
     for (int e = 0; e < VE; ++e) acc[e] = 0.f;
-    auto work = [&](long long j0, uint4 (&kk)[NB], uint4 (&vv)[NB]) {
+    auto work = [&](int j0, uint4 (&kk)[NB], uint4 (&vv)[NB]) {
         if (has_fresh) {
 #pragma unroll
             for (int u = 0; u < NB; ++u)
-                if (j0 + (long long)u * RG == pos && pos < n) {  // the token itself: not in the cache yet
+                if (row_of(j0, u) == fresh_row) {  // the token itself: not in the cache yet
                     kk[u] = k_new;
                     vv[u] = v_new;
                 }
@@ -214,19 +232,29 @@ __global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restri
 #pragma unroll
             for (int e = 0; e < VE; ++e) sc[u] = fmaf(f[e], qv[e], sc[u]);
         }
-        // the CPR lanes of a row add up their shares, the NB rows side by side: their exchanges do not wait for each other
+        // The CPR lanes of a row add up their shares, the NB rows side by side: their exchanges do not wait for each
+        // other.  Inside 16 lanes the partner's value comes through the vector unit's own lane permutations
+        // (mirror of 16, mirror of 8, pairs two apart, neighbours: every lane ends with the same total, as the sums of
+        // both partners of a step are the same two numbers added); only wider steps go through the LDS crossbar.
 #pragma unroll
-        for (int off = CPR / 2; off > 0; off >>= 1) {
+        for (int off = CPR / 2; off >= 16; off >>= 1) {
             float other[NB];
 #pragma unroll
             for (int u = 0; u < NB; ++u) other[u] = __shfl_xor(sc[u], off, 64);
 #pragma unroll
             for (int u = 0; u < NB; ++u) sc[u] += other[u];
         }
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            if constexpr (CPR >= 16) sc[u] += lane_permuted<0x140>(sc[u]);  // lane i of 16 <- lane 15 - i
+            if constexpr (CPR >= 8) sc[u] += lane_permuted<0x141>(sc[u]);   // lane i of 8 <- lane 7 - i
+            if constexpr (CPR >= 4) sc[u] += lane_permuted<0x4E>(sc[u]);    // lanes [2, 3, 0, 1] of every four
+            if constexpr (CPR >= 2) sc[u] += lane_permuted<0xB1>(sc[u]);    // lanes [1, 0, 3, 2] of every four
+        }
         float top = m;
 #pragma unroll
         for (int u = 0; u < NB; ++u) {
-            if (j0 + (long long)u * RG >= n) sc[u] = -INFINITY;
+            if (j0 + u * RG >= n_rows) sc[u] = -INFINITY;
             top = fmaxf(top, sc[u]);
         }
         const float keep = __expf(m - top);  // m == -inf on the first turn: exp(-inf) = 0, and l, acc are 0
@@ -244,9 +272,9 @@ __global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restri
         }
         m = top;
     };
-    if (j0 < n) {
+    if (j0 < n_rows) {
         work(j0, ka, va);
-        for (j0 += step; j0 < n; j0 += step) {
+        for (j0 += step; j0 < n_rows; j0 += step) {
             load_batch(j0, ka, va);
             work(j0, ka, va);
         }
@@ -262,16 +290,35 @@ __global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restri
         group_sum[rg] = l;
     }
     __syncthreads();
-    if (tid < HD) {
+    {
+        // The row groups' results are folded by all threads: SG threads per output value take RG / SG row groups each.
         float top = -INFINITY;
-#pragma unroll 8
-        for (int g = 0; g < RG; ++g) top = fmaxf(top, group_max[g]);
+        for (int g = tid & 63; g < RG; g += 64) top = fmaxf(top, group_max[g]);
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) top = fmaxf(top, __shfl_xor(top, off, 64));
+        const int d = tid % HD, sg = tid / HD;
         float norm = 0.f, o = 0.f;
-#pragma unroll 4
-        for (int g = 0; g < RG; ++g) {
+#pragma unroll
+        for (int i = 0; i < RG / SG; ++i) {
+            const int g = sg * (RG / SG) + i;
             const float wgt = group_max[g] == -INFINITY ? 0.f : __expf(group_max[g] - top);
             norm = fmaf(group_sum[g], wgt, norm);
-            o = fmaf(partial[g][tid], wgt, o);
+            o = fmaf(partial[g][d], wgt, o);
+        }
+        fold_o[sg][d] = o;
+        if (d == 0) {
+            fold_norm[sg] = norm;
+            if (sg == 0) fold_top = top;
+        }
+    }
+    __syncthreads();
+    if (tid < HD) {
+        const float top = fold_top;
+        float norm = 0.f, o = 0.f;
+#pragma unroll
+        for (int sg = 0; sg < SG; ++sg) {
+            norm += fold_norm[sg];
+            o += fold_o[sg][tid];
         }
         if (pieces) {
             float* mine = pieces + ((size_t)bh * splits + blockIdx.y) * (HD + 4);
@@ -584,6 +631,7 @@ int attention(const void* q, const FreshArgs& fresh, const void* k_cache, const 
     const size_t lds = 0;
     if (reinterpret_cast<uintptr_t>(k_cache) % 16 || reinterpret_cast<uintptr_t>(v_cache) % 16 || reinterpret_cast<uintptr_t>(q) % 16)
         return fail(TL_ERR_ALIGN, "q and the caches must be 16-byte aligned");
+    if (max_seq * head_dim * (dtype == TL_F16 ? 2 : 4) >= (1ll << 31)) return fail(TL_ERR_UNSUPPORTED, "a head's cache of %lld rows is 2 GiB or more", (long long)max_seq);
     if (reinterpret_cast<uintptr_t>(fresh.qkv) % 16 || reinterpret_cast<uintptr_t>(fresh.cos_table) % 16 || reinterpret_cast<uintptr_t>(fresh.sin_table) % 16)
         return fail(TL_ERR_ALIGN, "qkv and the rotary tables must be 16-byte aligned");
     if (splits < 1 || splits > kAttnMaxSplits) return fail(TL_ERR_ARG, "splits=%d (1 to %d expected)", splits, kAttnMaxSplits);
