@@ -443,6 +443,15 @@ int tl_spmv_attn_combine_add(const tl_layout_header* header, const void* blob_de
                              int splits, int head_dim, int x_dtype, const void* residual, void* Y, int y_dtype,
                              const void* scale, int scale_dtype, void* stream);
 
+/* The end of a greedy decode step in one launch: token[b] = argmax of logits[b][0 .. vocab) (the first of equal
+ * values; a NaN counts as larger than any number -- torch.argmax's rule), then, when pos_dev is not NULL,
+ * *pos_dev = min(*pos_dev + 1, max_pos) and, when mask is not NULL too, mask[*pos_dev] = 1 (one byte per cache slot).
+ * It stands for the argmax, copy, add, clamp and index_fill launches with which the reference's generation loop
+ * (Hugging Face generate() behind TernaryLLM/TernaryLlama.py) ends a step.  logits: [batch][vocab] of `dtype`,
+ * contiguous; token: int64 [batch]. */
+int tl_greedy_advance(const void* logits, int dtype, int64_t batch, int vocab, int64_t* token, int64_t* pos_dev,
+                      int64_t max_pos, void* mask, void* stream);
+
 /* x_out = x + y, h_out = RMSNorm(x_out) * weight, row by row ([rows][width], one dtype): the residual
  * add of a decoder layer fused with the normalisation that follows (the reference leaves both to the
  * Hugging Face Llama it patches, TernaryLLM/TernaryLlama.py:69-75).  y may be NULL: plain RMSNorm of x,

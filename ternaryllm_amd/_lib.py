@@ -89,6 +89,7 @@ SIGNATURES = {
     "tl_rope_cache_update": (_INT, [_VP, _INT, _I64, _INT, _INT, _VP, _VP, _VP, _VP, _VP, _VP, _I64, _VP]),
     "tl_decode_attention": (_INT, [_VP, _VP, _VP, _INT, _I64, _INT, _INT, _I64, _VP, _VP, _I64, _VP]),
     "tl_decode_attention_split": (_INT, [_VP, _VP, _VP, _INT, _I64, _INT, _INT, _I64, _VP, _VP, _I64, _INT, _VP, _I64, _VP]),
+    "tl_greedy_advance": (_INT, [_VP, _INT, _I64, _INT, _VP, _VP, _I64, _VP, _VP]),
     "tl_decode_attention_fold": (_INT, [_VP, _VP, _VP, _VP, _VP, _VP, _INT, _I64, _INT, _INT, _I64, _VP, _VP, _I64, _INT, _VP, _I64, _VP, _VP]),
     "tl_decode_attention_rope": (_INT, [_VP, _VP, _VP, _VP, _VP, _INT, _I64, _INT, _INT, _I64, _VP, _VP, _I64, _INT, _VP, _I64, _VP]),
     "tl_spmv_attn_combine": (_INT, [_HDRP, _VP, _VP, _INT, _INT, _INT, _VP, _INT, _VP, _INT, _VP]),

@@ -525,6 +525,62 @@ __global__ __launch_bounds__(256) void tl_silu_mul_k(const T* __restrict__ gu, T
     out[i] = from_f<T>(to_f(from_f<T>(g / (1.0f + __expf(-g)))) * u);  // the SiLU is rounded to T before the product, as two separate operators would
 }
 
+// The end of a greedy decode step as one launch: token[b] = index of the largest of row b's logits (the first of equal
+// ones, a NaN counted as larger than any number, as torch.argmax has it); the first workgroup then moves the position
+// on by one, held at max_pos, and marks it in the mask of valid cache slots when there is one.
+template <typename T>
+__global__ __launch_bounds__(1024) void tl_greedy_advance_k(const T* __restrict__ logits, int vocab, long long* __restrict__ token,
+                                                            long long* __restrict__ pos, long long max_pos, unsigned char* __restrict__ mask)
+{
+    __shared__ float best_v[16];
+    __shared__ int best_i[16];
+    const T* row = logits + (size_t)blockIdx.x * vocab;
+    const int tid = threadIdx.x;
+    float bv = 0.f;
+    int bi = -1;
+    auto better = [](float v, int i, float w, int j) {  // (v, i) before (w, j)?
+        if (j < 0) return true;
+        const bool vn = v != v, wn = w != w;
+        if (vn || wn) return vn && (!wn || i < j);
+        return v > w || (v == w && i < j);
+    };
+    for (int i = tid; i < vocab; i += 1024) {
+        const float v = to_f(row[i]);
+        if (better(v, i, bv, bi)) {
+            bv = v;
+            bi = i;
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(bv, off, 64);
+        const int oi = __shfl_xor(bi, off, 64);
+        if (oi >= 0 && better(ov, oi, bv, bi)) {
+            bv = ov;
+            bi = oi;
+        }
+    }
+    if ((tid & 63) == 0) {
+        best_v[tid >> 6] = bv;
+        best_i[tid >> 6] = bi;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        for (int w = 1; w < 16; ++w)
+            if (best_i[w] >= 0 && better(best_v[w], best_i[w], bv, bi)) {
+                bv = best_v[w];
+                bi = best_i[w];
+            }
+        token[blockIdx.x] = bi;
+        if (blockIdx.x == 0 && pos) {
+            long long p = *pos + 1;
+            if (p > max_pos) p = max_pos;
+            *pos = p;
+            if (mask && p >= 0) mask[p] = 1;
+        }
+    }
+}
+
 int check_common(int dtype, int64_t batch, int heads, int head_dim, int64_t max_seq, const void* pos_dev)
 {
     if (dtype != TL_F16 && dtype != TL_F32) return fail(TL_ERR_DTYPE, "dtype code %d unknown", dtype);
@@ -759,4 +815,24 @@ extern "C" int tl_decode_attention_fold(const void* q, const void* qkv, const vo
     if ((q != nullptr) == (qkv != nullptr)) return fail(TL_ERR_ARG, "give q, or qkv with the rotary tables");
     return attention(q, FreshArgs{qkv, qkv ? cos_table : nullptr, qkv ? sin_table : nullptr}, k_cache, v_cache, dtype, batch, heads, head_dim, max_seq,
                      pos_dev, out, out_kmajor_ld, splits, workspace, workspace_bytes, stream, arrivals);
+}
+
+extern "C" int tl_greedy_advance(const void* logits, int dtype, int64_t batch, int vocab, int64_t* token, int64_t* pos_dev, int64_t max_pos,
+                                 void* mask, void* stream)
+{
+    if (dtype != TL_F16 && dtype != TL_F32) return fail(TL_ERR_DTYPE, "dtype code %d unknown", dtype);
+    if (!logits || !token) return fail(TL_ERR_ARG, "device pointer is null");
+    if (batch <= 0 || batch > INT32_MAX || vocab <= 0) return fail(TL_ERR_SHAPE, "batch and vocab must be positive");
+    if (reinterpret_cast<uintptr_t>(token) % 8 || reinterpret_cast<uintptr_t>(pos_dev) % 8) return fail(TL_ERR_ALIGN, "token and pos must be 8-byte aligned");
+    if (pos_dev && max_pos < 0) return fail(TL_ERR_ARG, "max_pos=%lld is negative", (long long)max_pos);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    long long* tok = reinterpret_cast<long long*>(token);
+    long long* pos = reinterpret_cast<long long*>(pos_dev);
+    if (dtype == TL_F16)
+        hipLaunchKernelGGL(tl_greedy_advance_k<__half>, dim3((unsigned)batch), dim3(1024), 0, st, static_cast<const __half*>(logits), vocab, tok, pos,
+                           (long long)max_pos, static_cast<unsigned char*>(mask));
+    else
+        hipLaunchKernelGGL(tl_greedy_advance_k<float>, dim3((unsigned)batch), dim3(1024), 0, st, static_cast<const float*>(logits), vocab, tok, pos,
+                           (long long)max_pos, static_cast<unsigned char*>(mask));
+    return launched();
 }

@@ -374,9 +374,13 @@ class TernaryLlamaDecoder(nn.Module):
     def _advance(self, st):
         logits = self._decode_step(st["token"], st["pos"], st["mask"])
         self.last_logits = logits  # (under a captured graph: the tensor every replay writes)
-        st["token"].copy_(logits.argmax(-1))
         # positions stay inside the cache even if a caller steps past its end (the results are then
         # meaningless, but nothing is written out of bounds; generate() checks the length up front)
+        if logits.is_cuda and logits.dtype in (torch.float16, torch.float32) and logits.is_contiguous():
+            # argmax, the new position and its mask bit in one launch
+            ops.greedy_advance(logits, st["token"], st["pos"], self.max_seq_len - 1, st["mask"])
+            return
+        st["token"].copy_(logits.argmax(-1))
         st["pos"].add_(1).clamp_(max=self.max_seq_len - 1)
         st["mask"].index_fill_(3, st["pos"], True)
 

@@ -565,6 +565,27 @@ def decode_attention_pieces(q, k_cache, v_cache, pos, splits=None, fresh=None):
     return pieces
 
 
+def greedy_advance(logits, token, pos=None, max_pos=0, mask=None):
+    """token[b] = argmax(logits[b]) (torch.argmax's result), and, with pos, pos = min(pos + 1, max_pos) and
+    mask.view(-1)[pos] = True: the end of a greedy decode step in one launch (tl_greedy_advance).  logits: contiguous
+    [B, vocab]; token: int64 [B]; pos: one-element int64 tensor; mask: bool tensor with one element per cache slot."""
+    if logits.dim() != 2 or not logits.is_contiguous() or token.dtype != torch.int64 or token.numel() != logits.shape[0] or not token.is_contiguous():
+        raise ValueError("logits must be contiguous [B, vocab] and token an int64 tensor of B elements")
+    if pos is not None and (pos.dtype != torch.int64 or pos.numel() != 1):
+        raise ValueError("pos must be a one-element int64 tensor")
+    if mask is not None and (pos is None or mask.dtype != torch.bool or not mask.is_contiguous() or mask.numel() <= max_pos):
+        raise ValueError("mask must be a contiguous bool tensor with more than max_pos elements, given together with pos")
+    for t in (token, pos, mask):
+        if t is not None and t.device != logits.device:
+            raise ValueError("tensors must be on one device")
+    with torch.cuda.device(logits.device):
+        rc = _lib.lib().tl_greedy_advance(logits.data_ptr(), _code(logits.dtype, "logits"), logits.shape[0], logits.shape[1], token.data_ptr(),
+                                          pos.data_ptr() if pos is not None else None, int(max_pos),
+                                          mask.data_ptr() if mask is not None else None, _stream_ptr(logits.device))
+    _lib.check(rc)
+    return token
+
+
 def add_rmsnorm(x, y, weight, eps, kmajor=False):
     """(x + y, rmsnorm(x + y) * weight) for [rows, width] tensors of one dtype; y may be None (then the
     first result is x itself).  With kmajor the second result is its transpose [width, rows], a view of a

@@ -667,6 +667,33 @@ def test_fused_single_row_step_equals_the_unfused_one(tiny, cuda):
     tiny._state = None
 
 
+def test_greedy_advance_is_argmax_position_and_mask_in_one_launch(cuda):
+    """tl_greedy_advance against torch.argmax (first of equal values, NaN above every number), with the position
+    moved on and held at its maximum and the mask bit set."""
+    from ternaryllm_amd import ops
+    g = torch.Generator().manual_seed(9)
+    for dtype in (torch.float16, torch.float32):
+        for B, V in ((1, 32000), (3, 320), (16, 1031)):
+            logits = torch.randn((B, V), generator=g).to(dtype).to(cuda)
+            logits[0, V // 3] = logits[0, V // 2] = logits[0].max() + 1      # a tie: the first one wins
+            if B > 1:
+                logits[1, 7] = float("nan")
+                logits[1, V - 1] = float("nan")
+            token = torch.full((B,), -5, dtype=torch.long, device=cuda)
+            pos = torch.tensor([10], dtype=torch.long, device=cuda)
+            mask = torch.zeros((1, 1, 1, 13), dtype=torch.bool, device=cuda)
+            for expect in (11, 12, 12):                                      # held at max_pos = 12
+                ops.greedy_advance(logits, token, pos, 12, mask)
+                assert torch.equal(token, logits.argmax(-1)), (dtype, B, V)
+                assert int(pos) == expect and bool(mask.view(-1)[expect])
+            assert mask.view(-1).nonzero().flatten().tolist() == [11, 12]
+            only = torch.zeros(B, dtype=torch.long, device=cuda)
+            ops.greedy_advance(logits, only)                                  # the argmax alone
+            assert torch.equal(only, logits.argmax(-1))
+    with pytest.raises(ValueError):
+        ops.greedy_advance(logits, token.int())
+
+
 def test_graph_replay_equals_eager_decode(tiny, cuda):
     g = torch.Generator().manual_seed(4)
     tokens = torch.randint(0, tiny.config.vocab_size, (3, 40), generator=g).to(cuda)
