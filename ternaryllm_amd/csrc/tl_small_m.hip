@@ -1590,7 +1590,7 @@ __global__ __launch_bounds__(NT) void tl_spmv_tiles(KernelArgs a)
     // memory to the launch.  (Kept as loaded: a conversion here would wait for the value.  Issued behind the wave's
     // tile loads instead, the decoder's step was 1.6 % slower.)
     uint32_t raw_scale = 0u, raw_residual = 0u, raw_next_w = 0u;
-    if (tid < TL_BLOCK_COLUMNS && nb * TL_BLOCK_COLUMNS + tid < a.N) {
+    if ((a.w0.scale || a.residual || a.chain_w) && tid < TL_BLOCK_COLUMNS && nb * TL_BLOCK_COLUMNS + tid < a.N) {
         const int n = nb * TL_BLOCK_COLUMNS + tid;
         if (a.w0.scale) raw_scale = load_raw(a.w0.scale, a.scale_f16, n);
         if (a.residual) raw_residual = load_raw(a.residual, a.y_f16, n);
