@@ -1557,9 +1557,22 @@ constexpr int kTilesMaxOwn = 8;  // tiles a wave of tl_spmv_tiles may own
 
 constexpr int kNormNone = 0, kNormInside = 1, kNormSums = 2;
 
-template <bool XF16, int NT, int NORM = kNormNone>
+// EPI: what the epilogue does, as far as the launcher knows it when it picks the kernel.  kEpiAny looks at the
+// arguments; kEpiNone has no scale, residual row or next norm's weight to read and is built without that code (it
+// would stand in front of the plain product's first loads); the others are the decoder's three epilogues with every
+// operand a row of halves: a scale alone, a scale and the SiLU gate, a scale + residual row + next norm's weight.
+constexpr int kEpiNone = 0, kEpiAny = 1, kEpiScale = 2, kEpiGated = 3, kEpiChain = 4;
+
+template <bool XF16, int NT, int NORM = kNormNone, int EPI = kEpiAny>
 __global__ __launch_bounds__(NT) void tl_spmv_tiles(KernelArgs a)
 {
+    constexpr bool OPERANDS = EPI != kEpiNone;
+    constexpr bool FIXED = EPI >= kEpiScale;  // the set of operands and their types are known here
+    const bool has_scale = FIXED ? true : a.w0.scale != nullptr;
+    const bool has_residual = EPI == kEpiChain ? true : EPI == kEpiAny ? a.residual != nullptr : false;
+    const bool has_next = EPI == kEpiChain ? true : EPI == kEpiAny ? a.chain_w != nullptr : false;
+    const bool gated = EPI == kEpiGated ? true : EPI <= kEpiAny ? a.gated != 0 : false;
+    const int scale_f16 = FIXED ? 1 : a.scale_f16, y_f16 = FIXED ? 1 : a.y_f16;
     extern __shared__ __align__(16) unsigned char lds[];
     using XT = typename std::conditional<XF16, __half, float>::type;
     constexpr int ES = (int)sizeof(XT);
@@ -1582,19 +1595,19 @@ __global__ __launch_bounds__(NT) void tl_spmv_tiles(KernelArgs a)
     // (the table entries of this wave's first tile are asked for together with the block's first: what stands
     // between here and the tile loop then runs while they are on their way.  Asking for those of all its tiles here
     // made the decoder's step 3 % slower, in one batch behind the first tile's loads 2 %.)
-    const int first_tile = min(wave, a.T - 1);
-    const uint32_t first_lo = cs[first_tile], first_hi = cs[first_tile + 1];
+    const int first_tile = OPERANDS ? min(wave, a.T - 1) : 0;
+    const uint32_t first_lo = OPERANDS ? cs[first_tile] : 0u, first_hi = OPERANDS ? cs[first_tile + 1] : 0u;
 
     // What the epilogue's 16 lanes need from memory besides the sums -- the column's scale, the residual value, the
     // next norm's weight -- is asked for here, ahead of everything else: a load at the end would add its trip to
     // memory to the launch.  (Kept as loaded: a conversion here would wait for the value.  Issued behind the wave's
     // tile loads instead, the decoder's step was 1.6 % slower.)
     uint32_t raw_scale = 0u, raw_residual = 0u, raw_next_w = 0u;
-    if ((a.w0.scale || a.residual || a.chain_w) && tid < TL_BLOCK_COLUMNS && nb * TL_BLOCK_COLUMNS + tid < a.N) {
+    if (OPERANDS && tid < TL_BLOCK_COLUMNS && nb * TL_BLOCK_COLUMNS + tid < a.N) {
         const int n = nb * TL_BLOCK_COLUMNS + tid;
-        if (a.w0.scale) raw_scale = load_raw(a.w0.scale, a.scale_f16, n);
-        if (a.residual) raw_residual = load_raw(a.residual, a.y_f16, n);
-        if (a.chain_w) raw_next_w = load_raw(a.chain_w, a.y_f16, n);
+        if (has_scale) raw_scale = load_raw(a.w0.scale, scale_f16, n);
+        if (has_residual) raw_residual = load_raw(a.residual, y_f16, n);
+        if (has_next) raw_next_w = load_raw(a.chain_w, y_f16, n);
     }
 
     float squares = 0.f;  // this lane's share of sum(in^2): of the row itself (kNormInside), of the sums that came with it (kNormSums)
@@ -1627,8 +1640,8 @@ __global__ __launch_bounds__(NT) void tl_spmv_tiles(KernelArgs a)
         loads[j] = 0;
         const int t = wave + j * W;
         if (t < a.T) {
-            const uint32_t lo = j == 0 ? first_lo : cs[t];
-            const int vectors = (int)(((j == 0 ? first_hi : cs[t + 1]) - lo) / 4);
+            const uint32_t lo = OPERANDS && j == 0 ? first_lo : cs[t];
+            const int vectors = (int)(((OPERANDS && j == 0 ? first_hi : cs[t + 1]) - lo) / 4);
             unsigned char* dst = buf + (size_t)(lo - base) * 4;
             for (int first = 0; first < vectors; first += 64) {
                 if (first + lane < vectors)
@@ -1710,25 +1723,25 @@ __global__ __launch_bounds__(NT) void tl_spmv_tiles(KernelArgs a)
             sum *= rsqrtf(total / (float)a.K + a.eps);
         }
         const int n = nb * TL_BLOCK_COLUMNS + tid;
-        const float col_scale = a.w0.scale ? raw_value(raw_scale, a.scale_f16) : 1.0f;
-        const float col_residual = raw_value(raw_residual, a.y_f16), col_next_w = raw_value(raw_next_w, a.y_f16);
-        if (a.gated) {
-            const float y = n < a.N ? as_output(sum * col_scale, a.y_f16) : 0.f;
+        const float col_scale = OPERANDS && has_scale ? raw_value(raw_scale, scale_f16) : 1.0f;
+        const float col_residual = raw_value(raw_residual, y_f16), col_next_w = raw_value(raw_next_w, y_f16);
+        if (gated) {
+            const float y = n < a.N ? as_output(sum * col_scale, y_f16) : 0.f;
             const float up = __shfl_xor(y, 1, 64);  // the odd neighbour's
-            if (!(tid & 1) && n + 1 < a.N) store_out(a.Y, a.y_f16, n / 2, gate_pair(y, up, a.y_f16));
+            if (!(tid & 1) && n + 1 < a.N) store_out(a.Y, y_f16, n / 2, gate_pair(y, up, y_f16));
             return;
         }
         float v = sum * col_scale;
-        if (a.residual) v = as_output(v, a.y_f16) + col_residual;  // (as store_result adds it)
-        if (a.chain_w) {
+        if (has_residual) v = as_output(v, y_f16) + col_residual;  // (as store_result adds it)
+        if (has_next) {
             // The row goes on into an RMSNorm and a product: leave it multiplied by that norm's weight (rounded as the
             // norm inside the next kernel would round it) and the block's share of the sum of its squares beside the
             // row itself, so that the next product starts as a plain one (kNormSums).
             float y = 0.f;
             if (n < a.N) {
-                y = as_output(v, a.y_f16);
-                store_out(a.Y, a.y_f16, n, v);
-                store_out(a.chain_image, a.y_f16, n, y * col_next_w);
+                y = as_output(v, y_f16);
+                store_out(a.Y, y_f16, n, v);
+                store_out(a.chain_image, y_f16, n, y * col_next_w);
             }
             float q = y * y;
 #pragma unroll
@@ -1736,7 +1749,7 @@ __global__ __launch_bounds__(NT) void tl_spmv_tiles(KernelArgs a)
             if (tid == 0) a.chain_sq_out[nb] = q;
             return;
         }
-        if (n < a.N) store_out(a.Y, a.y_f16, n, v);
+        if (n < a.N) store_out(a.Y, y_f16, n, v);
     }
 }
 
@@ -1991,7 +2004,7 @@ int launch_spmv_direct_nt(KernelArgs a, const tl_layout_header* h, hipStream_t s
 
 // tl_spmv_tiles: every tile of the block resident (a wave loads its own and waits for nobody else's).
 // Returns TL_ERR_UNSUPPORTED when that does not fit; the caller then takes tl_spmv_direct.
-template <bool XF16, int NT, int NORM = kNormNone>
+template <bool XF16, int NT, int NORM = kNormNone, int EPI = kEpiAny>
 int launch_spmv_tiles_nt(KernelArgs a, const tl_layout_header* h, hipStream_t st)
 {
     constexpr int es = XF16 ? 2 : 4;
@@ -2004,7 +2017,7 @@ int launch_spmv_tiles_nt(KernelArgs a, const tl_layout_header* h, hipStream_t st
     int share = std::max(1, std::min(knob(TL_SPMV_SHARE, 4), (int)ceil_div(a.NB, compute_units())));
     if (NORM == kNormInside) share = std::min(share, 3);  // the second set of images: three workgroups of K = 4096 fit a compute unit, not four
     if (lds > (size_t)(160 * 1024 / share - 1024)) return TL_ERR_UNSUPPORTED;
-    auto kernel = tl_spmv_tiles<XF16, NT, NORM>;
+    auto kernel = tl_spmv_tiles<XF16, NT, NORM, EPI>;
     static bool raised = false;  // per instantiation; a repeated or racing call is harmless
     if (!raised) {
         if (int rc = raise_lds_limit(kernel, 160 * 1024)) return rc;
@@ -2014,6 +2027,41 @@ int launch_spmv_tiles_nt(KernelArgs a, const tl_layout_header* h, hipStream_t st
     return TL_OK;
 }
 
+// The epilogue the arguments ask for, among those a kernel is built for.
+template <bool XF16>
+int tiles_epilogue(const KernelArgs& a)
+{
+    if (!a.w0.scale && !a.residual && !a.chain_w) return kEpiNone;
+    if (XF16 && a.w0.scale && a.scale_f16 && a.y_f16) {
+        if (a.gated && !a.residual && !a.chain_w) return kEpiGated;
+        if (!a.gated && a.residual && a.chain_w) return kEpiChain;
+        if (!a.gated && !a.residual && !a.chain_w) return kEpiScale;
+    }
+    return kEpiAny;
+}
+
+template <bool XF16, int NORM, int EPI>
+int launch_spmv_tiles_wide(bool wide, const KernelArgs& a, const tl_layout_header* h, hipStream_t st)
+{
+    return wide ? launch_spmv_tiles_nt<XF16, 1024, NORM, EPI>(a, h, st) : launch_spmv_tiles_nt<XF16, kBlockThreads, NORM, EPI>(a, h, st);
+}
+
+// tl_spmv_tiles with the epilogue picked: the plain product and the product on a row with its sums of squares have
+// kernels for the decoder's epilogues (fp16 only), everything else takes the one that looks at its arguments.
+template <bool XF16, int NORM>
+int launch_spmv_tiles(bool wide, const KernelArgs& a, const tl_layout_header* h, hipStream_t st)
+{
+    const int epi = tiles_epilogue<XF16>(a);
+    if constexpr (NORM == kNormNone) {
+        if (epi == kEpiNone) return launch_spmv_tiles_wide<XF16, NORM, kEpiNone>(wide, a, h, st);
+        if constexpr (XF16) {
+            if (epi == kEpiChain) return launch_spmv_tiles_wide<XF16, NORM, kEpiChain>(wide, a, h, st);
+            if (epi == kEpiScale) return launch_spmv_tiles_wide<XF16, NORM, kEpiScale>(wide, a, h, st);
+        }
+    }
+    return launch_spmv_tiles_wide<XF16, NORM, kEpiAny>(wide, a, h, st);
+}
+
 // With no more blocks than compute units a workgroup has its compute unit to itself: 1024 threads
 // (64 lanes per column) then keep more gathers in flight than 512 do.
 template <bool XF16, int PRO = kProNone>
@@ -2021,12 +2069,12 @@ int launch_spmv_direct(const KernelArgs& a, const tl_layout_header* h, hipStream
 {
     const bool wide = knob(TL_SPMV_WIDE, a.NB <= compute_units() ? 1 : 0) != 0;
     if constexpr (PRO == kProNormSums) {
-        const int rc = wide ? launch_spmv_tiles_nt<XF16, 1024, kNormSums>(a, h, st) : launch_spmv_tiles_nt<XF16, kBlockThreads, kNormSums>(a, h, st);
+        const int rc = launch_spmv_tiles<XF16, kNormSums>(wide, a, h, st);
         if (rc == TL_ERR_UNSUPPORTED) return fail(TL_ERR_UNSUPPORTED, "the weight's blocks do not fit the kernel that takes a row with its sums of squares");
         return rc;
     } else if constexpr (PRO == kProNormDeferred) {
         if (knob(TL_SPMV_TILES, 1) != 0) {
-            const int rc = wide ? launch_spmv_tiles_nt<XF16, 1024, kNormInside>(a, h, st) : launch_spmv_tiles_nt<XF16, kBlockThreads, kNormInside>(a, h, st);
+            const int rc = launch_spmv_tiles<XF16, kNormInside>(wide, a, h, st);
             if (rc != TL_ERR_UNSUPPORTED) return rc;
         }
         return wide ? launch_spmv_direct_nt<XF16, 1024, kProAddNorm>(a, h, st) : launch_spmv_direct_nt<XF16, kBlockThreads, kProAddNorm>(a, h, st);
@@ -2034,7 +2082,7 @@ int launch_spmv_direct(const KernelArgs& a, const tl_layout_header* h, hipStream
         if constexpr (PRO == kProNone) {
             // the tile-per-wave kernel where the block fits it; with the other producers it is the slower of the two
             if (knob(TL_SPMV_TILES, 1) != 0 || a.chain_w) {
-                const int rc = wide ? launch_spmv_tiles_nt<XF16, 1024>(a, h, st) : launch_spmv_tiles_nt<XF16, kBlockThreads>(a, h, st);
+                const int rc = launch_spmv_tiles<XF16, kNormNone>(wide, a, h, st);
                 if (rc != TL_ERR_UNSUPPORTED) return rc;
             }
             if (a.chain_w) return fail(TL_ERR_UNSUPPORTED, "the weight's blocks do not fit the kernel that leaves the row for the next norm");
