@@ -663,6 +663,15 @@ def test_fused_single_row_step_equals_the_unfused_one(tiny, cuda):
     graphed = tiny.generate(tokens, 10, use_graph=True)
     again = tiny.generate(tokens, 10, use_graph=True)
     assert torch.equal(eager, graphed) and torch.equal(eager, again)
+    # the split attention (its pieces folded by the last workgroup to finish) under a captured graph, replayed
+    tiny._graph = None
+    tiny._state = None
+    tiny.split_attention = True
+    split_eager = tiny.generate(tokens, 10, use_graph=False)
+    split_graphed = tiny.generate(tokens, 10, use_graph=True)
+    split_again = tiny.generate(tokens, 10, use_graph=True)
+    tiny.split_attention = False
+    assert torch.equal(split_eager, split_graphed) and torch.equal(split_eager, split_again)
     tiny._graph = None
     tiny._state = None
 
