@@ -505,23 +505,45 @@ __device__ __forceinline__ void issue_images(const KernelArgs& a, const unsigned
     }
 }
 
-// What the chained epilogue of a 16-row block adds and multiplies: the residual values of a lane's four rows of
-// column n and the next norm's weight of that column.  Asked for early, so that they are there at the very end.
+// A value of a row of halves or floats as it lies in memory, and its conversion (apart, so that the load can be
+// issued long before the value is needed).
+__device__ __forceinline__ uint32_t load_raw(const void* p, int is_f16, long long n)
+{
+    return is_f16 ? (uint32_t)static_cast<const uint16_t*>(p)[n] : static_cast<const uint32_t*>(p)[n];
+}
+__device__ __forceinline__ float raw_value(uint32_t raw, int is_f16)
+{
+    return is_f16 ? __half2float(__ushort_as_half((unsigned short)raw)) : __uint_as_float(raw);
+}
+
+// What the epilogue of a 16-row block multiplies and adds: the column's scale, the residual values of a lane's four
+// rows of column n and the next norm's weight of that column.  Asked for early, so that they are there at the very
+// end, and kept as loaded: a conversion where they are asked for would make the wave wait for each of them in turn
+// (and for every tile load issued before).
 struct ChainOperands {
-    float res[4];
-    float w;
+    uint32_t res[4];
+    uint32_t w;
+    uint32_t scale;
 };
 
 __device__ __forceinline__ ChainOperands chain_operands(const KernelArgs& a, int n, int q)
 {
-    ChainOperands o = {{0.f, 0.f, 0.f, 0.f}, 0.f};
-    if (a.chain_res && n < a.N) {
+    ChainOperands o = {{0u, 0u, 0u, 0u}, 0u, 0u};
+    if (n < a.N) {
+        if (a.w0.scale) o.scale = load_raw(a.w0.scale, a.scale_f16, n);
+        if (a.chain_res) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-            if (q * 4 + j < a.M) o.res[j] = load_scale(a.chain_res, a.y_f16, (long long)(q * 4 + j) * a.chain_ldres + n);
+            for (int j = 0; j < 4; ++j)
+                if (q * 4 + j < a.M) o.res[j] = load_raw(a.chain_res, a.y_f16, (long long)(q * 4 + j) * a.chain_ldres + n);
+        }
+        if (a.chain_image) o.w = load_raw(a.chain_w, a.y_f16, n);
     }
-    if (a.chain_image && n < a.N) o.w = load_scale(a.chain_w, a.y_f16, n);
     return o;
+}
+// the column's scale among them (0 past the last column, 1 without a scale)
+__device__ __forceinline__ float chain_scale(const KernelArgs& a, int n, const ChainOperands& early)
+{
+    return n < a.N ? (a.w0.scale ? raw_value(early.scale, a.scale_f16) : 1.0f) : 0.f;
 }
 
 // The chained part of the way out of a block of 16 columns x 16 rows.  Called by one whole wave: lane = column
@@ -536,10 +558,10 @@ __device__ __forceinline__ void chain_epilogue16(const KernelArgs& a, int nb, in
     if (a.chain_res) {
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-            if (n < a.N && q * 4 + j < a.M) out[j] = as_output(out[j], a.y_f16) + early.res[j];
+            if (n < a.N && q * 4 + j < a.M) out[j] = as_output(out[j], a.y_f16) + raw_value(early.res[j], a.y_f16);
     }
     if (a.chain_image) {
-        const float w = early.w;
+        const float w = raw_value(early.w, a.y_f16);
         float sq[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -621,7 +643,7 @@ __global__ __launch_bounds__(NT) void tl_spmm_quad(KernelArgs a)
     float4 row_factors = make_float4(1.f, 1.f, 1.f, 1.f);  // chained product, first wave: the factors of rows 4 * (lane % 4) .. + 3
     if (MT == 16 && a.chain_sq_in && tid < 64) row_factors = chain_row_factors(a, tid);
     // what the chained epilogue of the first wave adds and multiplies, asked for now rather than at the very end
-    ChainOperands early = {{0.f, 0.f, 0.f, 0.f}, 0.f};
+    ChainOperands early = {{0u, 0u, 0u, 0u}, 0u, 0u};
     if (MT == 16 && tid < 64) early = chain_operands(a, nb * TL_BLOCK_COLUMNS + ((tid / Q) & 15), tid % Q);
     int which = 0;
     for (int t = 0; t < a.T; t += TG, which ^= 1) {
@@ -673,7 +695,7 @@ __global__ __launch_bounds__(NT) void tl_spmm_quad(KernelArgs a)
             sum.x += o.x; sum.y += o.y; sum.z += o.z; sum.w += o.w;
         }
         const int n = nb * TL_BLOCK_COLUMNS + c16;
-        const float sc = n < a.N ? load_scale(a.w0.scale, a.scale_f16, n) : 0.f;
+        const float sc = MT == 16 ? chain_scale(a, n, early) : n < a.N ? load_scale(a.w0.scale, a.scale_f16, n) : 0.f;
         float out[4] = {sum.x * sc, sum.y * sc, sum.z * sc, sum.w * sc};
         if constexpr (MT == 16) chain_epilogue16(a, nb, n, c16, q, out, row_factors, early);  // (one wave here: 16 columns x 4 row quads)
         if (n < a.N) {
@@ -1063,7 +1085,7 @@ __global__ __launch_bounds__(kResWaves * 64) void tl_spmm_res(KernelArgs a)
     }
     // the blocks this wave sends out at the end (b = wave, wave + 16, ...): what their chained epilogue needs, asked for now
     float4 row_factors = make_float4(1.f, 1.f, 1.f, 1.f);
-    ChainOperands early = {{0.f, 0.f, 0.f, 0.f}, 0.f};
+    ChainOperands early = {{0u, 0u, 0u, 0u}, 0u, 0u};
     if (XF16 && wave < nblk) {
         if (a.chain_sq_in) row_factors = chain_row_factors(a, lane);
         early = chain_operands(a, (b0 + wave) * TL_BLOCK_COLUMNS + (lane >> 2), lane & 3);
@@ -1176,8 +1198,8 @@ __global__ __launch_bounds__(kResWaves * 64) void tl_spmm_res(KernelArgs a)
         // the waves with units in block b, in order: unit x belongs to wave ((x + 1) * W - 1) / U
         const int w_first = ((b * T + 1) * W - 1) / U, w_last = ((b + 1) * T * W - 1) / U;
         const int nb = b0 + b, n = nb * TL_BLOCK_COLUMNS + col;
-        const float sc = n < a.N ? load_scale(a.w0.scale, a.scale_f16, n) : 0.f;
         if constexpr (!XF16) {
+            const float sc = n < a.N ? load_scale(a.w0.scale, a.scale_f16, n) : 0.f;
             // eight fp32 rows: two per lane; the plain product only
             float2 pair = make_float2(0.f, 0.f);
             for (int w = w_first; w <= w_last; ++w)
@@ -1201,6 +1223,7 @@ __global__ __launch_bounds__(kResWaves * 64) void tl_spmm_res(KernelArgs a)
             if (a.chain_sq_in) row_factors = chain_row_factors(a, lane);
             early = chain_operands(a, n, q);
         }
+        const float sc = chain_scale(a, n, early);
         if (a.gated) {
             // gate and up column of a pair sit four lanes apart (same rows): the even column's lane writes the four products
             // (the row factor multiplies the scaled sum, as in the plain product that tl_silu_mul_pairs would follow)
@@ -1519,17 +1542,6 @@ __global__ __launch_bounds__(NT) void tl_spmv_direct(KernelArgs a)
 // multiplied by the norm weight, with the sums of squares of its values in pieces beside it -- what the product
 // that made the row leaves in its epilogue (chain_w below) -- so this kernel is the plain one plus a factor at the
 // end, with one set of images and as many workgroups to a compute unit as the plain one.
-
-// A value of a row of halves or floats as it lies in memory, and its conversion (apart, so that the load can be
-// issued long before the value is needed).
-__device__ __forceinline__ uint32_t load_raw(const void* p, int is_f16, int n)
-{
-    return is_f16 ? (uint32_t)static_cast<const uint16_t*>(p)[n] : static_cast<const uint32_t*>(p)[n];
-}
-__device__ __forceinline__ float raw_value(uint32_t raw, int is_f16)
-{
-    return is_f16 ? __half2float(__ushort_as_half((unsigned short)raw)) : __uint_as_float(raw);
-}
 
 // Waits until at most `later` of this wave's vector-memory instructions are outstanding (they complete in
 // order): everything issued before the last `later` has then arrived.  Counts above 13 wait for a few more.
