@@ -313,6 +313,9 @@ def decode_nodes_leg(model, dev, pos_value):
     # the step's own launches: with row_chain the o and down products leave the next norm's image and sums of squares,
     # and the products behind a norm start from those
     chain = model.row_chain
+    fold = model.piece_fold if chain and not model.split_attention else 0   # the attention leaves pieces, the o product folds them
+    if fold:
+        pieces_row = model._attend(qkv_row, model._cache_of(L[0], 0), model._cache_of(L[0], 1), pos, False, pieces=True, splits=fold)
     if chain:
         _, image, squares = ops.spmv_add(L[0].o_proj.device_weight(), att_row, x, L[0].o_proj.w_scale, next_norm_weight=L[0].post_attention_layernorm.weight)
 
@@ -326,6 +329,18 @@ def decode_nodes_leg(model, dev, pos_value):
             return ops.spmv_add(m.device_weight(), row, x, m.w_scale, next_norm_weight=next_norm.weight)
         return ops.spmv_add(m.device_weight(), row, x, m.w_scale)
 
+    def attention(i):
+        caches = model._cache_of(L[i], 0), model._cache_of(L[i], 1)
+        if fold:
+            return model._attend(qkv_row, *caches, pos, False, pieces=True, splits=fold)
+        return model._attend(qkv_row, *caches, pos, False, splits=None if model.split_attention else 1)
+
+    def o_product(i):
+        if fold:
+            return ops.spmv_attn_combine(L[i].o_proj.device_weight(), pieces_row, c.head_dim, model.dtype, L[i].o_proj.w_scale, residual=x,
+                                         next_norm_weight=L[i].post_attention_layernorm.weight)
+        return ends_block(L[i].o_proj, att_row, L[i].post_attention_layernorm)
+
     norm_note = "RMSNorm factor from the sums that came with its input" if chain else "RMSNorm on its input"
     add_note = " + residual + next norm's image and sums" if chain else " + residual"
     kv_bytes = 2 * c.num_attention_heads * (pos_value + 1) * c.head_dim * x.element_size()
@@ -338,10 +353,9 @@ def decode_nodes_leg(model, dev, pos_value):
     kinds = [
         ("q|k|v product, " + norm_note, lambda i: behind_norm(L[i].qkv_proj, L[i].input_layernorm),
          lambda i: ops.stream_read_probe(blob(L[i].qkv_proj), folds), blob(L[0].qkv_proj).numel()),
-        ("rotary + cache row + attention over %d rows" % (pos_value + 1),
-         lambda i: model._attend(qkv_row, model._cache_of(L[i], 0), model._cache_of(L[i], 1), pos, False, splits=None if model.split_attention else 1),
+        ("rotary + cache row + attention over %d rows" % (pos_value + 1) + (", left as %d pieces per head" % fold if fold else ""), attention,
          lambda i: ops.stream_read_probe(model._cache[i].reshape(-1).view(torch.uint8)[:kv_bytes], folds), kv_bytes),
-        ("o product" + add_note, lambda i: ends_block(L[i].o_proj, att_row, L[i].post_attention_layernorm),
+        ("o product" + (" on the fold of the attention's pieces" if fold else "") + add_note, o_product,
          lambda i: ops.stream_read_probe(blob(L[i].o_proj), folds), blob(L[0].o_proj).numel()),
         ("gate|up product, " + norm_note + ", SiLU gate in its epilogue", lambda i: behind_norm(L[i].gate_up_proj, L[i].post_attention_layernorm, gated=True),
          lambda i: ops.stream_read_probe(blob(L[i].gate_up_proj), folds), blob(L[0].gate_up_proj).numel()),

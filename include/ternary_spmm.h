@@ -443,6 +443,15 @@ int tl_spmv_attn_combine_add(const tl_layout_header* header, const void* blob_de
                              int splits, int head_dim, int x_dtype, const void* residual, void* Y, int y_dtype,
                              const void* scale, int scale_dtype, void* stream);
 
+/* tl_spmv_attn_combine_add that also leaves what tl_spmv_add_norm leaves for the RMSNorm and product behind it:
+ * image_out[N] = Y * next_norm_weight and squares_out[ceil(N / 16)], the sums of Y^2 over runs of 16 values.  Served
+ * by the kernel that folds the pieces of each wave's own tiles; TL_ERR_UNSUPPORTED where the weight's blocks do not
+ * fit it (more than two tiles per wave, or more heads x splits under one tile than its table holds). */
+int tl_spmv_attn_combine_add_norm(const tl_layout_header* header, const void* blob_dev, const void* pieces,
+                                  int splits, int head_dim, int x_dtype, const void* residual, void* Y, int y_dtype,
+                                  const void* scale, int scale_dtype, const void* next_norm_weight,
+                                  void* image_out, float* squares_out, void* stream);
+
 /* The end of a greedy decode step in one launch: token[b] = argmax of logits[b][0 .. vocab) (the first of equal
  * values; a NaN counts as larger than any number -- torch.argmax's rule), then, when pos_dev is not NULL,
  * *pos_dev = min(*pos_dev + 1, max_pos) and, when mask is not NULL too, mask[*pos_dev] = 1 (one byte per cache slot).

@@ -94,6 +94,7 @@ SIGNATURES = {
     "tl_decode_attention_rope": (_INT, [_VP, _VP, _VP, _VP, _VP, _INT, _I64, _INT, _INT, _I64, _VP, _VP, _I64, _INT, _VP, _I64, _VP]),
     "tl_spmv_attn_combine": (_INT, [_HDRP, _VP, _VP, _INT, _INT, _INT, _VP, _INT, _VP, _INT, _VP]),
     "tl_spmv_attn_combine_add": (_INT, [_HDRP, _VP, _VP, _INT, _INT, _INT, _VP, _VP, _INT, _VP, _INT, _VP]),
+    "tl_spmv_attn_combine_add_norm": (_INT, [_HDRP, _VP, _VP, _INT, _INT, _INT, _VP, _VP, _INT, _VP, _INT, _VP, _VP, _VP, _VP]),
     "tl_spmv_add": (_INT, [_HDRP, _VP, _VP, _INT, _VP, _VP, _INT, _VP, _INT, _VP]),
     "tl_spmv_add_norm": (_INT, [_HDRP, _VP, _VP, _INT, _VP, _VP, _INT, _VP, _INT, _VP, _VP, _VP, _VP]),
     "tl_add_rmsnorm": (_INT, [_VP, _VP, _VP, _INT, _I64, _INT, ctypes.c_float, _VP, _VP, _I64, _VP]),

@@ -1287,6 +1287,11 @@ __global__ __launch_bounds__(kResWaves * 64) void tl_spmm_res(KernelArgs a)
 // Roundings are those of the separate kernels (tl_silu_mul, tl_add_rmsnorm, tl_attn_combine): s, the SiLU and x
 // are rounded to the activation type.
 constexpr int kProNone = 0, kProSiluGate = 1, kProAddNorm = 2, kProAttnCombine = 3;
+
+// exp(m - top) for the top score m of one piece of a head's cache rows and the top of all of them; a piece without
+// rows (m = -inf) weighs nothing
+__device__ __forceinline__ float attn_piece_weight(float m, float top) { return m == -INFINITY ? 0.f : __expf(m - top); }
+
 constexpr int kProNormDeferred = 4;  // launcher only: RMSNorm whose factor multiplies the sums (tl_spmv_tiles), else kProAddNorm
 constexpr int kProNormSums = 5;      // launcher only: the row comes multiplied by the norm weight, its squares summed in pieces (tl_spmv_tiles alone)
 
@@ -1449,14 +1454,9 @@ __global__ __launch_bounds__(NT) void tl_spmv_direct(KernelArgs a)
             float top = -INFINITY;
             for (int sidx = 0; sidx < sp; ++sidx) top = fmaxf(top, stats[(size_t)sidx * (hd + 4)]);
             float norm = 0.f;
-            for (int sidx = 0; sidx < sp; ++sidx) {
-                const float m = stats[(size_t)sidx * (hd + 4)];
-                norm = fmaf(stats[(size_t)sidx * (hd + 4) + 1], m == -INFINITY ? 0.f : __expf(m - top), norm);
-            }
-            for (int sidx = 0; sidx < sp; ++sidx) {
-                const float m = stats[(size_t)sidx * (hd + 4)];
-                wts[h * sp + sidx] = m == -INFINITY ? 0.f : __expf(m - top) / norm;
-            }
+            for (int sidx = 0; sidx < sp; ++sidx) norm = fmaf(stats[(size_t)sidx * (hd + 4) + 1], attn_piece_weight(stats[(size_t)sidx * (hd + 4)], top), norm);
+            const float inv = __builtin_amdgcn_rcpf(norm);  // (tl_spmv_tiles' kNormCombine takes the same steps)
+            for (int sidx = 0; sidx < sp; ++sidx) wts[h * sp + sidx] = attn_piece_weight(stats[(size_t)sidx * (hd + 4)], top) * inv;
         }
         piece_w = wts;
         __syncthreads();
@@ -1567,7 +1567,15 @@ __device__ __forceinline__ void tiles_wait_vm(int later)
 
 constexpr int kTilesMaxOwn = 8;  // tiles a wave of tl_spmv_tiles may own
 
-constexpr int kNormNone = 0, kNormInside = 1, kNormSums = 2;
+constexpr int kNormNone = 0, kNormInside = 1, kNormSums = 2, kNormCombine = 3;
+
+// NORM == kNormCombine: the row is the attention output that the pieces of a split decode attention add up to (the
+// layout tl_spmv_direct's kProAttnCombine reads, and its arithmetic, operation for operation).  A wave fetches the
+// pieces of its own tiles -- per split 16 bytes (4 rows) per lane, and the (top, norm) pairs of the heads the tile
+// touches -- into LDS ahead of its chunks, folds them while the chunks are on their way and writes the tile's image;
+// it waits for no other wave.  A wave owns at most kCombineOwn tiles here.
+constexpr int kCombineOwn = 2;
+constexpr int kCombineStats = 40;  // (top, norm) entries (heads a tile touches x splits) a tile may need, 16 bytes each
 
 // EPI: what the epilogue does, as far as the launcher knows it when it picks the kernel.  kEpiAny looks at the
 // arguments; kEpiNone has no scale, residual row or next norm's weight to read and is built without that code (it
@@ -1591,7 +1599,9 @@ __global__ __launch_bounds__(NT) void tl_spmv_tiles(KernelArgs a)
     constexpr int VE = 16 / ES;                  // values per 16-byte piece
     constexpr int PITCH = kTileSlots + kSpmvImageSkew / ES;  // slots from one tile image to the next
     constexpr int W = NT / 64;                   // waves
-    constexpr int kMaxOwn = kTilesMaxOwn;        // tiles a wave may own (the launcher holds T to W * kMaxOwn)
+    constexpr int kMaxOwn = NORM == kNormCombine ? kCombineOwn : kTilesMaxOwn;  // tiles a wave may own (the launcher holds T to W * kMaxOwn)
+    constexpr bool NORMED = NORM == kNormInside || NORM == kNormSums;  // the sums are multiplied by the row's 1/rms at the end
+    constexpr bool ROW_MADE = NORM == kNormInside || NORM == kNormCombine;  // the images are made here, not copied from the row
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nb = blockIdx.x;
@@ -1632,6 +1642,31 @@ __global__ __launch_bounds__(NT) void tl_spmv_tiles(KernelArgs a)
         squares = s0 + s1;
         for (int i = tid + 2 * NT; i < blocks; i += NT) squares += a.chain_sq_in[i];  // (K above 16 * 2 * NT)
     }
+    float* pcs = reinterpret_cast<float*>(weights);  // kNormCombine: [T][splits][256] values of the pieces, a tile's rows side by side
+    unsigned char* stats = weights + (size_t)a.T * a.pro_splits * (kTileSlots * 4) + (size_t)wave * (kCombineOwn * kCombineStats * 16);  // this wave's [kCombineOwn][kCombineStats] entries
+    if constexpr (NORM == kNormCombine) {
+        // the pieces of this wave's tiles, ahead of every chunk (k / head width and lane / splits by multiplication;
+        // offsets in 32 bits: the launcher holds the pieces to 2^31 bytes)
+        const int S = a.pro_splits, hd = a.pro_hd, pitch = hd + 4;
+        const float* pieces = static_cast<const float*>(a.X);
+        const int hh = (int)__umulhi((unsigned)lane, a.vpt_magic), stat_at = (hh * S + (lane - hh * S)) * pitch + hd;
+#pragma unroll
+        for (int j = 0; j < kMaxOwn; ++j) {
+            const int t = wave + j * W;
+            if (t < a.T) {
+                const int k0 = t * a.tile_rows, rows_here = min(a.tile_rows, a.K - k0);
+                const int k = k0 + lane * 4, h = (int)__umulhi((unsigned)k, a.tile_magic);
+                const float* src = pieces + (unsigned)(h * (S - 1) * pitch + h * 4 + k);  // (h * S) * pitch + (k - h * hd)
+                float* dst = pcs + (unsigned)(t * S) * kTileSlots;
+                for (int sidx = 0; sidx < S; ++sidx)
+                    if (lane * 4 < rows_here)
+                        __builtin_amdgcn_global_load_lds((global_ptr)(src + (unsigned)(sidx * pitch)), (lds_ptr)(dst + sidx * kTileSlots), 16, 0, 0);
+                const int h0 = (int)__umulhi((unsigned)k0, a.tile_magic), nh = (int)__umulhi((unsigned)(k0 + rows_here - 1), a.tile_magic) - h0 + 1;
+                if (lane < nh * S)
+                    __builtin_amdgcn_global_load_lds((global_ptr)(pieces + (unsigned)(h0 * S * pitch + stat_at)), (lds_ptr)(stats + j * (kCombineStats * 16)), 16, 0, 0);
+            }
+        }
+    }
     if constexpr (NORM == kNormInside) {
         // the row and the norm weight of this wave's tiles, ahead of every chunk
 #pragma unroll
@@ -1664,7 +1699,7 @@ __global__ __launch_bounds__(NT) void tl_spmv_tiles(KernelArgs a)
             // slot among them) is zeroed
             const int rows_here = min(a.tile_rows, a.K - t * a.tile_rows);
             unsigned char* image = xs + (size_t)t * PITCH * ES;
-            if constexpr (NORM != kNormInside) {
+            if constexpr (!ROW_MADE) {
                 if (lane * VE < rows_here)
                     __builtin_amdgcn_global_load_lds((global_ptr)(Xb + ((size_t)t * a.tile_rows + (size_t)lane * VE) * ES), (lds_ptr)image, 16, 0, 0);
                 ++loads[j];
@@ -1697,6 +1732,75 @@ __global__ __launch_bounds__(NT) void tl_spmv_tiles(KernelArgs a)
         }
     }
 
+    if constexpr (NORM == kNormCombine) {
+        int chunk_loads = 0;
+#pragma unroll
+        for (int j = 0; j < kMaxOwn; ++j) chunk_loads += loads[j];
+        tiles_wait_vm(chunk_loads);  // the pieces are here when only the chunk loads are outstanding
+        // SC: the number of pieces per head where the code is built for it (their weights then stay in registers), 0: any
+        auto fold = [&](auto SC) {
+            constexpr int SK = decltype(SC)::value;
+            const int S = SK ? SK : a.pro_splits;
+#pragma unroll
+            for (int j = 0; j < kMaxOwn; ++j) {
+                const int t = wave + j * W;
+                if (t < a.T) {
+                    const int k0 = t * a.tile_rows;
+                    if (lane * VE < min(a.tile_rows, a.K - k0)) {
+                        // the piece of VE values never straddles heads (the head width is a multiple of VE)
+                        const int hh = (int)__umulhi((unsigned)(k0 + lane * VE), a.tile_magic) - (int)__umulhi((unsigned)k0, a.tile_magic);
+                        const float4* st = reinterpret_cast<const float4*>(stats + j * (kCombineStats * 16)) + hh * S;
+                        const float* p = pcs + (unsigned)(t * S) * kTileSlots + lane * VE;
+                        float f[VE];
+#pragma unroll
+                        for (int e = 0; e < VE; ++e) f[e] = 0.f;
+                        auto add_piece = [&](int sidx, float w) {
+#pragma unroll
+                            for (int e4 = 0; e4 < VE; e4 += 4) {
+                                const float4 v = *reinterpret_cast<const float4*>(p + sidx * kTileSlots + e4);
+                                f[e4] = fmaf(v.x, w, f[e4]);
+                                f[e4 + 1] = fmaf(v.y, w, f[e4 + 1]);
+                                f[e4 + 2] = fmaf(v.z, w, f[e4 + 2]);
+                                f[e4 + 3] = fmaf(v.w, w, f[e4 + 3]);
+                            }
+                        };
+                        float top = -INFINITY, norm = 0.f;
+                        if constexpr (SK != 0) {
+                            float ex[SK ? SK : 1];
+#pragma unroll
+                            for (int sidx = 0; sidx < SK; ++sidx) top = fmaxf(top, st[sidx].x);
+#pragma unroll
+                            for (int sidx = 0; sidx < SK; ++sidx) {
+                                const float4 e = st[sidx];
+                                ex[sidx] = attn_piece_weight(e.x, top);
+                                norm = fmaf(e.y, ex[sidx], norm);
+                            }
+                            const float inv = __builtin_amdgcn_rcpf(norm);
+#pragma unroll
+                            for (int sidx = 0; sidx < SK; ++sidx) add_piece(sidx, ex[sidx] * inv);
+                        } else {
+                            for (int sidx = 0; sidx < S; ++sidx) top = fmaxf(top, st[sidx].x);
+                            for (int sidx = 0; sidx < S; ++sidx) {
+                                const float4 e = st[sidx];
+                                norm = fmaf(e.y, attn_piece_weight(e.x, top), norm);
+                            }
+                            const float inv = __builtin_amdgcn_rcpf(norm);
+                            for (int sidx = 0; sidx < S; ++sidx) add_piece(sidx, attn_piece_weight(st[sidx].x, top) * inv);
+                        }
+                        u32x4 out;
+                        XT* o = reinterpret_cast<XT*>(&out);
+#pragma unroll
+                        for (int e = 0; e < VE; ++e) o[e] = XT(f[e]);
+                        *reinterpret_cast<u32x4*>(xs + (size_t)t * PITCH * ES + (size_t)lane * 16) = out;
+                    }
+                }
+            }
+        };
+        if (a.pro_splits == 2) fold(std::integral_constant<int, 2>());
+        else if (a.pro_splits == 4) fold(std::integral_constant<int, 4>());
+        else fold(std::integral_constant<int, 0>());
+    }
+
     const int c16 = lane >> 2, lw = lane & 3;
     float acc[1] = {0.f};
 #pragma unroll
@@ -1718,7 +1822,7 @@ __global__ __launch_bounds__(NT) void tl_spmv_tiles(KernelArgs a)
     acc[0] += __shfl_xor(acc[0], 1, 64);
     acc[0] += __shfl_xor(acc[0], 2, 64);
     if (lw == 0) red[wave * TL_BLOCK_COLUMNS + c16] = acc[0];
-    if constexpr (NORM != kNormNone) {
+    if constexpr (NORMED) {
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) squares += __shfl_xor(squares, off, 64);
         if (lane == 0) red[W * TL_BLOCK_COLUMNS + wave] = squares;
@@ -1728,7 +1832,7 @@ __global__ __launch_bounds__(NT) void tl_spmv_tiles(KernelArgs a)
         float sum = 0.f;
 #pragma unroll
         for (int w = 0; w < W; ++w) sum += red[w * TL_BLOCK_COLUMNS + tid];
-        if constexpr (NORM != kNormNone) {
+        if constexpr (NORMED) {
             float total = 0.f;
 #pragma unroll
             for (int w = 0; w < W; ++w) total += red[W * TL_BLOCK_COLUMNS + w];
@@ -2022,10 +2126,20 @@ int launch_spmv_tiles_nt(KernelArgs a, const tl_layout_header* h, hipStream_t st
     constexpr int es = XF16 ? 2 : 4;
     const int tile_bytes = kTileSlots * es + kSpmvImageSkew;
     const int chunk_bytes = (int)h->max_chunk_dwords * 4;
-    if (a.T > (NT / 64) * kTilesMaxOwn) return TL_ERR_UNSUPPORTED;
+    if (a.T > (NT / 64) * (NORM == kNormCombine ? kCombineOwn : kTilesMaxOwn)) return TL_ERR_UNSUPPORTED;
     a.xs_bytes = a.T * tile_bytes;
     a.buf_bytes = (int)round_up((int64_t)a.T * chunk_bytes, 16);
-    const size_t lds = (size_t)a.xs_bytes * (NORM == kNormInside ? 2 : 1) + a.buf_bytes + (size_t)(((NT / 64) * (TL_BLOCK_COLUMNS + 1) + 3) & ~3) * 4;
+    size_t lds = (size_t)a.xs_bytes * (NORM == kNormInside ? 2 : 1) + a.buf_bytes + (size_t)(((NT / 64) * (TL_BLOCK_COLUMNS + 1) + 3) & ~3) * 4;
+    if (NORM == kNormCombine) {
+        // heads a tile may touch x splits: one 16-byte entry each in the wave's table; divisions by multiplication
+        const int heads_per_tile = (a.tile_rows + a.pro_hd - 2) / a.pro_hd + 1;
+        if (heads_per_tile * a.pro_splits > kCombineStats || a.tile_rows % 4 || a.pro_hd % 4 || (int64_t)a.K * a.pro_hd >= (1ll << 32) ||
+            (int64_t)(a.K / a.pro_hd) * a.pro_splits * (a.pro_hd + 4) * 4 >= (1ll << 31))
+            return TL_ERR_UNSUPPORTED;
+        lds += (size_t)a.T * a.pro_splits * (kTileSlots * 4) + (size_t)(NT / 64) * kCombineOwn * kCombineStats * 16;
+        a.tile_magic = (unsigned)(((1ull << 32) + a.pro_hd - 1) / a.pro_hd);          // k / head width
+        a.vpt_magic = (unsigned)(((1ull << 32) + a.pro_splits - 1) / a.pro_splits);  // lane / splits
+    }
     int share = std::max(1, std::min(knob(TL_SPMV_SHARE, 4), (int)ceil_div(a.NB, compute_units())));
     if (NORM == kNormInside) share = std::min(share, 3);  // the second set of images: three workgroups of K = 4096 fit a compute unit, not four
     if (lds > (size_t)(160 * 1024 / share - 1024)) return TL_ERR_UNSUPPORTED;
@@ -2064,6 +2178,9 @@ template <bool XF16, int NORM>
 int launch_spmv_tiles(bool wide, const KernelArgs& a, const tl_layout_header* h, hipStream_t st)
 {
     const int epi = tiles_epilogue<XF16>(a);
+    if constexpr (NORM == kNormCombine && XF16) {
+        if (epi == kEpiChain) return launch_spmv_tiles_wide<XF16, NORM, kEpiChain>(wide, a, h, st);
+    }
     if constexpr (NORM == kNormNone) {
         if (epi == kEpiNone) return launch_spmv_tiles_wide<XF16, NORM, kEpiNone>(wide, a, h, st);
         if constexpr (XF16) {
@@ -2091,6 +2208,14 @@ int launch_spmv_direct(const KernelArgs& a, const tl_layout_header* h, hipStream
         }
         return wide ? launch_spmv_direct_nt<XF16, 1024, kProAddNorm>(a, h, st) : launch_spmv_direct_nt<XF16, kBlockThreads, kProAddNorm>(a, h, st);
     } else {
+        if constexpr (PRO == kProAttnCombine) {
+            // the tile-per-wave kernel folds the pieces of a wave's own tiles; the other one folds all of them first
+            if (knob(TL_SPMV_TILES, 1) != 0 || a.chain_w) {
+                const int rc = launch_spmv_tiles<XF16, kNormCombine>(wide, a, h, st);
+                if (rc != TL_ERR_UNSUPPORTED) return rc;
+            }
+            if (a.chain_w) return fail(TL_ERR_UNSUPPORTED, "the weight's blocks do not fit the kernel that leaves the row for the next norm");
+        }
         if constexpr (PRO == kProNone) {
             // the tile-per-wave kernel where the block fits it; with the other producers it is the slower of the two
             if (knob(TL_SPMV_TILES, 1) != 0 || a.chain_w) {
@@ -2330,9 +2455,16 @@ extern "C" int tl_spmv_fused_gated(const tl_layout_header* header, const void* b
 
 namespace {
 int attn_combine_call(const tl_layout_header* header, const void* blob_dev, const void* pieces, int splits, int head_dim,
-                      int x_dtype, void* Y, int y_dtype, const void* scale, int scale_dtype, void* stream, const void* residual)
+                      int x_dtype, void* Y, int y_dtype, const void* scale, int scale_dtype, void* stream, const void* residual,
+                      const void* next_norm_weight = nullptr, void* image_out = nullptr, float* squares_out = nullptr)
 {
     if (int rc = check_header(header)) return rc;
+    if (next_norm_weight) {
+        if (!image_out || !squares_out) return fail(TL_ERR_ARG, "image_out or squares_out is null");
+        if (image_out == Y || image_out == residual) return fail(TL_ERR_ARG, "image_out must be a row of its own");
+        for (const void* p : {next_norm_weight, static_cast<const void*>(image_out), static_cast<const void*>(squares_out)})
+            if (reinterpret_cast<uintptr_t>(p) % 16) return fail(TL_ERR_ALIGN, "next_norm_weight, image_out and squares_out must be 16-byte aligned");
+    }
     if (reinterpret_cast<uintptr_t>(residual) % (y_dtype == TL_F16 ? 2 : 4)) return fail(TL_ERR_ALIGN, "residual is not aligned to its type");
     if (int rc = check_dtype(x_dtype, "x")) return rc;
     if (int rc = check_dtype(y_dtype, "y")) return rc;
@@ -2359,6 +2491,7 @@ int attn_combine_call(const tl_layout_header* header, const void* blob_dev, cons
     a.x_f16 = x_dtype == TL_F16; a.y_f16 = y_dtype == TL_F16; a.scale_f16 = scale_dtype == TL_F16;
     a.one = 1.0f;
     a.residual = residual;
+    a.chain_w = next_norm_weight; a.chain_image = image_out; a.chain_sq_out = squares_out;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int rc = a.x_f16 ? launch_spmv_direct<true, kProAttnCombine>(a, header, st) : launch_spmv_direct<false, kProAttnCombine>(a, header, st);
     if (rc) return rc;
@@ -2377,6 +2510,16 @@ extern "C" int tl_spmv_attn_combine_add(const tl_layout_header* header, const vo
 {
     if (!residual) return fail(TL_ERR_ARG, "residual is null");
     return attn_combine_call(header, blob_dev, pieces, splits, head_dim, x_dtype, Y, y_dtype, scale, scale_dtype, stream, residual);
+}
+
+extern "C" int tl_spmv_attn_combine_add_norm(const tl_layout_header* header, const void* blob_dev, const void* pieces, int splits, int head_dim,
+                                             int x_dtype, const void* residual, void* Y, int y_dtype, const void* scale, int scale_dtype,
+                                             const void* next_norm_weight, void* image_out, float* squares_out, void* stream)
+{
+    if (!residual) return fail(TL_ERR_ARG, "residual is null");
+    if (!next_norm_weight) return fail(TL_ERR_ARG, "next_norm_weight is null");
+    return attn_combine_call(header, blob_dev, pieces, splits, head_dim, x_dtype, Y, y_dtype, scale, scale_dtype, stream, residual, next_norm_weight,
+                             image_out, squares_out);
 }
 
 int tl::launch_small(KernelArgs a, const tl_layout_header* h, int x_dtype, void* workspace, int64_t workspace_bytes, hipStream_t st)

@@ -138,6 +138,11 @@ class TernaryLlamaDecoder(nn.Module):
         # single-row steps: the o and down projections prepare the row for the norm behind them (spmv_add with
         # next_norm_weight); switched off by the first step whose shapes have no such kernel
         self.row_chain = True
+        # single-row steps with a short cache and row_chain: the attention leaves this many pieces per head (their
+        # workgroups fill more of the chip than one per head does) and the o projection folds the pieces of each
+        # wave's own tiles on the way in (spmv_attn_combine); 0: one workgroup per head writes the output row.
+        # Switched off by the first step whose shapes have no such kernel.
+        self.piece_fold = 2
         self._layer_index = {id(layer): i for i, layer in enumerate(self.layers)}
 
     # -- pieces ------------------------------------------------------------------------------
@@ -226,13 +231,16 @@ class TernaryLlamaDecoder(nn.Module):
         # 5 to 48 rows: the products read a K-major image, so whatever feeds one writes it in that layout
         # (its transpose as a view) and no re-layout pass runs in front of the products
         if B == 1 and self.fused_decode:
-            if self.row_chain:
+            while self.row_chain:
                 try:
                     return self._decode_step_fused(x, pos)
                 except RuntimeError as e:
                     if "TL_ERR_UNSUPPORTED" not in str(e) or torch.cuda.is_current_stream_capturing():
                         raise
-                    self.row_chain = False
+                    if self.piece_fold and not self.split_attention:
+                        self.piece_fold = 0     # first without the fold in the o projection,
+                    else:
+                        self.row_chain = False  # then without the chain
             return self._decode_step_fused(x, pos)
         km = 5 <= B <= 48 and c.hidden_size != B and c.intermediate_size != B
         if km and 9 <= B <= 16 and self.chain_decode:
@@ -285,8 +293,9 @@ class TernaryLlamaDecoder(nn.Module):
         gate|up product applies the SiLU gate in its epilogue (columns packed as gate/up pairs); the attention rotates
         q and k and writes the cache row; with a long cache (split_attention) it shares the cache rows of a head out
         among several workgroups (32 heads alone leave seven compute units in eight idle), the last of which folds
-        their pieces (tl_decode_attention_fold); the o and down projections add their result to the residual stream
-        in their epilogue."""
+        their pieces (tl_decode_attention_fold), with a short one it leaves two pieces per head that the o projection
+        folds on its way in (piece_fold); the o and down projections add their result to the residual stream in their
+        epilogue."""
         eps = self.config.rms_norm_eps
         # x is the residual stream: every product that ends a block adds its result to it in the epilogue, and the
         # products that start one normalise it on the way in (the factor applied to their sums).  With row_chain the
@@ -301,13 +310,20 @@ class TernaryLlamaDecoder(nn.Module):
             else:
                 qkv = ops.spmv_fused(layer.qkv_proj.device_weight(), "rmsnorm_sums", image, squares, None, eps, layer.qkv_proj.w_scale)
             squares = None
-            # a long cache: the rows of a head shared out among several workgroups, the last of which folds their pieces
-            att = self._attend(qkv, self._cache_of(layer, 0), self._cache_of(layer, 1), pos, False, splits=None if self.split_attention else 1)
-            if chain:
-                x, image, squares = ops.spmv_add(layer.o_proj.device_weight(), att, x, layer.o_proj.w_scale,
-                                                 next_norm_weight=layer.post_attention_layernorm.weight)
+            caches = self._cache_of(layer, 0), self._cache_of(layer, 1)
+            if chain and self.piece_fold and not self.split_attention:
+                # a short cache: two pieces per head, folded by the o projection as it reads them
+                pieces = self._attend(qkv, *caches, pos, False, pieces=True, splits=self.piece_fold)
+                x, image, squares = ops.spmv_attn_combine(layer.o_proj.device_weight(), pieces, self.config.head_dim, qkv.dtype, layer.o_proj.w_scale,
+                                                          residual=x, next_norm_weight=layer.post_attention_layernorm.weight)
             else:
-                x = ops.spmv_add(layer.o_proj.device_weight(), att, x, layer.o_proj.w_scale)
+                # a long cache: the rows of a head shared out among several workgroups, the last of which folds their pieces
+                att = self._attend(qkv, *caches, pos, False, splits=None if self.split_attention else 1)
+                if chain:
+                    x, image, squares = ops.spmv_add(layer.o_proj.device_weight(), att, x, layer.o_proj.w_scale,
+                                                     next_norm_weight=layer.post_attention_layernorm.weight)
+                else:
+                    x = ops.spmv_add(layer.o_proj.device_weight(), att, x, layer.o_proj.w_scale)
             if squares is None:
                 gated = ops.spmv_fused(layer.gate_up_proj.device_weight(), "rmsnorm", x, None, layer.post_attention_layernorm.weight, eps,
                                        layer.gate_up_proj.w_scale, gated=True)

@@ -349,11 +349,12 @@ def spmv_add(weight, x, residual, scale=None, next_norm_weight=None):
     return y
 
 
-def spmv_attn_combine(weight, pieces, head_dim, x_dtype, scale=None, out_dtype=None, residual=None):
+def spmv_attn_combine(weight, pieces, head_dim, x_dtype, scale=None, out_dtype=None, residual=None, next_norm_weight=None):
     """y[1, N] = (a @ W) * scale where a is the attention output (rounded to x_dtype) that `pieces` -- what
     decode_attention_pieces returned for batch 1 -- add up to: the output projection with the fold of the
     pieces inside (tl_spmv_attn_combine).  residual: a row of N values of the output dtype that the result is
-    added to, as in spmv_add.  Raises RuntimeError (TL_ERR_UNSUPPORTED) where the fused kernel does not apply."""
+    added to, as in spmv_add; with next_norm_weight [N] as well, returns (y, image, squares) as spmv_add does
+    (tl_spmv_attn_combine_add_norm).  Raises RuntimeError (TL_ERR_UNSUPPORTED) where the fused kernel does not apply."""
     K, N = weight.inners, weight.columns
     if pieces.dtype != torch.float32 or pieces.dim() != 3 or not pieces.is_contiguous() or pieces.device != weight.device:
         raise ValueError("pieces must be a contiguous float32 [heads, splits, head_dim + 4] tensor on the weight's device")
@@ -365,6 +366,21 @@ def spmv_attn_combine(weight, pieces, head_dim, x_dtype, scale=None, out_dtype=N
         raise ValueError("residual must be a contiguous row of N values of the output dtype on the weight's device")
     y = torch.empty((1, N), dtype=out_dtype, device=pieces.device)
     scale, s_code = _scale_args(scale, N, pieces.device)
+    if next_norm_weight is not None:
+        if residual is None:
+            raise ValueError("next_norm_weight goes with a residual row")
+        if next_norm_weight.numel() != N or next_norm_weight.dtype != out_dtype or not next_norm_weight.is_contiguous() or \
+                next_norm_weight.device != weight.device:
+            raise ValueError("next_norm_weight must be a contiguous row of N values of the output dtype on the weight's device")
+        image = torch.empty((1, N), dtype=out_dtype, device=pieces.device)
+        squares = torch.empty((N + 15) // 16, dtype=torch.float32, device=pieces.device)
+        with torch.cuda.device(pieces.device):
+            rc = _lib.lib().tl_spmv_attn_combine_add_norm(ctypes.byref(weight.header), weight.blob.data_ptr(), pieces.data_ptr(), splits, head_dim,
+                                                          _code(x_dtype, "x_dtype"), residual.data_ptr(), y.data_ptr(), _code(out_dtype, "out_dtype"),
+                                                          scale.data_ptr() if scale is not None else None, s_code, next_norm_weight.data_ptr(),
+                                                          image.data_ptr(), squares.data_ptr(), _stream_ptr(pieces.device))
+        _lib.check(rc)
+        return y, image, squares
     with torch.cuda.device(pieces.device):
         if residual is None:
             rc = _lib.lib().tl_spmv_attn_combine(ctypes.byref(weight.header), weight.blob.data_ptr(), pieces.data_ptr(), splits, head_dim,

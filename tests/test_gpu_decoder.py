@@ -299,7 +299,7 @@ def test_split_attention_and_its_fold_inside_the_output_projection(cuda, oracle)
     launch, against the single-pass kernel and a float64 restatement (few rows, pieces without rows, a position
     past the end); and the pieces folded inside the output projection (tl_spmv_attn_combine) against the
     separate fold followed by the plain product."""
-    from tests.util import max_rel_err, ternary_weight
+    from tests.util import knobs, max_rel_err, ternary_weight
     from ternaryllm_amd import ops
     from ternaryllm_amd.packing import PackedWeight
     g = torch.Generator().manual_seed(23)
@@ -335,7 +335,7 @@ def test_split_attention_and_its_fold_inside_the_output_projection(cuda, oracle)
         vc = torch.randn((1, H, S, hd), generator=g).to(dtype).to(cuda)
         for pos in (1, 333, S - 1):
             p = torch.tensor([pos], dtype=torch.long, device=cuda)
-            for splits in (1, 4, 8):
+            for splits in (1, 2, 4, 8):
                 pieces = ops.decode_attention_pieces(q, kc, vc, p, splits=splits)
                 assert pieces.shape == (H, splits, hd + 4)
                 out = ops.spmv_attn_combine(dw, pieces, hd, dtype, scale)
@@ -344,7 +344,34 @@ def test_split_attention_and_its_fold_inside_the_output_projection(cuda, oracle)
                 # the folded row may differ from the separately folded one in its last bit (fp32 sums in another order)
                 assert max_rel_err(out.double().cpu().numpy(), unfused.double().cpu().numpy(), a.double().cpu().numpy(), w) <= tol
                 res = torch.randn(N, generator=g).to(dtype).to(cuda)
-                assert torch.equal(ops.spmv_attn_combine(dw, pieces, hd, dtype, scale, residual=res), out + res[None])
+                summed = ops.spmv_attn_combine(dw, pieces, hd, dtype, scale, residual=res)
+                assert torch.equal(summed, out + res[None])
+                # the kernel that folds the pieces of each wave's own tiles (the default where the block fits it) and
+                # the one that folds all of them first: the same row, summed over K in another order
+                with knobs(TL_SPMV_TILES="0"):
+                    other = ops.spmv_attn_combine(dw, pieces, hd, dtype, scale)
+                    assert max_rel_err(other.double().cpu().numpy(), out.double().cpu().numpy(), a.double().cpu().numpy(), w) <= tol, (pos, splits)
+                    assert torch.equal(ops.spmv_attn_combine(dw, pieces, hd, dtype, scale, residual=res), other + res[None])
+                # ... and what it leaves for the next norm, as tl_spmv_add_norm leaves it
+                nw = (1 + 0.1 * torch.randn(N, generator=g)).to(dtype).to(cuda)
+                if splits == 8:   # that many pieces of all of K do not fit the kernel's LDS
+                    with pytest.raises(RuntimeError, match="UNSUPPORTED"):
+                        ops.spmv_attn_combine(dw, pieces, hd, dtype, scale, residual=res, next_norm_weight=nw)
+                    continue
+                y, image, squares = ops.spmv_attn_combine(dw, pieces, hd, dtype, scale, residual=res, next_norm_weight=nw)
+                assert torch.equal(y, summed)
+                assert torch.equal(image, (y.float() * nw.float()[None]).to(dtype))
+                want = y[0].double().pow(2).view(N // 16, 16).sum(1)
+                assert squares.shape == (N // 16,) and (squares.double() - want).abs().max().item() <= 1e-6 * want.max().item()
+        # a weight whose tiles are too many for two per wave at 512 threads: the other kernel takes the product, and
+        # there is none that leaves the next norm's inputs
+        low = ops.DeviceWeight(PackedWeight.from_dense(w, tile_rows=120), cuda)
+        with knobs(TL_SPMV_WIDE="0"):
+            base = ops.spmv_attn_combine(low, pieces, hd, dtype, scale)
+            assert max_rel_err(base.double().cpu().numpy(), unfused.double().cpu().numpy(), a.double().cpu().numpy(), w) <= tol
+            assert torch.equal(ops.spmv_attn_combine(low, pieces, hd, dtype, scale, residual=res), base + res[None])
+            with pytest.raises(RuntimeError, match="UNSUPPORTED"):
+                ops.spmv_attn_combine(low, pieces, hd, dtype, scale, residual=res, next_norm_weight=nw)
     with pytest.raises(ValueError):
         ops.spmv_attn_combine(dw, torch.zeros((H, 2, hd + 3), device=cuda), hd, torch.float16)
     with pytest.raises(ValueError, match="splits"):
@@ -636,10 +663,14 @@ def test_fused_single_row_step_equals_the_unfused_one(tiny, cuda):
     outs = {}
     assert not tiny.split_attention   # a short cache: one workgroup per head; the split form is forced below
     assert tiny.row_chain
-    for fused in (False, True, "split", "plain"):   # "plain": the products behind a norm multiply the row and sum its squares themselves
+    assert tiny.piece_fold == 2
+    # "plain": the products behind a norm multiply the row and sum its squares themselves; "whole": one workgroup per
+    # head writes the attention's output row (the default leaves two pieces per head for the o projection to fold)
+    for fused in (False, True, "split", "plain", "whole"):
         tiny.fused_decode = bool(fused)
         tiny.split_attention = fused == "split"
         tiny.row_chain = fused != "plain"
+        tiny.piece_fold = 0 if fused == "whole" else 2
         tiny._graph = None
         tiny.prefill(tokens[:, :28])
         st = tiny._decode_state(1)
@@ -650,7 +681,8 @@ def test_fused_single_row_step_equals_the_unfused_one(tiny, cuda):
             st["mask"].copy_((torch.arange(tiny.max_seq_len, device=cuda) <= 28 + j)[None, None, None])
             logits.append(tiny._decode_step(st["token"], st["pos"], st["mask"]).float())
         outs[fused] = torch.stack(logits)
-        assert tiny.row_chain == (fused != "plain")   # no step fell back
+        assert tiny.row_chain == (fused != "plain") and tiny.piece_fold == (0 if fused == "whole" else 2)   # no step fell back
+    tiny.piece_fold = 2
     tiny.fused_decode = True
     tiny.split_attention = False
     tiny.row_chain = True
@@ -659,6 +691,7 @@ def test_fused_single_row_step_equals_the_unfused_one(tiny, cuda):
     assert (outs[True] - outs[False]).abs().max().item() <= 2e-3 * outs[False].abs().max().item()
     assert (outs["plain"] - outs[False]).abs().max().item() <= 2e-3 * outs[False].abs().max().item()
     assert (outs["split"] - outs[False]).abs().max().item() <= 2e-3 * outs[False].abs().max().item()
+    assert (outs["whole"] - outs[False]).abs().max().item() <= 2e-3 * outs[False].abs().max().item()
     eager = tiny.generate(tokens, 10, use_graph=False)
     graphed = tiny.generate(tokens, 10, use_graph=True)
     again = tiny.generate(tokens, 10, use_graph=True)
