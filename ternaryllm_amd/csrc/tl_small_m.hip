@@ -2142,6 +2142,8 @@ int launch_spmv_tiles_nt(KernelArgs a, const tl_layout_header* h, hipStream_t st
     }
     int share = std::max(1, std::min(knob(TL_SPMV_SHARE, 4), (int)ceil_div(a.NB, compute_units())));
     if (NORM == kNormInside) share = std::min(share, 3);  // the second set of images: three workgroups of K = 4096 fit a compute unit, not four
+    // (a product that only this kernel serves runs with fewer workgroups to a compute unit rather than not at all)
+    if (NORM == kNormSums || a.chain_w) share = 1;
     if (lds > (size_t)(160 * 1024 / share - 1024)) return TL_ERR_UNSUPPORTED;
     auto kernel = tl_spmv_tiles<XF16, NT, NORM, EPI>;
     static bool raised = false;  // per instantiation; a repeated or racing call is harmless

@@ -557,6 +557,23 @@ def test_single_row_product_prepares_the_next_norm(cuda, dtype, tol):
             ops.spmv_add(low, act, res, next_norm_weight=nw)
         with pytest.raises(RuntimeError, match="UNSUPPORTED"):
             ops.spmv_fused(low, "rmsnorm_sums", act, torch.ones(256, dtype=torch.float32, device=cuda), None, eps)
+    # a wide output (more than four blocks per compute unit): where four workgroups with an fp32 row's images do not fit
+    # a compute unit's LDS, fewer of them share it
+    units = torch.cuda.get_device_properties(cuda).multi_processor_count
+    for K in (4096, 1000):
+        N = 16 * (4 * units + units // 2) + 6
+        w = ternary_weight(K, N, 0.66, K + 1)
+        dw = ops.DeviceWeight(PackedWeight.from_dense(w), cuda)
+        sc = (0.5 + torch.rand(N, generator=g)).to(dtype).to(cuda)
+        y = torch.randn(K, generator=g).to(dtype).to(cuda)
+        nw = (1 + 0.1 * torch.randn(K, generator=g)).to(dtype).to(cuda)
+        image = (y.float() * nw.float()).to(dtype)[None]
+        squares = torch.nn.functional.pad(y.float().pow(2), (0, -K % 16)).view(-1, 16).sum(1).contiguous()
+        h64 = y.double() * torch.rsqrt(y.double().pow(2).mean() + eps) * nw.double()
+        ref = (image[0].double() * torch.rsqrt(y.double().pow(2).mean() + eps)).cpu().numpy()[None, :] @ w.astype("float64") * sc.double().cpu().numpy()[None, :]
+        out = ops.spmv_fused(dw, "rmsnorm_sums", image, squares, None, eps, sc)
+        assert max_rel_err(out.double().cpu().numpy(), ref, h64.cpu().numpy()[None, :], w) <= 2 * tol, K
+        assert torch.equal(ops.spmv_fused(dw, "rmsnorm_sums", image, squares, None, eps, sc, gated=True), ops.silu_mul(out, pairs=True))
 
 
 def test_silu_gate_in_the_epilogue_of_the_gate_up_product(cuda):
