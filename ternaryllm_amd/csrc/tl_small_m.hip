@@ -1645,11 +1645,11 @@ __global__ __launch_bounds__(NT) void tl_spmv_tiles(KernelArgs a)
     float* pcs = reinterpret_cast<float*>(weights);  // kNormCombine: [T][splits][256] values of the pieces, a tile's rows side by side
     unsigned char* stats = weights + (size_t)a.T * a.pro_splits * (kTileSlots * 4) + (size_t)wave * (kCombineOwn * kCombineStats * 16);  // this wave's [kCombineOwn][kCombineStats] entries
     if constexpr (NORM == kNormCombine) {
-        // the pieces of this wave's tiles, ahead of every chunk (k / head width and lane / splits by multiplication;
-        // offsets in 32 bits: the launcher holds the pieces to 2^31 bytes)
+        // the pieces of this wave's tiles, ahead of every chunk (k / head width by multiplication; offsets in 32 bits:
+        // the launcher holds the pieces to 2^31 bytes)
         const int S = a.pro_splits, hd = a.pro_hd, pitch = hd + 4;
         const float* pieces = static_cast<const float*>(a.X);
-        const int hh = (int)__umulhi((unsigned)lane, a.vpt_magic), stat_at = (hh * S + (lane - hh * S)) * pitch + hd;
+        const int stat_at = lane * pitch + hd;  // lane l asks for the l-th (top, norm) entry from the tile's first head on
 #pragma unroll
         for (int j = 0; j < kMaxOwn; ++j) {
             const int t = wave + j * W;
@@ -2131,14 +2131,13 @@ int launch_spmv_tiles_nt(KernelArgs a, const tl_layout_header* h, hipStream_t st
     a.buf_bytes = (int)round_up((int64_t)a.T * chunk_bytes, 16);
     size_t lds = (size_t)a.xs_bytes * (NORM == kNormInside ? 2 : 1) + a.buf_bytes + (size_t)(((NT / 64) * (TL_BLOCK_COLUMNS + 1) + 3) & ~3) * 4;
     if (NORM == kNormCombine) {
-        // heads a tile may touch x splits: one 16-byte entry each in the wave's table; divisions by multiplication
+        // heads a tile may touch x splits: one 16-byte entry each in the wave's table; k / head width by multiplication
         const int heads_per_tile = (a.tile_rows + a.pro_hd - 2) / a.pro_hd + 1;
         if (heads_per_tile * a.pro_splits > kCombineStats || a.tile_rows % 4 || a.pro_hd % 4 || (int64_t)a.K * a.pro_hd >= (1ll << 32) ||
             (int64_t)(a.K / a.pro_hd) * a.pro_splits * (a.pro_hd + 4) * 4 >= (1ll << 31))
             return TL_ERR_UNSUPPORTED;
         lds += (size_t)a.T * a.pro_splits * (kTileSlots * 4) + (size_t)(NT / 64) * kCombineOwn * kCombineStats * 16;
-        a.tile_magic = (unsigned)(((1ull << 32) + a.pro_hd - 1) / a.pro_hd);          // k / head width
-        a.vpt_magic = (unsigned)(((1ull << 32) + a.pro_splits - 1) / a.pro_splits);  // lane / splits
+        a.tile_magic = (unsigned)(((1ull << 32) + a.pro_hd - 1) / a.pro_hd);  // k / head width
     }
     int share = std::max(1, std::min(knob(TL_SPMV_SHARE, 4), (int)ceil_div(a.NB, compute_units())));
     if (NORM == kNormInside) share = std::min(share, 3);  // the second set of images: three workgroups of K = 4096 fit a compute unit, not four
