@@ -557,11 +557,12 @@ def test_single_row_product_prepares_the_next_norm(cuda, dtype, tol):
             ops.spmv_add(low, act, res, next_norm_weight=nw)
         with pytest.raises(RuntimeError, match="UNSUPPORTED"):
             ops.spmv_fused(low, "rmsnorm_sums", act, torch.ones(256, dtype=torch.float32, device=cuda), None, eps)
-    # a wide output (more than four blocks per compute unit): where four workgroups with an fp32 row's images do not fit
-    # a compute unit's LDS, fewer of them share it
+    # wide outputs.  More than four blocks per compute unit: where four workgroups with an fp32 row's images do not fit a
+    # compute unit's LDS, fewer of them share it.  Between one and three: workgroups of nine waves where K's 17 tiles
+    # are then two per wave at most.
     units = torch.cuda.get_device_properties(cuda).multi_processor_count
-    for K in (4096, 1000):
-        N = 16 * (4 * units + units // 2) + 6
+    for K, halves in ((4096, 9), (1000, 9), (4096, 3)):
+        N = 16 * (halves * units // 2) + 6
         w = ternary_weight(K, N, 0.66, K + 1)
         dw = ops.DeviceWeight(PackedWeight.from_dense(w), cuda)
         sc = (0.5 + torch.rand(N, generator=g)).to(dtype).to(cuda)
