@@ -313,7 +313,7 @@ def decode_nodes_leg(model, dev, pos_value):
     # the step's own launches: with row_chain the o and down products leave the next norm's image and sums of squares,
     # and the products behind a norm start from those
     chain = model.row_chain
-    fold = model.piece_fold if chain and not model.split_attention else 0   # the attention leaves pieces, the o product folds them
+    fold = model.pieces_per_head()   # the attention leaves pieces, the o product folds them
     if fold:
         pieces_row = model._attend(qkv_row, model._cache_of(L[0], 0), model._cache_of(L[0], 1), pos, False, pieces=True, splits=fold)
     if chain:

@@ -138,10 +138,11 @@ class TernaryLlamaDecoder(nn.Module):
         # single-row steps: the o and down projections prepare the row for the norm behind them (spmv_add with
         # next_norm_weight); switched off by the first step whose shapes have no such kernel
         self.row_chain = True
-        # single-row steps with a short cache and row_chain: the attention leaves this many pieces per head (their
-        # workgroups fill more of the chip than one per head does) and the o projection folds the pieces of each
-        # wave's own tiles on the way in (spmv_attn_combine); 0: one workgroup per head writes the output row.
-        # Switched off by the first step whose shapes have no such kernel.
+        # single-row steps with row_chain: the attention leaves this many pieces per head (their workgroups fill more of
+        # the chip than one per head does; four with a long cache, split_attention) and the o projection folds the
+        # pieces of each wave's own tiles on the way in (spmv_attn_combine); 0: the attention writes the output row
+        # (one workgroup per head, or the last of several to finish).  Switched off by the first step whose shapes
+        # have no such kernel.
         self.piece_fold = 2
         self._layer_index = {id(layer): i for i, layer in enumerate(self.layers)}
 
@@ -237,7 +238,7 @@ class TernaryLlamaDecoder(nn.Module):
                 except RuntimeError as e:
                     if "TL_ERR_UNSUPPORTED" not in str(e) or torch.cuda.is_current_stream_capturing():
                         raise
-                    if self.piece_fold and not self.split_attention:
+                    if self.piece_fold:
                         self.piece_fold = 0     # first without the fold in the o projection,
                     else:
                         self.row_chain = False  # then without the chain
@@ -292,10 +293,10 @@ class TernaryLlamaDecoder(nn.Module):
         normalise their input themselves (RMSNorm with the factor applied to the sums, tl_spmv_fused "rmsnorm"); the
         gate|up product applies the SiLU gate in its epilogue (columns packed as gate/up pairs); the attention rotates
         q and k and writes the cache row; with a long cache (split_attention) it shares the cache rows of a head out
-        among several workgroups (32 heads alone leave seven compute units in eight idle), the last of which folds
-        their pieces (tl_decode_attention_fold), with a short one it leaves two pieces per head that the o projection
-        folds on its way in (piece_fold); the o and down projections add their result to the residual stream in their
-        epilogue."""
+        among several workgroups (32 heads alone leave seven compute units in eight idle); it leaves two pieces per head
+        (four with a long cache) that the o projection folds on its way in (piece_fold), or, without that, the last
+        of its workgroups to finish folds them (tl_decode_attention_fold); the o and down projections add their
+        result to the residual stream in their epilogue."""
         eps = self.config.rms_norm_eps
         # x is the residual stream: every product that ends a block adds its result to it in the epilogue, and the
         # products that start one normalise it on the way in (the factor applied to their sums).  With row_chain the
@@ -311,9 +312,9 @@ class TernaryLlamaDecoder(nn.Module):
                 qkv = ops.spmv_fused(layer.qkv_proj.device_weight(), "rmsnorm_sums", image, squares, None, eps, layer.qkv_proj.w_scale)
             squares = None
             caches = self._cache_of(layer, 0), self._cache_of(layer, 1)
-            if chain and self.piece_fold and not self.split_attention:
-                # a short cache: two pieces per head, folded by the o projection as it reads them
-                pieces = self._attend(qkv, *caches, pos, False, pieces=True, splits=self.piece_fold)
+            if self.pieces_per_head():
+                # two pieces per head (four with a long cache), folded by the o projection as it reads them
+                pieces = self._attend(qkv, *caches, pos, False, pieces=True, splits=self.pieces_per_head())
                 x, image, squares = ops.spmv_attn_combine(layer.o_proj.device_weight(), pieces, self.config.head_dim, qkv.dtype, layer.o_proj.w_scale,
                                                           residual=x, next_norm_weight=layer.post_attention_layernorm.weight)
             else:
@@ -339,6 +340,12 @@ class TernaryLlamaDecoder(nn.Module):
         if squares is None:
             return ops.spmv_fused(self.lm_head.device_weight(), "rmsnorm", x, None, self.norm.weight, eps, self.lm_head.w_scale)
         return ops.spmv_fused(self.lm_head.device_weight(), "rmsnorm_sums", image, squares, None, eps, self.lm_head.w_scale)
+
+    def pieces_per_head(self):
+        """Pieces the attention of a single-row step leaves per head for the o projection to fold; 0: it folds them itself."""
+        if not (self.row_chain and self.piece_fold):
+            return 0
+        return max(self.piece_fold, 4) if self.split_attention else self.piece_fold
 
     def _attend(self, qkv, k_cache, v_cache, pos, kmajor, pieces=False, splits=None):
         """Rotary embedding, cache update and attention for the token whose q | k | v the projection just wrote: one

@@ -683,12 +683,15 @@ def test_fused_single_row_step_equals_the_unfused_one(tiny, cuda):
     assert tiny.row_chain
     assert tiny.piece_fold == 2
     # "plain": the products behind a norm multiply the row and sum its squares themselves; "whole": one workgroup per
-    # head writes the attention's output row (the default leaves two pieces per head for the o projection to fold)
-    for fused in (False, True, "split", "plain", "whole"):
+    # head writes the attention's output row (the default leaves two pieces per head for the o projection to fold);
+    # "split": the rows of a head shared out as for a long cache, the pieces folded by the last workgroup to finish;
+    # "split4": four pieces per head folded by the o projection
+    for fused in (False, True, "split", "split4", "plain", "whole"):
         tiny.fused_decode = bool(fused)
-        tiny.split_attention = fused == "split"
+        tiny.split_attention = fused in ("split", "split4")
         tiny.row_chain = fused != "plain"
-        tiny.piece_fold = 0 if fused == "whole" else 2
+        tiny.piece_fold = 0 if fused in ("whole", "split") else 2
+        assert not fused or tiny.pieces_per_head() == {True: 2, "split4": 4}.get(fused, 0)
         tiny._graph = None
         tiny.prefill(tokens[:, :28])
         st = tiny._decode_state(1)
@@ -699,7 +702,7 @@ def test_fused_single_row_step_equals_the_unfused_one(tiny, cuda):
             st["mask"].copy_((torch.arange(tiny.max_seq_len, device=cuda) <= 28 + j)[None, None, None])
             logits.append(tiny._decode_step(st["token"], st["pos"], st["mask"]).float())
         outs[fused] = torch.stack(logits)
-        assert tiny.row_chain == (fused != "plain") and tiny.piece_fold == (0 if fused == "whole" else 2)   # no step fell back
+        assert tiny.row_chain == (fused != "plain") and tiny.piece_fold == (0 if fused in ("whole", "split") else 2)   # no step fell back
     tiny.piece_fold = 2
     tiny.fused_decode = True
     tiny.split_attention = False
@@ -710,19 +713,25 @@ def test_fused_single_row_step_equals_the_unfused_one(tiny, cuda):
     assert (outs["plain"] - outs[False]).abs().max().item() <= 2e-3 * outs[False].abs().max().item()
     assert (outs["split"] - outs[False]).abs().max().item() <= 2e-3 * outs[False].abs().max().item()
     assert (outs["whole"] - outs[False]).abs().max().item() <= 2e-3 * outs[False].abs().max().item()
+    assert (outs["split4"] - outs[False]).abs().max().item() <= 2e-3 * outs[False].abs().max().item()
     eager = tiny.generate(tokens, 10, use_graph=False)
     graphed = tiny.generate(tokens, 10, use_graph=True)
     again = tiny.generate(tokens, 10, use_graph=True)
     assert torch.equal(eager, graphed) and torch.equal(eager, again)
-    # the split attention (its pieces folded by the last workgroup to finish) under a captured graph, replayed
-    tiny._graph = None
-    tiny._state = None
-    tiny.split_attention = True
-    split_eager = tiny.generate(tokens, 10, use_graph=False)
-    split_graphed = tiny.generate(tokens, 10, use_graph=True)
-    split_again = tiny.generate(tokens, 10, use_graph=True)
-    tiny.split_attention = False
-    assert torch.equal(split_eager, split_graphed) and torch.equal(split_eager, split_again)
+    # the split attention under a captured graph, replayed: four pieces per head folded by the o projection, then the
+    # pieces folded by the last workgroup to finish
+    for fold in (2, 0):
+        tiny._graph = None
+        tiny._state = None
+        tiny.split_attention = True
+        tiny.piece_fold = fold
+        split_eager = tiny.generate(tokens, 10, use_graph=False)
+        split_graphed = tiny.generate(tokens, 10, use_graph=True)
+        split_again = tiny.generate(tokens, 10, use_graph=True)
+        assert tiny.piece_fold == fold and tiny.row_chain
+        tiny.split_attention = False
+        tiny.piece_fold = 2
+        assert torch.equal(split_eager, split_graphed) and torch.equal(split_eager, split_again)
     tiny._graph = None
     tiny._state = None
 
