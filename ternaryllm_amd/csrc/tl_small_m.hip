@@ -2174,8 +2174,8 @@ int launch_spmv_tiles_wide(bool wide, const KernelArgs& a, const tl_layout_heade
     // A ninth wave where it lowers the most tiles a wave owns (K = 4096 is 17 tiles: three for the first of eight waves,
     // two for each of nine) and the workgroups that share a compute unit still fit its 32 waves.  (4096 -> 12288: 9.5
     // against 9.7-9.9 us; with four workgroups to a compute unit, of which only three of nine waves fit, the decoder's
-    // step was 3 % slower.)
-    if (ceil_div(a.NB, compute_units()) <= 3 && ceil_div(a.T, 9) < ceil_div(a.T, 8)) return launch_spmv_tiles_nt<XF16, kBlockThreads + 64, NORM, EPI>(a, h, st);
+    // step was 3 % slower; the kernel that norms its row itself took 12.3 us with nine waves against 10 with eight.)
+    if (NORM != kNormInside && ceil_div(a.NB, compute_units()) <= 3 && ceil_div(a.T, 9) < ceil_div(a.T, 8)) return launch_spmv_tiles_nt<XF16, kBlockThreads + 64, NORM, EPI>(a, h, st);
     return launch_spmv_tiles_nt<XF16, kBlockThreads, NORM, EPI>(a, h, st);
 }
 
