@@ -77,6 +77,12 @@ __global__ __launch_bounds__(256) void tl_rope_cache(const T* __restrict__ qkv, 
 // combined through LDS at the end.
 constexpr int kAttnThreads = 1024;
 constexpr int kAttnBatch = 5;  // rows of a row group whose loads are in flight together
+// With more workgroups than compute units (batches of nine rows and more at 32 heads) two workgroups to a compute unit
+// run through the cache faster than one after the other: tl_decode_attn_packed is the same kernel held to 64
+// registers a lane, which it fits with two rows of a row group in flight (fp16, heads of up to 128 values).  Batch
+// 16 over 577 cache rows: 30.1 against 30.7-31.4 us per layer, over 101 rows 11.2 against 14.6; with three rows in
+// flight it spills and takes 37.4.
+constexpr int kAttnBatchPacked = 2;
 
 
 // The value another lane of the same row of 16 holds, by a data-parallel-primitive code
@@ -101,17 +107,16 @@ struct FreshToken {
     T* v_cache;
 };
 
-template <typename T, int HD>
-__global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restrict__ q, const T* __restrict__ k_cache,
-                                                               const T* __restrict__ v_cache, const long long* __restrict__ pos_p,
-                                                               T* __restrict__ out, long long out_kld, int heads, long long max_seq,
-                                                               float scale, int splits, float* __restrict__ pieces,
-                                                               unsigned* __restrict__ arrivals, FreshToken<T> fresh)
+template <typename T, int HD, int NB>
+__device__ __forceinline__ void decode_attn_body(const T* __restrict__ q, const T* __restrict__ k_cache,
+                                                 const T* __restrict__ v_cache, const long long* __restrict__ pos_p,
+                                                 T* __restrict__ out, long long out_kld, int heads, long long max_seq,
+                                                 float scale, int splits, float* __restrict__ pieces,
+                                                 unsigned* __restrict__ arrivals, const FreshToken<T>& fresh)
 {
     constexpr int VE = 16 / (int)sizeof(T);   // values per 16-byte piece
     constexpr int CPR = HD / VE;              // lanes per cache row
     constexpr int RG = kAttnThreads / CPR;    // row groups
-    constexpr int NB = kAttnBatch;
     static_assert(CPR <= 64 && (CPR & (CPR - 1)) == 0, "a row's lanes must sit in one wave");
     __shared__ float partial[RG][HD + 1];
     constexpr int SG = kAttnThreads / HD;     // threads that share the fold of one output value
@@ -374,6 +379,26 @@ __global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restri
         const size_t col = (size_t)(bh % heads) * HD + tid;
         out[out_kld ? col * out_kld + b : (size_t)b * heads * HD + col] = from_f<T>(o / norm);
     }
+}
+
+template <typename T, int HD>
+__global__ __launch_bounds__(kAttnThreads) void tl_decode_attn(const T* __restrict__ q, const T* __restrict__ k_cache,
+                                                               const T* __restrict__ v_cache, const long long* __restrict__ pos_p,
+                                                               T* __restrict__ out, long long out_kld, int heads, long long max_seq,
+                                                               float scale, int splits, float* __restrict__ pieces,
+                                                               unsigned* __restrict__ arrivals, FreshToken<T> fresh)
+{
+    decode_attn_body<T, HD, kAttnBatch>(q, k_cache, v_cache, pos_p, out, out_kld, heads, max_seq, scale, splits, pieces, arrivals, fresh);
+}
+
+// two workgroups to a compute unit: eight waves per SIMD, 64 registers a lane
+template <typename T, int HD>
+__global__ __launch_bounds__(kAttnThreads) __attribute__((amdgpu_waves_per_eu(8, 8))) void tl_decode_attn_packed(
+    const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache, const long long* __restrict__ pos_p,
+    T* __restrict__ out, long long out_kld, int heads, long long max_seq, float scale, int splits, float* __restrict__ pieces,
+    unsigned* __restrict__ arrivals, FreshToken<T> fresh)
+{
+    decode_attn_body<T, HD, kAttnBatchPacked>(q, k_cache, v_cache, pos_p, out, out_kld, heads, max_seq, scale, splits, pieces, arrivals, fresh);
 }
 
 // Folds the pieces that a split tl_decode_attn left: one workgroup of HD threads per (batch row, head).
@@ -650,7 +675,12 @@ template <typename T, int HD>
 int attn_launch(dim3 grid, size_t lds, hipStream_t st, const void* q, const void* k, const void* v, const long long* pos, void* out,
                 long long out_kld, int heads, long long max_seq, float scale, int splits, float* partial, unsigned* arrivals, const FreshArgs& f)
 {
+    // more workgroups than compute units: the kernel of which two fit a compute unit (built for fp16 heads of up to 128 values)
+    constexpr bool kPacked = sizeof(T) == 2 && HD <= 128;
     auto kernel = tl_decode_attn<T, HD>;
+    if constexpr (kPacked) {
+        if ((int64_t)grid.x * splits > device_units()) kernel = tl_decode_attn_packed<T, HD>;
+    }
     FreshToken<T> fresh{static_cast<const T*>(f.qkv), static_cast<const T*>(f.cos_table), static_cast<const T*>(f.sin_table),
                         f.qkv ? static_cast<T*>(const_cast<void*>(k)) : nullptr, f.qkv ? static_cast<T*>(const_cast<void*>(v)) : nullptr};
     hipLaunchKernelGGL(kernel, dim3(grid.x, (unsigned)splits), dim3(kAttnThreads), lds, st, static_cast<const T*>(q), static_cast<const T*>(k),

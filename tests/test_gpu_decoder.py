@@ -274,11 +274,17 @@ def test_decode_attention_ignores_what_lies_past_the_position(cuda):
     them before it knows the position): NaN and infinities there change nothing, for 1 to 8 workgroups per head."""
     from ternaryllm_amd import ops
     g = torch.Generator().manual_seed(13)
-    B, H, hd, S = 2, 4, 128, 700
+    # (the second shape: more workgroups than compute units, two of which share one)
+    for B, H, hd, S, positions in ((2, 4, 128, 700, (0, 5, 63, 64, 127, 128, 300, 698)), (12, 32, 128, 330, (0, 1, 127, 128, 200, 329))):
+        _attention_ignores_rows_past(cuda, g, B, H, hd, S, positions)
+
+
+def _attention_ignores_rows_past(cuda, g, B, H, hd, S, positions):
+    from ternaryllm_amd import ops
     q = torch.randn((B, H, hd), generator=g).to(torch.float16).to(cuda)
     kc = torch.randn((B, H, S, hd), generator=g).to(torch.float16).to(cuda)
     vc = torch.randn((B, H, S, hd), generator=g).to(torch.float16).to(cuda)
-    for pos in (0, 5, 63, 64, 127, 128, 300, 698):
+    for pos in positions:
         p = torch.tensor([pos], dtype=torch.long, device=cuda)
         kz, vz, kn, vn = kc.clone(), vc.clone(), kc.clone(), vc.clone()
         kz[:, :, pos + 1:] = 0
@@ -385,7 +391,8 @@ def test_attention_that_rotates_and_updates_the_cache_itself(cuda):
     from ternaryllm_amd import ops
     g = torch.Generator().manual_seed(29)
     for dtype in (torch.float16, torch.float32):
-        for B, H, hd, S in ((1, 32, 128, 300), (3, 5, 64, 150), (2, 2, 256, 70)):
+        # (the last two: more workgroups than the chip has compute units, which for fp16 is a kernel of its own)
+        for B, H, hd, S in ((1, 32, 128, 300), (3, 5, 64, 150), (2, 2, 256, 70), (9, 32, 128, 150), (18, 16, 64, 90)):
             inv = 1.0 / (10000 ** (torch.arange(0, hd, 2).double() / hd))
             ang = torch.arange(S).double()[:, None] * inv[None, :]
             cos = torch.cat([ang.cos(), ang.cos()], 1).to(dtype).to(cuda)
@@ -591,7 +598,8 @@ def test_silu_gate_in_the_epilogue_of_the_gate_up_product(cuda):
 
     def fused_rc(dw, x, M, layout=0):
         """status of the one-launch call by itself (ops.spmm_gated falls back silently)"""
-        out = torch.empty((M, dw.columns // 2), dtype=x.dtype, device=cuda)
+        # (a K-major image has 16 rows per column whatever M is)
+        out = torch.empty((M, dw.columns // 2) if layout == 0 else (dw.columns // 2, 16), dtype=x.dtype, device=cuda)
         ws = torch.empty(1 << 22, dtype=torch.uint8, device=cuda)
         return L.tl_spmm_gated(ctypes.byref(dw.header), dw.blob.data_ptr(), x.data_ptr(), ops._code(x.dtype, "x"), 0, dw.inners, M,
                                out.data_ptr(), ops._code(x.dtype, "x"), dw.columns // 2 if layout == 0 else 16, layout, None, 0,
